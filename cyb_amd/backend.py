@@ -1,0 +1,261 @@
+"""ctypes binding of libcybq.so and the host-side mirror of the runtime's
+backend seam.
+
+Reference shape being mirrored (the runtime crate itself is outside the
+reference tree, so these are the in-tree facts the mirror is built from):
+  * one backend object per process, created when the mind is spawned
+    (/root/reference/shell/src/worlds/soma_bridge.rs:65);
+  * weights are handed over once per model load and kept until the model is
+    swapped (/root/reference/shell/src/worlds/models/mod.rs:7-8,386);
+  * the graph IR names an op, its weight tensor (HF-style name) and its in/out
+    edges (/root/reference/decide/pipeline.md:28-30); the executor calls the
+    backend once per node per token (:51);
+  * failures surface as values, never as panics
+    (/root/reference/shell/src/worlds/soma_bridge.rs:322-333) - here CybqError.
+
+Nothing in this module computes the op on the host.  If libcybq.so cannot be
+loaded the import of this module still succeeds (so that CPU-only tooling can
+use cyb_amd.formats), but constructing a Backend raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from dataclasses import dataclass, field
+from typing import Dict, Optional
+
+import numpy as np
+
+from . import formats
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "lib", "libcybq.so")
+
+F32, F16, BF16 = 0, 1, 2
+_DTYPE_CODES = {"torch.float32": F32, "torch.float16": F16, "torch.bfloat16": BF16,
+                "float32": F32, "float16": F16}
+_ITEMSIZE = {F32: 4, F16: 2, BF16: 2}
+
+
+class CybqError(RuntimeError):
+    def __init__(self, status: int, text: str, detail: str = ""):
+        self.status = status
+        msg = f"cybq status {status} ({text})"
+        if detail:
+            msg += f": {detail}"
+        super().__init__(msg)
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def load_library() -> ctypes.CDLL:
+    """Loads libcybq.so from cyb_amd/lib (built in-tree by __graft_entry__.build())."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise CybqError(-4, "library missing", f"{_LIB_PATH} not built; run __graft_entry__.build()")
+    lib = ctypes.CDLL(_LIB_PATH)
+    vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    lib.cybq_version.restype = ctypes.c_char_p
+    lib.cybq_strerror.restype = ctypes.c_char_p
+    lib.cybq_strerror.argtypes = [ci]
+    lib.cybq_last_error.restype = ctypes.c_char_p
+    lib.cybq_last_error.argtypes = [vp]
+    lib.cybq_init.argtypes = [ci, ctypes.POINTER(vp)]
+    lib.cybq_destroy.argtypes = [vp]
+    lib.cybq_destroy.restype = None
+    lib.cybq_weight_upload.argtypes = [vp, ci, ci, i64, i64, vp, vp, ctypes.POINTER(vp)]
+    lib.cybq_weight_from_device.argtypes = [vp, ci, i64, i64, vp, vp, vp, ctypes.POINTER(vp)]
+    lib.cybq_weight_clone.argtypes = [vp, vp, ctypes.POINTER(vp)]
+    lib.cybq_weight_free.argtypes = [vp, vp]
+    lib.cybq_weight_info.argtypes = [vp, ctypes.POINTER(ci), ctypes.POINTER(i64), ctypes.POINTER(i64),
+                                     ctypes.POINTER(i64)]
+    lib.cybq_matmul.argtypes = [vp, vp, vp, ci, i64, vp, ci, vp]
+    lib.cybq_dequant.argtypes = [vp, vp, vp, vp]
+    lib.cybq_quantize.argtypes = [vp, ci, vp, i64, i64, vp, vp, vp]
+    lib.cybq_debug_set_gemv_tuning.argtypes = [ci, ci, ci]
+    _lib = lib
+    return lib
+
+
+def _ptr(t) -> int:
+    if t is None:
+        return 0
+    if isinstance(t, int):
+        return t
+    return int(t.data_ptr())
+
+
+def _dtype_code(t, explicit: Optional[int]) -> int:
+    if explicit is not None:
+        return explicit
+    key = str(getattr(t, "dtype", ""))
+    if key not in _DTYPE_CODES:
+        raise CybqError(-1, "invalid argument", f"unsupported dtype {key!r}")
+    return _DTYPE_CODES[key]
+
+
+@dataclass
+class QMatMul:
+    """Stand-in for the graph-IR node of the op: y = x @ dequant(w)^T.
+
+    `w` is the HF-style tensor name, `x` / `y` are edge names.  The field list of
+    the reference's node is not available in its tree; these are the facts any
+    such node has to carry."""
+    w: str
+    x: str
+    y: str
+    quant: int = formats.Q4
+    group: int = formats.GROUP
+    M: int = 1
+    N: int = 0
+    K: int = 0
+    op: str = "qmatmul"
+
+
+class QWeight:
+    """One uploaded quantised tensor (device-native layout), immutable."""
+
+    def __init__(self, backend: "Backend", handle: int):
+        self._backend = backend
+        self._h = ctypes.c_void_p(handle)
+        q, n, k, b = ctypes.c_int(), ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
+        backend._check(backend._lib.cybq_weight_info(self._h, q, n, k, b))
+        self.quant, self.N, self.K, self.device_bytes = q.value, n.value, k.value, b.value
+
+    @property
+    def handle(self) -> ctypes.c_void_p:
+        if not self._h:
+            raise CybqError(-1, "invalid argument", "weight already freed")
+        return self._h
+
+    @property
+    def algorithmic_bytes(self) -> int:
+        return formats.weight_bytes(self.quant, self.N, self.K)
+
+    def clone(self) -> "QWeight":
+        out = ctypes.c_void_p()
+        b = self._backend
+        b._check(b._lib.cybq_weight_clone(b._ctx, self.handle, ctypes.byref(out)))
+        return QWeight(b, out.value)
+
+    def free(self) -> None:
+        if self._h and self._backend._ctx:
+            self._backend._lib.cybq_weight_free(self._backend._ctx, self._h)
+        self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Backend:
+    """A device context plus the tensors of the loaded model, keyed by name."""
+
+    def __init__(self, device: int = 0):
+        self._lib = load_library()
+        self._ctx = ctypes.c_void_p()
+        rc = self._lib.cybq_init(device, ctypes.byref(self._ctx))
+        if rc != 0:
+            self._ctx = ctypes.c_void_p()
+            raise CybqError(rc, self._lib.cybq_strerror(rc).decode())
+        self.device = device
+        self.weights: Dict[str, QWeight] = {}
+
+    # ---- plumbing
+    def _check(self, rc: int) -> None:
+        if rc != 0:
+            detail = self._lib.cybq_last_error(self._ctx).decode() if self._ctx else ""
+            raise CybqError(rc, self._lib.cybq_strerror(rc).decode(), detail)
+
+    def close(self) -> None:
+        for w in list(self.weights.values()):
+            w.free()
+        self.weights.clear()
+        if self._ctx:
+            self._lib.cybq_destroy(self._ctx)
+            self._ctx = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def version(self) -> str:
+        return self._lib.cybq_version().decode()
+
+    # ---- weights
+    def upload(self, quant: int, layout: int, N: int, K: int, q: np.ndarray,
+               scales: Optional[np.ndarray] = None, name: Optional[str] = None) -> QWeight:
+        """Host interchange buffers -> device-native weight (repacked once, here)."""
+        q = np.ascontiguousarray(q)
+        qp = q.ctypes.data_as(ctypes.c_void_p)
+        sp = None
+        if scales is not None:
+            scales = np.ascontiguousarray(scales)
+            sp = scales.ctypes.data_as(ctypes.c_void_p)
+        out = ctypes.c_void_p()
+        self._check(self._lib.cybq_weight_upload(self._ctx, quant, layout, N, K, qp, sp, ctypes.byref(out)))
+        w = QWeight(self, out.value)
+        if name is not None:
+            self.weights[name] = w
+        return w
+
+    def upload_quantized(self, q: np.ndarray, scales: np.ndarray, quant: int, layout: int = formats.PLANAR,
+                         name: Optional[str] = None) -> QWeight:
+        """Canonical (q int8 [N,K], scales u16 [N,K/32]) -> pack -> upload."""
+        N, K = q.shape
+        if layout == formats.PLANAR:
+            return self.upload(quant, layout, N, K, formats.pack_planar(q, quant), scales, name)
+        return self.upload(quant, layout, N, K, formats.pack_blocks(q, scales, quant), None, name)
+
+    def weight_from_device(self, quant: int, N: int, K: int, q_dev, scales_dev, stream: int = 0,
+                           name: Optional[str] = None) -> QWeight:
+        out = ctypes.c_void_p()
+        self._check(self._lib.cybq_weight_from_device(self._ctx, quant, N, K, _ptr(q_dev), _ptr(scales_dev),
+                                                      stream, ctypes.byref(out)))
+        w = QWeight(self, out.value)
+        if name is not None:
+            self.weights[name] = w
+        return w
+
+    # ---- ops (x / y / out: torch tensors on this device, or raw device addresses)
+    def matmul(self, w: QWeight, x, y, M: Optional[int] = None, xdt: Optional[int] = None,
+               ydt: Optional[int] = None, stream: int = 0) -> None:
+        if M is None:
+            M = int(x.shape[0]) if x.dim() == 2 else 1
+        self._check(self._lib.cybq_matmul(self._ctx, w.handle, _ptr(x), _dtype_code(x, xdt), M, _ptr(y),
+                                          _dtype_code(y, ydt), stream))
+
+    def dequant(self, w: QWeight, out, stream: int = 0) -> None:
+        self._check(self._lib.cybq_dequant(self._ctx, w.handle, _ptr(out), stream))
+
+    def quantize(self, quant: int, src, N: int, K: int, q_out, scales_out, stream: int = 0) -> None:
+        self._check(self._lib.cybq_quantize(self._ctx, quant, _ptr(src), N, K, _ptr(q_out), _ptr(scales_out),
+                                            stream))
+
+    def run(self, node: QMatMul, edges: dict, stream: int = 0) -> None:
+        """Executes one graph node: edges[node.y] = edges[node.x] @ W[node.w]^T."""
+        if node.op != "qmatmul":
+            raise CybqError(-7, "unsupported", f"op {node.op!r}")
+        if node.group != formats.GROUP:
+            raise CybqError(-2, "bad shape", "group must be 32")
+        w = self.weights.get(node.w)
+        if w is None:
+            raise CybqError(-1, "invalid argument", f"weight {node.w!r} not loaded")
+        if (node.N and node.N != w.N) or (node.K and node.K != w.K) or node.quant != w.quant:
+            raise CybqError(-2, "bad shape", f"node {node.w!r} does not match the loaded tensor")
+        self.matmul(w, edges[node.x], edges[node.y], M=node.M, stream=stream)
+
+    def set_gemv_tuning(self, waves: int = 0, strips: int = 0, unroll: int = 0) -> None:
+        self._lib.cybq_debug_set_gemv_tuning(waves, strips, unroll)

@@ -1,0 +1,349 @@
+// api.hip - the C ABI declared in include/cybq.h: argument checking, device
+// memory ownership, dispatch to the kernels.  No torch, no C++ types cross
+// this boundary.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+
+#include "../../include/cybq.h"
+#include "cybq_internal.h"
+
+struct cybq_ctx {
+    int device = 0;
+    int num_cus = 0;
+    std::string last_error;
+};
+
+struct cybq_weight {
+    int device = 0;
+    int bits = 0;
+    int64_t N = 0, K = 0;
+    int NT = 0, KT = 0;
+    uint32_t* q = nullptr;
+    uint16_t* s = nullptr;
+    size_t q_bytes = 0, s_bytes = 0;
+};
+
+namespace {
+
+int fail(cybq_ctx* ctx, int code, const char* what)
+{
+    if (ctx) ctx->last_error = what ? what : "";
+    return code;
+}
+
+int fail_hip(cybq_ctx* ctx, hipError_t e, const char* where)
+{
+    if (ctx) {
+        ctx->last_error = std::string(where) + ": " + hipGetErrorString(e);
+    }
+    (void)hipGetLastError();   // clear the sticky error so the next call starts clean
+    return e == hipErrorOutOfMemory ? CYBQ_ERR_NOMEM : CYBQ_ERR_HIP;
+}
+
+// The device is made current for every call: contexts may live on different
+// devices inside one process.
+struct DeviceGuard {
+    hipError_t err;
+    explicit DeviceGuard(int device) : err(hipSetDevice(device)) {}
+};
+
+cybq::WeightView view_of(const cybq_weight* w)
+{
+    cybq::WeightView v;
+    v.q = w->q;
+    v.s = w->s;
+    v.N = (int)w->N;
+    v.K = (int)w->K;
+    v.NT = w->NT;
+    v.KT = w->KT;
+    v.bits = w->bits;
+    return v;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+size_t dtype_size(int dt) { return dt == CYBQ_F32 ? 4 : 2; }
+bool dtype_ok(int dt) { return dt == CYBQ_F32 || dt == CYBQ_F16 || dt == CYBQ_BF16; }
+
+int alloc_weight(cybq_ctx* ctx, int bits, int64_t N, int64_t K, cybq_weight** out)
+{
+    cybq_weight* w = new (std::nothrow) cybq_weight();
+    if (!w) return fail(ctx, CYBQ_ERR_NOMEM, "host allocation failed");
+    w->device = ctx->device;
+    w->bits = bits;
+    w->N = N;
+    w->K = K;
+    w->NT = (int)((N + cybq::kTileN - 1) / cybq::kTileN);
+    w->KT = (int)((K + cybq::kTileK - 1) / cybq::kTileK);
+    w->q_bytes = (size_t)w->NT * w->KT * (bits == 4 ? 1024 : 2048);
+    w->s_bytes = (size_t)w->NT * w->KT * 128;
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&w->q), w->q_bytes);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&w->s), w->s_bytes);
+    if (e != hipSuccess) {
+        if (w->q) (void)hipFree(w->q);
+        delete w;
+        return fail_hip(ctx, e, "hipMalloc(weight)");
+    }
+    *out = w;
+    return CYBQ_OK;
+}
+
+int check_weight_shape(cybq_ctx* ctx, int quant, int64_t N, int64_t K)
+{
+    if (quant != CYBQ_Q4 && quant != CYBQ_Q8) return fail(ctx, CYBQ_ERR_INVALID, "quant must be CYBQ_Q4 or CYBQ_Q8");
+    if (N < 1 || K < 1) return fail(ctx, CYBQ_ERR_SHAPE, "N and K must be >= 1");
+    if (K % CYBQ_GROUP) return fail(ctx, CYBQ_ERR_SHAPE, "K must be a multiple of 32");
+    if (N > (int64_t)1 << 30 || K > (int64_t)1 << 30 || N * K > (int64_t)1 << 40)
+        return fail(ctx, CYBQ_ERR_SHAPE, "tensor too large");
+    return CYBQ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* cybq_version(void) { return "0.1.0"; }
+
+const char* cybq_strerror(int status)
+{
+    switch (status) {
+        case CYBQ_OK: return "ok";
+        case CYBQ_ERR_INVALID: return "invalid argument";
+        case CYBQ_ERR_SHAPE: return "bad shape";
+        case CYBQ_ERR_ALIGN: return "misaligned pointer";
+        case CYBQ_ERR_NO_DEVICE: return "no usable gfx950 device";
+        case CYBQ_ERR_HIP: return "HIP runtime error";
+        case CYBQ_ERR_NOMEM: return "out of memory";
+        case CYBQ_ERR_UNSUPPORTED: return "unsupported";
+        default: return "unknown status";
+    }
+}
+
+const char* cybq_last_error(const cybq_ctx* ctx) { return ctx ? ctx->last_error.c_str() : ""; }
+
+int cybq_init(int device, cybq_ctx** out)
+{
+    if (!out) return CYBQ_ERR_INVALID;
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count < 1) { (void)hipGetLastError(); return CYBQ_ERR_NO_DEVICE; }
+    if (device < 0 || device >= count) return CYBQ_ERR_INVALID;
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) { (void)hipGetLastError(); return CYBQ_ERR_NO_DEVICE; }
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) return CYBQ_ERR_NO_DEVICE;
+    e = hipSetDevice(device);
+    if (e != hipSuccess) { (void)hipGetLastError(); return CYBQ_ERR_HIP; }
+    cybq_ctx* ctx = new (std::nothrow) cybq_ctx();
+    if (!ctx) return CYBQ_ERR_NOMEM;
+    ctx->device = device;
+    ctx->num_cus = prop.multiProcessorCount;
+    *out = ctx;
+    return CYBQ_OK;
+}
+
+void cybq_destroy(cybq_ctx* ctx) { delete ctx; }
+
+int cybq_weight_upload(cybq_ctx* ctx, cybq_quant quant, cybq_layout layout, int64_t N, int64_t K,
+                       const void* q, const void* scales, cybq_weight** out)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (!out) return fail(ctx, CYBQ_ERR_INVALID, "out is NULL");
+    *out = nullptr;
+    if (!q) return fail(ctx, CYBQ_ERR_INVALID, "q is NULL");
+    if (layout != CYBQ_LAYOUT_PLANAR && layout != CYBQ_LAYOUT_BLOCK_AOS)
+        return fail(ctx, CYBQ_ERR_INVALID, "unknown layout");
+    if (layout == CYBQ_LAYOUT_PLANAR && !scales) return fail(ctx, CYBQ_ERR_INVALID, "PLANAR needs a scale plane");
+    if (layout == CYBQ_LAYOUT_BLOCK_AOS && scales) return fail(ctx, CYBQ_ERR_INVALID, "BLOCK_AOS carries its scales; pass NULL");
+    int rc = check_weight_shape(ctx, quant, N, K);
+    if (rc) return rc;
+    DeviceGuard guard(ctx->device);
+    if (guard.err != hipSuccess) return fail_hip(ctx, guard.err, "hipSetDevice");
+
+    const int64_t groups = N * (K / CYBQ_GROUP);
+    size_t q_src_bytes, s_src_bytes = 0;
+    if (layout == CYBQ_LAYOUT_PLANAR) {
+        q_src_bytes = (size_t)(quant == CYBQ_Q4 ? N * K / 2 : N * K);
+        s_src_bytes = (size_t)groups * 2;
+    } else {
+        q_src_bytes = (size_t)groups * (quant == CYBQ_Q4 ? 18 : 34);
+    }
+    void *q_tmp = nullptr, *s_tmp = nullptr;
+    hipError_t e = hipMalloc(&q_tmp, q_src_bytes);
+    if (e == hipSuccess && s_src_bytes) e = hipMalloc(&s_tmp, s_src_bytes);
+    if (e != hipSuccess) {
+        if (q_tmp) (void)hipFree(q_tmp);
+        return fail_hip(ctx, e, "hipMalloc(staging)");
+    }
+    cybq_weight* w = nullptr;
+    rc = alloc_weight(ctx, quant, N, K, &w);
+    if (rc == CYBQ_OK) {
+        e = hipMemcpy(q_tmp, q, q_src_bytes, hipMemcpyHostToDevice);
+        if (e == hipSuccess && s_src_bytes) e = hipMemcpy(s_tmp, scales, s_src_bytes, hipMemcpyHostToDevice);
+        if (e == hipSuccess)
+            e = cybq::launch_repack(quant, layout, q_tmp, s_tmp, w->q, w->s, (int)N, (int)K, w->NT, w->KT, nullptr);
+        if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+        if (e != hipSuccess) {
+            rc = fail_hip(ctx, e, "weight upload");
+            (void)hipFree(w->q);
+            (void)hipFree(w->s);
+            delete w;
+            w = nullptr;
+        }
+    }
+    (void)hipFree(q_tmp);
+    if (s_tmp) (void)hipFree(s_tmp);
+    if (rc) return rc;
+    *out = w;
+    return CYBQ_OK;
+}
+
+int cybq_weight_from_device(cybq_ctx* ctx, cybq_quant quant, int64_t N, int64_t K, const void* q_dev,
+                            const void* scales_dev, void* stream, cybq_weight** out)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (!out) return fail(ctx, CYBQ_ERR_INVALID, "out is NULL");
+    *out = nullptr;
+    if (!q_dev || !scales_dev) return fail(ctx, CYBQ_ERR_INVALID, "q_dev / scales_dev is NULL");
+    int rc = check_weight_shape(ctx, quant, N, K);
+    if (rc) return rc;
+    DeviceGuard guard(ctx->device);
+    if (guard.err != hipSuccess) return fail_hip(ctx, guard.err, "hipSetDevice");
+    cybq_weight* w = nullptr;
+    rc = alloc_weight(ctx, quant, N, K, &w);
+    if (rc) return rc;
+    hipError_t e = cybq::launch_repack(quant, CYBQ_LAYOUT_PLANAR, q_dev, scales_dev, w->q, w->s, (int)N, (int)K,
+                                       w->NT, w->KT, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) {
+        (void)hipFree(w->q);
+        (void)hipFree(w->s);
+        delete w;
+        return fail_hip(ctx, e, "repack launch");
+    }
+    *out = w;
+    return CYBQ_OK;
+}
+
+int cybq_weight_clone(cybq_ctx* ctx, const cybq_weight* src, cybq_weight** out)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (!src || !out) return fail(ctx, CYBQ_ERR_INVALID, "src / out is NULL");
+    *out = nullptr;
+    if (src->device != ctx->device) return fail(ctx, CYBQ_ERR_INVALID, "weight lives on another device");
+    DeviceGuard guard(ctx->device);
+    if (guard.err != hipSuccess) return fail_hip(ctx, guard.err, "hipSetDevice");
+    cybq_weight* w = nullptr;
+    int rc = alloc_weight(ctx, src->bits, src->N, src->K, &w);
+    if (rc) return rc;
+    hipError_t e = hipMemcpy(w->q, src->q, src->q_bytes, hipMemcpyDeviceToDevice);
+    if (e == hipSuccess) e = hipMemcpy(w->s, src->s, src->s_bytes, hipMemcpyDeviceToDevice);
+    if (e != hipSuccess) {
+        (void)hipFree(w->q);
+        (void)hipFree(w->s);
+        delete w;
+        return fail_hip(ctx, e, "weight clone");
+    }
+    *out = w;
+    return CYBQ_OK;
+}
+
+int cybq_weight_free(cybq_ctx* ctx, cybq_weight* w)
+{
+    if (!w) return CYBQ_OK;
+    hipError_t e = hipSetDevice(w->device);
+    if (e == hipSuccess) e = hipFree(w->q);
+    hipError_t e2 = hipFree(w->s);
+    delete w;
+    if (e != hipSuccess) return fail_hip(ctx, e, "hipFree(weight)");
+    if (e2 != hipSuccess) return fail_hip(ctx, e2, "hipFree(weight)");
+    return CYBQ_OK;
+}
+
+int cybq_weight_info(const cybq_weight* w, int* quant, int64_t* N, int64_t* K, int64_t* device_bytes)
+{
+    if (!w) return CYBQ_ERR_INVALID;
+    if (quant) *quant = w->bits;
+    if (N) *N = w->N;
+    if (K) *K = w->K;
+    if (device_bytes) *device_bytes = (int64_t)(w->q_bytes + w->s_bytes);
+    return CYBQ_OK;
+}
+
+int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M, void* y,
+                cybq_dtype ydt, void* stream)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (!w || !x || !y) return fail(ctx, CYBQ_ERR_INVALID, "w / x / y is NULL");
+    if (!dtype_ok(xdt) || !dtype_ok(ydt)) return fail(ctx, CYBQ_ERR_INVALID, "unknown dtype");
+    if (M < 1 || M > (1 << 24)) return fail(ctx, CYBQ_ERR_SHAPE, "M must be in 1..2^24");
+    if (w->device != ctx->device) return fail(ctx, CYBQ_ERR_INVALID, "weight lives on another device");
+    if (!aligned16(x)) return fail(ctx, CYBQ_ERR_ALIGN, "x must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(y) % dtype_size(ydt)) return fail(ctx, CYBQ_ERR_ALIGN, "y is not aligned to its element size");
+    DeviceGuard guard(ctx->device);
+    if (guard.err != hipSuccess) return fail_hip(ctx, guard.err, "hipSetDevice");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    cybq::WeightView v = view_of(w);
+    hipError_t e;
+    if (M <= 16) {
+        e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, st);
+    } else if (xdt != CYBQ_F32) {
+        e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, st);
+    } else {
+        // fp32 activations keep full precision through the decode kernel's
+        // hi/lo split; prefill in fp32 is walked 16 rows at a time.
+        e = hipSuccess;
+        for (int64_t m0 = 0; m0 < M && e == hipSuccess; m0 += 16) {
+            int mm = (int)((M - m0) < 16 ? (M - m0) : 16);
+            const char* xp = static_cast<const char*>(x) + (size_t)m0 * w->K * 4;
+            char* yp = static_cast<char*>(y) + (size_t)m0 * w->N * dtype_size(ydt);
+            e = cybq::launch_gemv(v, xp, xdt, mm, yp, ydt, ctx->num_cus, st);
+        }
+    }
+    if (e != hipSuccess) return fail_hip(ctx, e, "matmul launch");
+    return CYBQ_OK;
+}
+
+int cybq_dequant(cybq_ctx* ctx, const cybq_weight* w, float* out, void* stream)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (!w || !out) return fail(ctx, CYBQ_ERR_INVALID, "w / out is NULL");
+    if (w->device != ctx->device) return fail(ctx, CYBQ_ERR_INVALID, "weight lives on another device");
+    if (!aligned16(out)) return fail(ctx, CYBQ_ERR_ALIGN, "out must be 16-byte aligned");
+    DeviceGuard guard(ctx->device);
+    if (guard.err != hipSuccess) return fail_hip(ctx, guard.err, "hipSetDevice");
+    hipError_t e = cybq::launch_dequant(view_of(w), out, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail_hip(ctx, e, "dequant launch");
+    return CYBQ_OK;
+}
+
+int cybq_quantize(cybq_ctx* ctx, cybq_quant quant, const float* src, int64_t N, int64_t K, void* q_out,
+                  void* scales_out, void* stream)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (!src || !q_out || !scales_out) return fail(ctx, CYBQ_ERR_INVALID, "src / q_out / scales_out is NULL");
+    int rc = check_weight_shape(ctx, quant, N, K);
+    if (rc) return rc;
+    if (!aligned16(src)) return fail(ctx, CYBQ_ERR_ALIGN, "src must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(q_out) % 4 || reinterpret_cast<uintptr_t>(scales_out) % 2)
+        return fail(ctx, CYBQ_ERR_ALIGN, "q_out must be 4-byte and scales_out 2-byte aligned");
+    DeviceGuard guard(ctx->device);
+    if (guard.err != hipSuccess) return fail_hip(ctx, guard.err, "hipSetDevice");
+    hipError_t e = cybq::launch_quantize(quant, src, (int)N, (int)K, q_out, scales_out, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail_hip(ctx, e, "quantize launch");
+    return CYBQ_OK;
+}
+
+/* Test and benchmark hook (not part of the operator interface): overrides the
+ * decode kernel's launch heuristics; 0 restores the automatic choice. */
+int cybq_debug_set_gemv_tuning(int waves_per_group, int strips_per_group, int unroll)
+{
+    cybq::set_gemv_tuning(waves_per_group, strips_per_group, unroll);
+    return CYBQ_OK;
+}
+
+}  // extern "C"

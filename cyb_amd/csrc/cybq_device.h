@@ -1,0 +1,127 @@
+// cybq_device.h - device-native weight layout and register-level unpack helpers
+// shared by every kernel of libcybq (gfx950 only).
+//
+// Native layout.  A weight tensor W[N,K] is cut into tiles of 16 rows x 128 k
+// (4 scale groups).  Tiles are stored strip-major: tile (nt, kt) sits at index
+// nt*KT + kt, so a 16-row strip is one contiguous stream along K.
+//
+//   Q4 q plane : tile = 64 lanes x 16 B (1024 B).  Lane l, word j (0..3) holds
+//       row   n = 16*nt + (l & 15)
+//       group g = 4*kt + j
+//       the 8 weights k = 32*g + 8*(l >> 4) + s,  s = 0..7
+//       as nibbles u = q + 8, weight s at nibble position (s >> 1) + 4*(s & 1).
+//     One 128-bit load per lane is therefore four ready-made B operands of
+//     v_mfma_f32_16x16x32 (lane = column n, 8 consecutive k per lane), and the
+//     nibble order lets one and-or peel two weights into one packed-f16 register.
+//   Q8 q plane : tile = 2 halves x 64 lanes x 16 B (2048 B).  Half h, lane l
+//     holds groups 4*kt + 2*h and 4*kt + 2*h + 1, 8 bytes each, byte s =
+//     q + 128 for k = 32*g + 8*(l >> 4) + s.
+//   scale plane: tile = 16 rows x 4 groups of IEEE f16 (128 B): [row][group].
+//
+// N is padded to 16 and K to 128 with q = 0 / scale = 0.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace cybq {
+
+constexpr int kGroup = 32;
+constexpr int kTileN = 16;
+constexpr int kTileK = 128;
+constexpr int kGroupsPerTile = kTileK / kGroup;
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+union Frag16 {            // 8 x 16-bit values = one MFMA A/B operand
+    u32x4_t u;
+    half8_t h;
+    bf16x8_t b;
+};
+
+__device__ __forceinline__ uint32_t as_u32(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
+__device__ __forceinline__ half2_t as_h2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t bits16)
+{
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
+}
+
+// nibble position of weight slot s inside a native Q4 word
+__host__ __device__ __forceinline__ int q4_nibble_pos(int s) { return (s >> 1) + 4 * (s & 1); }
+
+// One native Q4 word -> 8 exact f16 integers in MFMA operand order.
+// 0x6400 | u is the f16 number 1024 + u; 0x6400 | (u << 4) is 1024 + 16u.
+__device__ __forceinline__ void unpack_q4_f16(uint32_t w, uint32_t out[4])
+{
+    const uint32_t lo = 0x000F000Fu, hi = 0x00F000F0u, magic = 0x64006400u;
+    const half2_t sub = {(_Float16)-1032.0f, (_Float16)-1032.0f};
+    const half2_t mul = {(_Float16)0.0625f, (_Float16)0.0625f};
+    const half2_t add = {(_Float16)-72.0f, (_Float16)-72.0f};
+    uint32_t w8 = w >> 8;
+    half2_t t0 = as_h2((w & lo) | magic) + sub;
+    half2_t t1 = as_h2((w & hi) | magic) * mul + add;
+    half2_t t2 = as_h2((w8 & lo) | magic) + sub;
+    half2_t t3 = as_h2((w8 & hi) | magic) * mul + add;
+    out[0] = as_u32(t0);
+    out[1] = as_u32(t1);
+    out[2] = as_u32(t2);
+    out[3] = as_u32(t3);
+}
+
+// Two native Q8 words (8 bytes, u = q + 128) -> 8 exact f16 integers.
+__device__ __forceinline__ void unpack_q8_f16(uint32_t w0, uint32_t w1, uint32_t out[4])
+{
+    const uint32_t magic = 0x64646464u;
+    const half2_t sub = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+    // v_perm_b32 selector bytes: 0..3 pick from the second operand, 4..7 from the first
+    uint32_t p0 = __builtin_amdgcn_perm(magic, w0, 0x04010400u);   // [b0,64,b1,64]
+    uint32_t p1 = __builtin_amdgcn_perm(magic, w0, 0x04030402u);   // [b2,64,b3,64]
+    uint32_t p2 = __builtin_amdgcn_perm(magic, w1, 0x04010400u);
+    uint32_t p3 = __builtin_amdgcn_perm(magic, w1, 0x04030402u);
+    out[0] = as_u32(as_h2(p0) + sub);
+    out[1] = as_u32(as_h2(p1) + sub);
+    out[2] = as_u32(as_h2(p2) + sub);
+    out[3] = as_u32(as_h2(p3) + sub);
+}
+
+// packed pair of exact small f16 integers -> packed pair of bf16 (exact)
+__device__ __forceinline__ uint32_t h2_to_bf16x2_exact(uint32_t h2)
+{
+    half2_t v = as_h2(h2);
+    uint32_t a = __builtin_bit_cast(uint32_t, (float)v.x);
+    uint32_t b = __builtin_bit_cast(uint32_t, (float)v.y);
+    return __builtin_amdgcn_perm(b, a, 0x07060302u);   // [a.hi16, b.hi16]
+}
+
+__device__ __forceinline__ void f16frag_to_bf16frag(uint32_t f[4])
+{
+#pragma unroll
+    for (int i = 0; i < 4; i++) f[i] = h2_to_bf16x2_exact(f[i]);
+}
+
+// signed value of weight slot s of a native Q4 word / Q8 word pair (scalar helpers)
+__device__ __forceinline__ int q4_slot_value(uint32_t w, int s)
+{
+    return (int)((w >> (4 * q4_nibble_pos(s))) & 15u) - 8;
+}
+__device__ __forceinline__ int q8_slot_value(uint32_t w0, uint32_t w1, int s)
+{
+    uint32_t w = s < 4 ? w0 : w1;
+    return (int)((w >> (8 * (s & 3))) & 255u) - 128;
+}
+
+struct WeightView {       // what kernels need to know about an uploaded tensor
+    const uint32_t* q;    // native q plane
+    const uint16_t* s;    // native scale plane
+    int N, K;             // logical
+    int NT, KT;           // tiles (padded)
+    int bits;             // 4 or 8
+};
+
+}  // namespace cybq

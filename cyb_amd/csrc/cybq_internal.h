@@ -1,0 +1,33 @@
+// cybq_internal.h - launcher prototypes shared between the C ABI (api.hip) and
+// the kernel translation units.  Every launcher validates nothing: api.hip
+// checks shapes, alignment and pointers before it calls down here.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "cybq_device.h"
+
+namespace cybq {
+
+// dtype codes mirror enum cybq_dtype
+constexpr int kF32 = 0, kF16 = 1, kBF16 = 2;
+
+hipError_t launch_repack(int bits, int layout, const void* q, const void* scales, uint32_t* qdst,
+                         uint16_t* sdst, int N, int K, int NT, int KT, hipStream_t st);
+hipError_t launch_dequant(const WeightView& w, float* out, hipStream_t st);
+
+// decode path, 1 <= M <= 16
+hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
+                       int num_cus, hipStream_t st);
+// prefill path, M > 16
+hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
+                       int num_cus, hipStream_t st);
+
+hipError_t launch_quantize(int bits, const float* src, int N, int K, void* q_out, void* s_out,
+                           hipStream_t st);
+
+// test/bench hook: overrides the decode kernel's launch heuristics (0 = automatic)
+void set_gemv_tuning(int waves_per_group, int strips_per_group, int unroll);
+
+}  // namespace cybq

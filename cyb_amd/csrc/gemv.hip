@@ -1,0 +1,297 @@
+// gemv.hip - decode kernel: y[M,N] = x[M,K] * W^T for 1 <= M <= 16.
+//
+// HBM-bound: every weight byte is read exactly once with 128-bit loads; the
+// only other traffic is x (staged once per workgroup into LDS) and y.
+//
+// Mapping.  One workgroup owns one 16-row strip of W (a contiguous stream in
+// the native layout) and splits the strip's K tiles over its waves; tile kt
+// goes to wave kt % waves, so neighbouring waves read neighbouring kilobytes.
+// A lane's 16 B load is four MFMA B operands (one per scale group), x comes
+// out of LDS as the A operand, and v_mfma_f32_16x16x32 does the 32-long dot
+// product of one group for 16 columns x 16 batch rows at once.  The per-group
+// f16 scale is applied in fp32 on the MFMA result, so the weight operand stays
+// an exact small integer and the only rounding is the fp32 accumulation.
+// Split-K partials meet in LDS in a fixed order: results are deterministic and
+// row m of a batch is bit-identical to the same row run alone.
+#include "cybq_device.h"
+#include "cybq_internal.h"
+
+namespace cybq {
+
+namespace {
+
+constexpr int XF16 = 0, XBF16 = 1, XF32 = 2;
+
+template <int BITS>
+struct TileRegs {
+    u32x4_t q[BITS == 4 ? 1 : 2];
+    u32x2_t s;
+};
+
+template <int BITS>
+__device__ __forceinline__ void load_tile(TileRegs<BITS>& t, const WeightView& w, int64_t tile, int lane)
+{
+    const u32x4_t* qp = reinterpret_cast<const u32x4_t*>(w.q);
+    if (BITS == 4) {
+        t.q[0] = __builtin_nontemporal_load(qp + tile * 64 + lane);
+    } else {
+        t.q[0] = __builtin_nontemporal_load(qp + tile * 128 + lane);
+        t.q[1] = __builtin_nontemporal_load(qp + tile * 128 + 64 + lane);
+    }
+    const u32x2_t* sp = reinterpret_cast<const u32x2_t*>(w.s);
+    t.s = __builtin_nontemporal_load(sp + tile * 16 + (lane & 15));
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f)
+{
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ void store_out(void* y, int ydt, int64_t idx, float v)
+{
+    if (ydt == kF32) reinterpret_cast<float*>(y)[idx] = v;
+    else if (ydt == kF16) reinterpret_cast<_Float16*>(y)[idx] = (_Float16)v;
+    else reinterpret_cast<uint16_t*>(y)[idx] = f32_to_bf16_rne(v);
+}
+
+// x rows of one K slab -> LDS (row stride ldx 16-bit elements; XF32: a second
+// plane of low halves follows the first at plane_elems).
+template <int XMODE>
+__device__ __forceinline__ void stage_x(uint16_t* xs, const void* x, int M, int K, int k_begin,
+                                        int slab_k, int ldx, int plane_elems, int tid, int nthreads)
+{
+    const int chunks_per_row = slab_k >> 3;
+    const int total = M * chunks_per_row;
+    for (int c = tid; c < total; c += nthreads) {
+        int row = c / chunks_per_row;
+        int col = (c - row * chunks_per_row) << 3;
+        int k = k_begin + col;
+        u32x4_t* dst = reinterpret_cast<u32x4_t*>(xs + row * ldx + col);
+        if (XMODE != XF32) {
+            u32x4_t v = {0u, 0u, 0u, 0u};
+            if (k < K) v = *reinterpret_cast<const u32x4_t*>(
+                           reinterpret_cast<const uint16_t*>(x) + (int64_t)row * K + k);
+            *dst = v;
+        } else {
+            float f[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (k < K) {
+                const float4* p = reinterpret_cast<const float4*>(
+                    reinterpret_cast<const float*>(x) + (int64_t)row * K + k);
+                float4 a = p[0], b = p[1];
+                f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w;
+                f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+            }
+            Frag16 hi, lo;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                _Float16 h = (_Float16)f[i];
+                hi.h[i] = h;
+                lo.h[i] = (_Float16)(f[i] - (float)h);
+            }
+            *dst = hi.u;
+            *reinterpret_cast<u32x4_t*>(xs + plane_elems + row * ldx + col) = lo.u;
+        }
+    }
+}
+
+template <int BITS, int XMODE, int RMAX>
+__device__ __forceinline__ void compute_tile(const TileRegs<BITS>& t, const uint16_t* xrow,
+                                             int plane_elems, float acc[RMAX])
+{
+    const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        Frag16 b;
+        uint32_t bw[4];
+        if (BITS == 4) unpack_q4_f16(t.q[0][j], bw);
+        else unpack_q8_f16(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
+        if (XMODE == XBF16) f16frag_to_bf16frag(bw);
+        b.u = (u32x4_t){bw[0], bw[1], bw[2], bw[3]};
+        Frag16 a;
+        a.u = *reinterpret_cast<const u32x4_t*>(xrow + j * 32);
+        float4_t d;
+        if (XMODE == XBF16) {
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, zero, 0, 0, 0);
+        } else {
+            d = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, zero, 0, 0, 0);
+            if (XMODE == XF32) {
+                Frag16 al;
+                al.u = *reinterpret_cast<const u32x4_t*>(xrow + plane_elems + j * 32);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_f16(al.h, b.h, d, 0, 0, 0);
+            }
+        }
+        uint32_t sb = (j & 1) ? (t.s[j >> 1] >> 16) : (t.s[j >> 1] & 0xffffu);
+        float sc = f16_bits_to_f32(sb);
+#pragma unroll
+        for (int r = 0; r < RMAX; r++) acc[r] = __builtin_fmaf(sc, d[r], acc[r]);
+    }
+}
+
+// U = tiles a wave keeps in flight per batch (two batches are live: ping-pong).
+template <int BITS, int XMODE, int RMAX, int U>
+__global__ __launch_bounds__(512) void gemv_kernel(WeightView w, const void* __restrict__ x, int M, void* __restrict__ y,
+                            int ydt, int slab_tiles, int ldx)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint16_t* xs = reinterpret_cast<uint16_t*>(smem);
+
+    const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
+    const int lane = tid & 63;
+    const int wv = tid >> 6;
+    const int nwaves = nthreads >> 6;
+    const int nt = blockIdx.x;
+    const int mrow = min(lane & 15, M - 1);
+    const int oct = lane >> 4;
+    const int plane_elems = M * ldx;
+    const int64_t strip = (int64_t)nt * w.KT;
+    const int stride = nwaves * U;
+
+    float acc[RMAX];
+#pragma unroll
+    for (int r = 0; r < RMAX; r++) acc[r] = 0.f;
+
+    TileRegs<BITS> bufA[U], bufB[U];
+
+    for (int slab0 = 0; slab0 < w.KT; slab0 += slab_tiles) {
+        const int st = min(slab_tiles, w.KT - slab0);
+        // first batch of this slab goes out before x is staged: HBM latency
+        // overlaps the staging and the barrier
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            int i = wv + u * nwaves;
+            if (i < st) load_tile<BITS>(bufA[u], w, strip + slab0 + i, lane);
+        }
+        if (slab0 > 0) __syncthreads();
+        stage_x<XMODE>(xs, x, M, w.K, slab0 * kTileK, st * kTileK, ldx, plane_elems, tid, nthreads);
+        __syncthreads();
+
+        const uint16_t* xbase = xs + mrow * ldx + oct * 8;
+        for (int i0 = wv; i0 < st; i0 += 2 * stride) {
+            // ---- bufA holds batch i0; fetch batch i0 + stride into bufB
+            const int i1 = i0 + stride;
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                int i = i1 + u * nwaves;
+                if (i < st) load_tile<BITS>(bufB[u], w, strip + slab0 + i, lane);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                int i = i0 + u * nwaves;
+                if (i < st) compute_tile<BITS, XMODE, RMAX>(bufA[u], xbase + i * kTileK, plane_elems, acc);
+            }
+            // ---- bufB holds batch i1; fetch batch i1 + stride into bufA
+            const int i2 = i1 + stride;
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                int i = i2 + u * nwaves;
+                if (i < st) load_tile<BITS>(bufA[u], w, strip + slab0 + i, lane);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                int i = i1 + u * nwaves;
+                if (i < st) compute_tile<BITS, XMODE, RMAX>(bufB[u], xbase + i * kTileK, plane_elems, acc);
+            }
+        }
+    }
+
+    // split-K partials -> LDS, summed in wave order by wave 0
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(smem);
+#pragma unroll
+    for (int r = 0; r < RMAX; r++) red[(wv * RMAX + r) * 64 + lane] = acc[r];
+    __syncthreads();
+    if (wv == 0) {
+        const int n = nt * 16 + (lane & 15);
+#pragma unroll
+        for (int r = 0; r < RMAX; r++) {
+            float v = 0.f;
+            for (int k = 0; k < nwaves; k++) v += red[(k * RMAX + r) * 64 + lane];
+            int m = 4 * oct + r;
+            if (m < M && n < w.N) store_out(y, ydt, (int64_t)m * w.N + n, v);
+        }
+    }
+}
+
+int g_tune_waves = 0, g_tune_unroll = 0;
+
+template <int BITS, int XMODE, int RMAX, int U>
+hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves,
+                    hipStream_t st)
+{
+    const int planes = XMODE == XF32 ? 2 : 1;
+    const int budget = 64 * 1024;
+    int slab_tiles = w.KT;
+    if ((int64_t)M * (w.KT * kTileK + 8) * 2 * planes > budget) {
+        int k_fit = budget / (2 * M * planes) - 8;
+        slab_tiles = k_fit / kTileK;
+        int step = nwaves * U;
+        if (slab_tiles > step) slab_tiles -= slab_tiles % step;
+        if (slab_tiles < 1) slab_tiles = 1;
+    }
+    int ldx = slab_tiles * kTileK + 8;
+    size_t lds = (size_t)M * ldx * 2 * planes;
+    size_t red = (size_t)nwaves * RMAX * 64 * sizeof(float);
+    if (lds < red) lds = red;
+    hipLaunchKernelGGL((gemv_kernel<BITS, XMODE, RMAX, U>), dim3(w.NT), dim3(nwaves * 64), lds, st,
+                       w, x, M, y, ydt, slab_tiles, ldx);
+    return hipGetLastError();
+}
+
+template <int BITS, int XMODE, int U>
+hipError_t launch_r(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves,
+                    hipStream_t st)
+{
+    if (M == 1) return launch_t<BITS, XMODE, 1, U>(w, x, M, y, ydt, nwaves, st);
+    if (M == 2) return launch_t<BITS, XMODE, 2, U>(w, x, M, y, ydt, nwaves, st);
+    return launch_t<BITS, XMODE, 4, U>(w, x, M, y, ydt, nwaves, st);
+}
+
+template <int BITS, int XMODE>
+hipError_t launch_u(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, int unroll,
+                    hipStream_t st)
+{
+    if (BITS == 4 && XMODE == XF16) {
+        if (unroll == 2) return launch_r<BITS, XMODE, 2>(w, x, M, y, ydt, nwaves, st);
+        if (unroll == 8) return launch_r<BITS, XMODE, 8>(w, x, M, y, ydt, nwaves, st);
+    }
+    return launch_r<BITS, XMODE, 4>(w, x, M, y, ydt, nwaves, st);
+}
+
+}  // namespace
+
+void set_gemv_tuning(int waves_per_group, int strips_per_group, int unroll)
+{
+    (void)strips_per_group;
+    g_tune_waves = waves_per_group;
+    g_tune_unroll = unroll;
+}
+
+hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
+                       int num_cus, hipStream_t st)
+{
+    // enough waves to keep ~8 per CU in flight, never more than there are tiles
+    int nwaves = g_tune_waves;
+    if (nwaves <= 0) {
+        int64_t want = (int64_t)num_cus * 8;
+        nwaves = 2;
+        while (nwaves < 8 && (int64_t)w.NT * nwaves < want) nwaves *= 2;
+    }
+    if (nwaves > 8) nwaves = 8;   // the kernel is compiled for at most 512 threads
+    while (nwaves > 1 && nwaves > w.KT) nwaves >>= 1;
+    int unroll = g_tune_unroll > 0 ? g_tune_unroll : 4;
+
+    if (w.bits == 4) {
+        if (xdt == kF16) return launch_u<4, XF16>(w, x, M, y, ydt, nwaves, unroll, st);
+        if (xdt == kBF16) return launch_u<4, XBF16>(w, x, M, y, ydt, nwaves, unroll, st);
+        return launch_u<4, XF32>(w, x, M, y, ydt, nwaves, unroll, st);
+    }
+    if (xdt == kF16) return launch_u<8, XF16>(w, x, M, y, ydt, nwaves, unroll, st);
+    if (xdt == kBF16) return launch_u<8, XBF16>(w, x, M, y, ydt, nwaves, unroll, st);
+    return launch_u<8, XF32>(w, x, M, y, ydt, nwaves, unroll, st);
+}
+
+}  // namespace cybq

@@ -1,0 +1,141 @@
+/*
+ * cybq.h - C ABI of libcybq, the MI355X (gfx950) implementation of cyb's
+ * block-quantized matmul operator.
+ *
+ * What it replaces.  In cyb every linear layer of the decode loop
+ * (QKV, O proj, FFN, LM head - /root/reference/decide/pipeline.md:51) is one
+ * dequantize-and-multiply over Q4/Q8 tensor data
+ * (/root/reference/decide/pipeline.md:28,38) executed by the model runtime
+ * crate `run` on one of its backends (cpu | wgpu WGSL | Metal;
+ * /root/reference/decide/model-lifecycle.md:25-26,37).  That crate is a path
+ * dependency outside the tree (/root/reference/Cargo.lock:8443-8462), so its
+ * backend trait cannot be cited line by line; the entry points below are what
+ * a fourth backend of that runtime has to bind: create a device context,
+ * hand over each weight tensor once at model load, run the op per graph node,
+ * read back dequantised weights for verification.
+ *
+ * Conventions
+ *   - every function returns 0 (CYBQ_OK) or a negative cybq_status; nothing
+ *     aborts, nothing throws across the boundary (the caller surfaces errors
+ *     as SomaEvent::Error - /root/reference/shell/src/worlds/soma_bridge.rs:322-333).
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *     cybq_matmul / cybq_dequant / cybq_quantize are asynchronous and
+ *     stream-ordered; they allocate nothing.
+ *   - x, y, out are DEVICE pointers owned by the caller; weight source
+ *     buffers given to cybq_weight_upload are HOST pointers (the mmap'd
+ *     .model file - /root/reference/shell/src/lib.rs:31-33).
+ *   - a cybq_ctx is bound to one device and is used from one thread at a time
+ *     (the runtime has a single inference thread -
+ *     /root/reference/shell/src/worlds/soma_bridge.rs:49-50,65).
+ *   - a cybq_weight is immutable after upload.
+ */
+#ifndef CYBQ_H
+#define CYBQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CYBQ_GROUP 32            /* weights per scale, along K */
+
+typedef struct cybq_ctx cybq_ctx;
+typedef struct cybq_weight cybq_weight;
+
+typedef enum cybq_status {
+    CYBQ_OK = 0,
+    CYBQ_ERR_INVALID = -1,       /* null pointer, bad enum, bad size */
+    CYBQ_ERR_SHAPE = -2,         /* K % 32 != 0, M/N/K < 1, K mismatch */
+    CYBQ_ERR_ALIGN = -3,         /* x / y / out not aligned as documented */
+    CYBQ_ERR_NO_DEVICE = -4,     /* no HIP device, or not a gfx950 part */
+    CYBQ_ERR_HIP = -5,           /* a HIP runtime call failed; see cybq_last_error */
+    CYBQ_ERR_NOMEM = -6,
+    CYBQ_ERR_UNSUPPORTED = -7    /* valid request this build does not implement */
+} cybq_status;
+
+/* tensor data kinds of the container (/root/reference/decide/pipeline.md:28) */
+typedef enum cybq_quant { CYBQ_Q4 = 4, CYBQ_Q8 = 8 } cybq_quant;
+
+/* Interchange layouts accepted at upload.  W is [N,K] = [out,in]
+ * (/root/reference/decide/pipeline.md:30), groups of 32 run along K.
+ *   PLANAR     q plane then a separate scale plane.
+ *              Q4: q[N][K/2], byte j of a row = (w[2j] & 15) | (w[2j+1] & 15) << 4,
+ *                  two's-complement nibbles in -8..7;  Q8: q[N][K] int8.
+ *              scales[N][K/32] IEEE binary16.
+ *   BLOCK_AOS  [N][K/32] blocks, the Q4_0 / Q8_0 block shape named at
+ *              /root/reference/decide/pipeline.md:38 (18 B and 34 B per 32
+ *              weights, cf. shell/src/worlds/models/mod.rs:69-73):
+ *              Q4: f16 d, then 16 bytes, byte j = (w[j]+8) | (w[j+16]+8) << 4;
+ *              Q8: f16 d, then 32 int8.   `scales` must be NULL.
+ * On the device both are repacked once into one native tiled layout. */
+typedef enum cybq_layout { CYBQ_LAYOUT_PLANAR = 0, CYBQ_LAYOUT_BLOCK_AOS = 1 } cybq_layout;
+
+typedef enum cybq_dtype { CYBQ_F32 = 0, CYBQ_F16 = 1, CYBQ_BF16 = 2 } cybq_dtype;
+
+/* ---- context ---------------------------------------------------------- */
+
+/* Replaces: backend construction when the runtime is spawned
+ * (Soma::spawn(SomaConfig::default()) - shell/src/worlds/soma_bridge.rs:65). */
+int cybq_init(int device, cybq_ctx** out);
+void cybq_destroy(cybq_ctx* ctx);
+
+const char* cybq_strerror(int status);
+/* text of the last failure on this context (never NULL; "" when none) */
+const char* cybq_last_error(const cybq_ctx* ctx);
+/* "major.minor.patch" of the library */
+const char* cybq_version(void);
+
+/* ---- weights ---------------------------------------------------------- */
+
+/* Replaces: the load of one quantised tensor from the mmap'd .model file at
+ * model-switch time (use_model, lazy load - shell/src/worlds/models/mod.rs:7-8,386;
+ * "all conversion happens at import" - decide/pipeline.md:59: the repack to the
+ * device layout happens here, once, never in cybq_matmul).
+ * `q` / `scales` are host pointers (see cybq_layout); requires K % 32 == 0. */
+int cybq_weight_upload(cybq_ctx* ctx, cybq_quant quant, cybq_layout layout,
+                       int64_t N, int64_t K, const void* q, const void* scales,
+                       cybq_weight** out);
+/* A second device copy of the same tensor at a different address (used by
+ * benchmarks to stream more bytes than the last-level cache holds). */
+int cybq_weight_clone(cybq_ctx* ctx, const cybq_weight* src, cybq_weight** out);
+int cybq_weight_free(cybq_ctx* ctx, cybq_weight* w);
+/* any of the out pointers may be NULL.  device_bytes = bytes the tensor
+ * occupies in HBM (with padding of N to 16 and K to 128). */
+int cybq_weight_info(const cybq_weight* w, int* quant, int64_t* N, int64_t* K,
+                     int64_t* device_bytes);
+
+/* ---- the op ------------------------------------------------------------ */
+
+/* Replaces: execution of one block-quantized matmul node of the graph IR
+ * (decide/pipeline.md:28,51):   y[m,n] = sum_k x[m,k] * (scale[n,k/32] * q[n,k])
+ * with fp32 accumulation.
+ *   x  [M,K] row-major, xdt in {F16,BF16,F32}, 16-byte aligned
+ *   y  [M,N] row-major, ydt in {F32,F16,BF16} (fp32 accumulator rounded once)
+ *   M >= 1.  M <= 16 runs the HBM-streaming decode kernel, larger M the
+ *   LDS-tiled MFMA prefill kernel; there is no other path. */
+int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt,
+                int64_t M, void* y, cybq_dtype ydt, void* stream);
+
+/* Replaces: nothing the runtime calls per token; it is the verification hook
+ * ("dequantised weights match bit-exactly"): out[N,K] f32 = f32(scale) * q. */
+int cybq_dequant(cybq_ctx* ctx, const cybq_weight* w, float* out, void* stream);
+
+/* Replaces: the quantise step of the import pipeline
+ * (glia_import::pipeline::import_snapshot - shell/src/worlds/models/mod.rs:428;
+ * decide/pipeline.md:38-40).  src [N,K] f32 on the device; writes the PLANAR
+ * interchange layout to device buffers q_out ([N][K/2] or [N][K] bytes) and
+ * scales_out ([N][K/32] f16):  d = f16(absmax/qmax), q = clamp(round(w/d)). */
+int cybq_quantize(cybq_ctx* ctx, cybq_quant quant, const float* src, int64_t N, int64_t K,
+                  void* q_out, void* scales_out, void* stream);
+/* Builds a weight handle from PLANAR buffers that already live on the device
+ * (the output of cybq_quantize); stream-ordered, allocates the handle. */
+int cybq_weight_from_device(cybq_ctx* ctx, cybq_quant quant, int64_t N, int64_t K,
+                            const void* q_dev, const void* scales_dev, void* stream,
+                            cybq_weight** out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,321 @@
+"""Parity of the HIP path (through the C ABI) against the oracle, on an MI355X.
+
+Bars: dequantised weights bit-exact; matmul outputs within 1e-3 relative L2 of
+the float64 oracle (the fp32-accumulating kernels land near 1e-6, asserted at
+2e-5 for fp32 outputs so that a dropped group or a wrong scale cannot hide)."""
+import numpy as np
+import pytest
+
+from cyb_amd import QMatMul, formats, synth
+from cyb_amd.backend import CybqError
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3          # the operator's stated tolerance
+TIGHT = 2e-5        # what fp32 accumulation actually delivers
+
+TDT = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
+
+
+def _quant(oracle, bits, N, K, cfg=21):
+    w = synth.weights(cfg, N, K)
+    return oracle.quantize(w, bits)
+
+
+def _x(M, K, dt, cfg=21, outliers=0.0):
+    x = torch.from_numpy(synth.activations(cfg, M, K, outliers=outliers)).cuda().to(TDT[dt])
+    return x
+
+
+def _run(backend, qw, x, ydt="f32"):
+    M = x.shape[0]
+    y = torch.full((M, qw.N), float("nan"), dtype=TDT[ydt], device="cuda")
+    backend.matmul(qw, x, y)
+    torch.cuda.synchronize()
+    return y
+
+
+# ------------------------------------------------------------------ dequant
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("layout", [formats.PLANAR, formats.BLOCK_AOS])
+@pytest.mark.parametrize("shape", [(1, 32), (17, 160), (16, 128), (100, 4096), (1024, 4096)])
+def test_dequant_bit_exact(backend, oracle, bits, layout, shape):
+    N, K = shape
+    q, s = _quant(oracle, bits, N, K)
+    qw = backend.upload_quantized(q, s, bits, layout)
+    out = torch.empty((N, K), dtype=torch.float32, device="cuda")
+    backend.dequant(qw, out)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), oracle.dequant(q, s).view(np.uint32))
+    assert qw.algorithmic_bytes == formats.weight_bytes(bits, N, K)
+    qw.free()
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_dequant_exhaustive_scales_and_values(backend, oracle, bits):
+    # every finite f16 scale against every representable q (extremes included)
+    scales = np.arange(65536, dtype=np.uint16)
+    fin = np.isfinite(scales.view(np.float16))
+    scales = scales[fin]
+    qs = np.arange(-8, 8) if bits == 4 else np.arange(-128, 128)
+    reps = -(-len(qs) // 32)
+    qrow = np.resize(qs, reps * 32).astype(np.int8)
+    q = np.tile(qrow, (len(scales), 1))
+    s = np.repeat(scales[:, None], reps, axis=1)
+    qw = backend.upload_quantized(q, s, bits)
+    out = torch.empty(q.shape, dtype=torch.float32, device="cuda")
+    backend.dequant(qw, out)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), oracle.dequant(q, s).view(np.uint32))
+
+
+# ------------------------------------------------------------ decode (M <= 16)
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("xdt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 7, 8, 16])
+def test_decode_matches_oracle(backend, oracle, bits, xdt, M):
+    N, K = 272, 1024
+    q, s = _quant(oracle, bits, N, K)
+    qw = backend.upload_quantized(q, s, bits)
+    x = _x(M, K, xdt, outliers=0.001)
+    y = _run(backend, qw, x).cpu().numpy()
+    ref = oracle.matmul_f64(q, s, x.float().cpu().numpy())
+    err = oracle.rel_l2(y, ref)
+    assert err < TIGHT, err
+    # and against the fp32-accumulating CPU path itself
+    y32 = oracle.matmul_f32(q, s, x.float().cpu().numpy())
+    assert oracle.rel_l2(y, y32.astype(np.float64)) < TIGHT
+
+
+@pytest.mark.parametrize("shape", [(1, 32), (5, 64), (16, 128), (33, 160), (1000, 2080), (48, 32768)])
+def test_decode_ragged_shapes(backend, oracle, shape):
+    N, K = shape
+    q, s = _quant(oracle, 4, N, K)
+    qw = backend.upload_quantized(q, s, 4, formats.BLOCK_AOS)
+    for M in (1, 5, 16):
+        x = _x(M, K, "f16")
+        y = _run(backend, qw, x).cpu().numpy()
+        assert not np.isnan(y).any()
+        assert oracle.rel_l2(y, oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT
+
+
+def test_decode_long_k_uses_several_slabs(backend, oracle):
+    # M * K * 2 B exceeds the kernel's LDS budget: x is staged slab by slab
+    N, K = 64, 14336
+    q, s = _quant(oracle, 4, N, K)
+    qw = backend.upload_quantized(q, s, 4)
+    for M, xdt in ((16, "f16"), (8, "f32"), (3, "bf16")):
+        x = _x(M, K, xdt)
+        y = _run(backend, qw, x).cpu().numpy()
+        assert oracle.rel_l2(y, oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT
+
+
+def test_decode_batched_rows_equal_single_rows_bitwise(backend, oracle):
+    N, K = 512, 4096
+    q, s = _quant(oracle, 4, N, K)
+    qw = backend.upload_quantized(q, s, 4)
+    x = _x(16, K, "f16")
+    yb = _run(backend, qw, x)
+    for m in (0, 5, 15):
+        y1 = _run(backend, qw, x[m:m + 1].contiguous())
+        assert torch.equal(y1[0], yb[m])
+    # and the kernel is deterministic run to run
+    assert torch.equal(_run(backend, qw, x), yb)
+
+
+def test_decode_special_cases(backend, oracle):
+    N, K = 64, 256
+    ones = np.full((N, K // 32), 0x3C00, np.uint16)
+    # q = 0 -> 0 ; q = 1, d = 1 -> row sums of x
+    qw0 = backend.upload_quantized(np.zeros((N, K), np.int8), ones, 4)
+    x = _x(4, K, "f16")
+    assert not _run(backend, qw0, x).any()
+    qw1 = backend.upload_quantized(np.ones((N, K), np.int8), ones, 4)
+    y = _run(backend, qw1, x).cpu().numpy()
+    want = x.double().sum(dim=1).cpu().numpy()
+    assert np.allclose(y, np.repeat(want[:, None], N, axis=1), rtol=1e-5, atol=1e-4)
+    # one-hot x picks a dequantised column exactly
+    q, s = _quant(oracle, 4, N, K)
+    qw = backend.upload_quantized(q, s, 4)
+    wd = oracle.dequant(q, s)
+    for k in (0, 7, 8, 31, 32, 255):
+        e = torch.zeros((1, K), dtype=torch.float16, device="cuda")
+        e[0, k] = 1.0
+        assert np.array_equal(_run(backend, qw, e).cpu().numpy()[0], wd[:, k])
+    # extreme weights: every nibble value in every slot position
+    qe = np.resize(np.arange(-8, 8), (N, K)).astype(np.int8)
+    qe[1::2] = qe[1::2, ::-1]
+    qwe = backend.upload_quantized(qe, s, 4)
+    xe = _x(2, K, "f16")
+    assert oracle.rel_l2(_run(backend, qwe, xe).cpu().numpy(),
+                         oracle.matmul_f64(qe, s, xe.float().cpu().numpy())) < TIGHT
+
+
+@pytest.mark.parametrize("ydt", ["f16", "bf16"])
+def test_output_dtypes_round_once(backend, oracle, ydt):
+    N, K = 128, 512
+    q, s = _quant(oracle, 4, N, K)
+    qw = backend.upload_quantized(q, s, 4)
+    for M in (2, 40):
+        x = _x(M, K, "bf16" if M > 16 else "f16")
+        y32 = _run(backend, qw, x)
+        y16 = _run(backend, qw, x, ydt)
+        assert torch.equal(y16, y32.to(TDT[ydt]))
+
+
+def test_config1_q8_fp32_activations(backend, oracle):
+    q, s = _quant(oracle, 8, 2048, 2048, cfg=1)
+    qw = backend.upload_quantized(q, s, 8, formats.BLOCK_AOS)
+    x = _x(1, 2048, "f32", cfg=1)
+    y = _run(backend, qw, x).cpu().numpy()
+    assert oracle.rel_l2(y, oracle.matmul_f64(q, s, x.cpu().numpy())) < TIGHT
+
+
+@pytest.mark.parametrize("shape", [(4096, 4096), (4096, 1024), (4096, 14336), (14336, 4096)])
+def test_config2_and_3_full_size(backend, oracle, shape):
+    K, N = shape
+    q, s = _quant(oracle, 4, N, K, cfg=2)
+    qw = backend.upload_quantized(q, s, 4)
+    assert qw.algorithmic_bytes == formats.weight_bytes(4, N, K)
+    for M in (1, 4, 8, 16):
+        x = _x(M, K, "f16", cfg=3, outliers=0.001)
+        y = _run(backend, qw, x).cpu().numpy()
+        ref = oracle.matmul_f64(q, s, x[: min(M, 2)].float().cpu().numpy())
+        assert oracle.rel_l2(y[: min(M, 2)], ref) < TIGHT
+        # remaining rows: float64 library matmul on the dequantised weights
+        full = x.double().cpu().numpy() @ oracle.dequant(q, s).astype(np.float64).T
+        assert oracle.rel_l2(y, full) < TIGHT
+
+
+# ------------------------------------------------------------ prefill (M > 16)
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("xdt", ["bf16", "f16", "f32"])
+@pytest.mark.parametrize("M", [17, 64, 300])
+def test_prefill_matches_oracle(backend, oracle, bits, xdt, M):
+    N, K = 240, 512
+    q, s = _quant(oracle, bits, N, K)
+    qw = backend.upload_quantized(q, s, bits)
+    x = _x(M, K, xdt)
+    y = _run(backend, qw, x).cpu().numpy()
+    assert not np.isnan(y).any()
+    err = oracle.rel_l2(y, oracle.matmul_f64(q, s, x.float().cpu().numpy()))
+    assert err < TIGHT, err
+
+
+@pytest.mark.parametrize("shape", [(17, 32), (112, 160), (113, 96), (130, 2080)])
+def test_prefill_ragged_shapes(backend, oracle, shape):
+    N, K = shape
+    q, s = _quant(oracle, 4, N, K)
+    qw = backend.upload_quantized(q, s, 4)
+    for M in (17, 257):
+        x = _x(M, K, "bf16")
+        y = _run(backend, qw, x).cpu().numpy()
+        assert not np.isnan(y).any()
+        assert oracle.rel_l2(y, oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT
+
+
+def test_prefill_rows_agree_with_decode_rows(backend, oracle):
+    N, K = 448, 1024
+    q, s = _quant(oracle, 4, N, K)
+    qw = backend.upload_quantized(q, s, 4)
+    x = _x(64, K, "bf16")
+    yp = _run(backend, qw, x)
+    yd = _run(backend, qw, x[:16].contiguous())
+    num = (yp[:16] - yd).double().norm() / yd.double().norm()
+    assert num.item() < TIGHT
+    assert torch.equal(_run(backend, qw, x), yp)            # deterministic
+
+
+@pytest.mark.parametrize("M", [128, 512])
+@pytest.mark.parametrize("shape", [(4096, 14336), (14336, 4096)])
+def test_config4_full_size(backend, oracle, M, shape):
+    K, N = shape
+    q, s = _quant(oracle, 4, N, K, cfg=4)
+    qw = backend.upload_quantized(q, s, 4)
+    x = _x(M, K, "bf16", cfg=4)
+    y = _run(backend, qw, x)
+    wd = torch.from_numpy(oracle.dequant(q, s)).cuda().double()
+    full = (x.double() @ wd.T)
+    err = ((y.double() - full).norm() / full.norm()).item()
+    assert err < TIGHT, err
+    # the oracle itself on a few rows
+    rows = [0, M // 2, M - 1]
+    ref = oracle.matmul_f64(q, s, x[rows].float().cpu().numpy())
+    assert oracle.rel_l2(y[rows].cpu().numpy(), ref) < TIGHT
+    # linearity in x: f(2x) == 2 f(x) exactly (powers of two commute with every rounding)
+    y2 = _run(backend, qw, (x * 2).contiguous())
+    assert torch.equal(y2, y * 2)
+
+
+# ------------------------------------------------------------------ quantise
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_device_quantizer_bit_exact(backend, oracle, bits):
+    N, K = 300, 1024
+    w = synth.weights(31, N, K)
+    w[0, :32] = 0
+    w[1, 32:64] *= 1e-6
+    w[2, 5] = 0.35
+    src = torch.from_numpy(w).cuda()
+    qd = torch.empty(N * K * bits // 8, dtype=torch.uint8, device="cuda")
+    sd = torch.empty(N * K // 32, dtype=torch.int16, device="cuda")
+    backend.quantize(bits, src, N, K, qd, sd)
+    torch.cuda.synchronize()
+    q, s = oracle.quantize(w, bits)
+    assert np.array_equal(sd.cpu().numpy().view(np.uint16).reshape(N, -1), s)
+    assert np.array_equal(qd.cpu().numpy(), oracle.pack_planar(q, bits))
+    # device buffers -> weight handle -> the op, without touching the host
+    qw = backend.weight_from_device(bits, N, K, qd, sd)
+    out = torch.empty((N, K), dtype=torch.float32, device="cuda")
+    backend.dequant(qw, out)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), oracle.dequant(q, s).view(np.uint32))
+
+
+# ------------------------------------------------------------ interface / errors
+
+def test_graph_node_execution(backend, oracle):
+    N, K = 64, 128
+    q, s = _quant(oracle, 4, N, K)
+    backend.upload_quantized(q, s, 4, name="model.layers.0.self_attn.q_proj.weight")
+    node = QMatMul(w="model.layers.0.self_attn.q_proj.weight", x="h0", y="q0", quant=4, M=2, N=N, K=K)
+    edges = {"h0": _x(2, K, "f16"), "q0": torch.empty((2, N), dtype=torch.float32, device="cuda")}
+    backend.run(node, edges)
+    torch.cuda.synchronize()
+    assert oracle.rel_l2(edges["q0"].cpu().numpy(),
+                         oracle.matmul_f64(q, s, edges["h0"].float().cpu().numpy())) < TIGHT
+    with pytest.raises(CybqError):
+        backend.run(QMatMul(w="missing", x="h0", y="q0"), edges)
+    with pytest.raises(CybqError):
+        backend.run(QMatMul(w=node.w, x="h0", y="q0", quant=4, N=N + 16, K=K), edges)
+
+
+def test_error_codes(backend, oracle):
+    q, s = _quant(oracle, 4, 16, 64)
+    with pytest.raises(CybqError) as e:
+        backend.upload(4, formats.PLANAR, 16, 48, formats.pack_planar(q, 4), s)       # K % 32
+    assert e.value.status == -2
+    with pytest.raises(CybqError) as e:
+        backend.upload(4, formats.PLANAR, 16, 64, formats.pack_planar(q, 4), None)    # no scales
+    assert e.value.status == -1
+    with pytest.raises(CybqError) as e:
+        backend.upload(5, formats.PLANAR, 16, 64, formats.pack_planar(q, 4), s)       # bad quant
+    assert e.value.status == -1
+    qw = backend.upload_quantized(q, s, 4)
+    x = _x(2, 64, "f16")
+    y = torch.empty((2, 16), dtype=torch.float32, device="cuda")
+    with pytest.raises(CybqError) as e:
+        backend.matmul(qw, x, y, M=0)
+    assert e.value.status == -2
+    buf = torch.empty(2 * 64 + 8, dtype=torch.float16, device="cuda")
+    with pytest.raises(CybqError) as e:
+        backend.matmul(qw, buf.data_ptr() + 2, y, M=2, xdt=1)                         # misaligned x
+    assert e.value.status == -3
+    # the context stays usable after errors
+    backend.matmul(qw, x, y)
+    torch.cuda.synchronize()
+    assert oracle.rel_l2(y.cpu().numpy(), oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT
