@@ -224,18 +224,30 @@ hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt,
 {
     const int planes = XMODE == XF32 ? 2 : 1;
     const int budget = 64 * 1024;
+    // x is staged in K slabs that fit the LDS budget.  A slab is a whole number
+    // of rounds over the waves, so which wave owns tile kt (kt % nwaves) - and
+    // with it the summation order - does not depend on M.
     int slab_tiles = w.KT;
     if ((int64_t)M * (w.KT * kTileK + 8) * 2 * planes > budget) {
         int k_fit = budget / (2 * M * planes) - 8;
         slab_tiles = k_fit / kTileK;
         int step = nwaves * U;
-        if (slab_tiles > step) slab_tiles -= slab_tiles % step;
-        if (slab_tiles < 1) slab_tiles = 1;
+        if (slab_tiles >= step) slab_tiles -= slab_tiles % step;
+        else slab_tiles -= slab_tiles % nwaves;
+        if (slab_tiles < nwaves) slab_tiles = nwaves;
     }
     int ldx = slab_tiles * kTileK + 8;
     size_t lds = (size_t)M * ldx * 2 * planes;
     size_t red = (size_t)nwaves * RMAX * 64 * sizeof(float);
     if (lds < red) lds = red;
+    static bool attr_set = false;
+    if (!attr_set) {
+        // M = 16 fp32 activations with 8 waves need 66 KB, just over the default cap
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_kernel<BITS, XMODE, RMAX, U>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
     hipLaunchKernelGGL((gemv_kernel<BITS, XMODE, RMAX, U>), dim3(w.NT), dim3(nwaves * 64), lds, st,
                        w, x, M, y, ydt, slab_tiles, ldx);
     return hipGetLastError();
