@@ -77,6 +77,7 @@ def load_library() -> ctypes.CDLL:
     lib.cybq_weight_info.argtypes = [vp, ctypes.POINTER(ci), ctypes.POINTER(i64), ctypes.POINTER(i64),
                                      ctypes.POINTER(i64)]
     lib.cybq_matmul.argtypes = [vp, vp, vp, ci, i64, vp, ci, vp]
+    lib.cybq_matmul_many.argtypes = [vp, i64, vp, vp, vp, ci, i64, ci, vp]
     lib.cybq_dequant.argtypes = [vp, vp, vp, vp]
     lib.cybq_quantize.argtypes = [vp, ci, vp, i64, i64, vp, vp, vp]
     lib.cybq_debug_set_gemv_tuning.argtypes = [ci, ci, ci]
@@ -155,6 +156,23 @@ class QWeight:
             self.free()
         except Exception:
             pass
+
+
+class MatmulPlan:
+    """Pointer arrays of a fixed node list (one decode step's linears)."""
+
+    def __init__(self, backend: "Backend", weights, xs, ys):
+        n = len(weights)
+        if not (n == len(xs) == len(ys)):
+            raise CybqError(-1, "invalid argument", "weights / xs / ys differ in length")
+        self.count = n
+        self.keep = (list(weights), list(xs), list(ys))      # keeps tensors and handles alive
+        arr = ctypes.c_void_p * n
+        self.w = arr(*[w.handle.value for w in weights])
+        self.x = arr(*[_ptr(t) for t in xs])
+        self.y = arr(*[_ptr(t) for t in ys])
+        self.xdt = _dtype_code(xs[0], None) if n else F16
+        self.ydt = _dtype_code(ys[0], None) if n else F32
 
 
 class Backend:
@@ -236,6 +254,14 @@ class Backend:
             M = int(x.shape[0]) if x.dim() == 2 else 1
         self._check(self._lib.cybq_matmul(self._ctx, w.handle, _ptr(x), _dtype_code(x, xdt), M, _ptr(y),
                                           _dtype_code(y, ydt), stream))
+
+    def plan_many(self, weights, xs, ys) -> "MatmulPlan":
+        """Freezes a list of (weight, x, y) nodes into pointer arrays for matmul_many."""
+        return MatmulPlan(self, weights, xs, ys)
+
+    def matmul_many(self, plan: "MatmulPlan", M: int, stream: int = 0) -> None:
+        self._check(self._lib.cybq_matmul_many(self._ctx, plan.count, plan.w, plan.x, plan.y, plan.xdt, M,
+                                               plan.ydt, stream))
 
     def dequant(self, w: QWeight, out, stream: int = 0) -> None:
         self._check(self._lib.cybq_dequant(self._ctx, w.handle, _ptr(out), stream))

@@ -308,6 +308,18 @@ int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype x
     return CYBQ_OK;
 }
 
+int cybq_matmul_many(cybq_ctx* ctx, int64_t count, const cybq_weight* const* w, const void* const* x,
+                     void* const* y, cybq_dtype xdt, int64_t M, cybq_dtype ydt, void* stream)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (count < 0 || (count > 0 && (!w || !x || !y))) return fail(ctx, CYBQ_ERR_INVALID, "bad node list");
+    for (int64_t i = 0; i < count; i++) {
+        int rc = cybq_matmul(ctx, w[i], x[i], xdt, M, y[i], ydt, stream);
+        if (rc) return rc;
+    }
+    return CYBQ_OK;
+}
+
 int cybq_dequant(cybq_ctx* ctx, const cybq_weight* w, float* out, void* stream)
 {
     if (!ctx) return CYBQ_ERR_INVALID;
@@ -340,9 +352,9 @@ int cybq_quantize(cybq_ctx* ctx, cybq_quant quant, const float* src, int64_t N, 
 
 /* Test and benchmark hook (not part of the operator interface): overrides the
  * decode kernel's launch heuristics; 0 restores the automatic choice. */
-int cybq_debug_set_gemv_tuning(int waves_per_group, int strips_per_group, int unroll)
+int cybq_debug_set_gemv_tuning(int waves_per_group, int reserved, int unroll)
 {
-    cybq::set_gemv_tuning(waves_per_group, strips_per_group, unroll);
+    cybq::set_gemv_tuning(waves_per_group, reserved, unroll);
     return CYBQ_OK;
 }
 

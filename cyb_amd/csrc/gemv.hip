@@ -130,8 +130,10 @@ __device__ __forceinline__ void compute_tile(const TileRegs<BITS>& t, const uint
     }
 }
 
-// U = tiles a wave keeps in flight per batch (two batches are live: ping-pong).
-template <int BITS, int XMODE, int RMAX, int U>
+// U = tiles a wave keeps in flight per batch.  ONESHOT: the wave's whole share
+// of the strip is at most U tiles, all requested before anything else happens
+// (one register set); otherwise two batches are live and ping-pong.
+template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT>
 __global__ __launch_bounds__(512) void gemv_kernel(WeightView w, const void* __restrict__ x, int M, void* __restrict__ y,
                             int ydt, int slab_tiles, int ldx)
 {
@@ -154,6 +156,22 @@ __global__ __launch_bounds__(512) void gemv_kernel(WeightView w, const void* __r
 #pragma unroll
     for (int r = 0; r < RMAX; r++) acc[r] = 0.f;
 
+    if (ONESHOT) {
+        TileRegs<BITS> buf[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            int i = wv + u * nwaves;
+            if (i < w.KT) load_tile<BITS>(buf[u], w, strip + i, lane);
+        }
+        stage_x<XMODE>(xs, x, M, w.K, 0, w.KT * kTileK, ldx, plane_elems, tid, nthreads);
+        __syncthreads();
+        const uint16_t* xbase = xs + mrow * ldx + oct * 8;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            int i = wv + u * nwaves;
+            if (i < w.KT) compute_tile<BITS, XMODE, RMAX>(buf[u], xbase + i * kTileK, plane_elems, acc);
+        }
+    } else {
     TileRegs<BITS> bufA[U], bufB[U];
 
     for (int slab0 = 0; slab0 < w.KT; slab0 += slab_tiles) {
@@ -197,6 +215,7 @@ __global__ __launch_bounds__(512) void gemv_kernel(WeightView w, const void* __r
             }
         }
     }
+    }
 
     // split-K partials -> LDS, summed in wave order by wave 0
     __syncthreads();
@@ -218,18 +237,19 @@ __global__ __launch_bounds__(512) void gemv_kernel(WeightView w, const void* __r
 
 int g_tune_waves = 0, g_tune_unroll = 0;
 
-template <int BITS, int XMODE, int RMAX, int U>
+constexpr int kLdsBudget = 64 * 1024;
+
+template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT>
 hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves,
                     hipStream_t st)
 {
     const int planes = XMODE == XF32 ? 2 : 1;
-    const int budget = 64 * 1024;
     // x is staged in K slabs that fit the LDS budget.  A slab is a whole number
     // of rounds over the waves, so which wave owns tile kt (kt % nwaves) - and
     // with it the summation order - does not depend on M.
     int slab_tiles = w.KT;
-    if ((int64_t)M * (w.KT * kTileK + 8) * 2 * planes > budget) {
-        int k_fit = budget / (2 * M * planes) - 8;
+    if (!ONESHOT && (int64_t)M * (w.KT * kTileK + 8) * 2 * planes > kLdsBudget) {
+        int k_fit = kLdsBudget / (2 * M * planes) - 8;
         slab_tiles = k_fit / kTileK;
         int step = nwaves * U;
         if (slab_tiles >= step) slab_tiles -= slab_tiles % step;
@@ -240,37 +260,42 @@ hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt,
     size_t lds = (size_t)M * ldx * 2 * planes;
     size_t red = (size_t)nwaves * RMAX * 64 * sizeof(float);
     if (lds < red) lds = red;
+    auto kern = gemv_kernel<BITS, XMODE, RMAX, U, ONESHOT>;
     static bool attr_set = false;
     if (!attr_set) {
         // M = 16 fp32 activations with 8 waves need 66 KB, just over the default cap
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_kernel<BITS, XMODE, RMAX, U>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    hipLaunchKernelGGL((gemv_kernel<BITS, XMODE, RMAX, U>), dim3(w.NT), dim3(nwaves * 64), lds, st,
-                       w, x, M, y, ydt, slab_tiles, ldx);
+    hipLaunchKernelGGL(kern, dim3(w.NT), dim3(nwaves * 64), lds, st, w, x, M, y, ydt, slab_tiles, ldx);
     return hipGetLastError();
 }
 
-template <int BITS, int XMODE, int U>
+template <int BITS, int XMODE, int U, bool ONESHOT>
 hipError_t launch_r(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves,
                     hipStream_t st)
 {
-    if (M == 1) return launch_t<BITS, XMODE, 1, U>(w, x, M, y, ydt, nwaves, st);
-    if (M == 2) return launch_t<BITS, XMODE, 2, U>(w, x, M, y, ydt, nwaves, st);
-    return launch_t<BITS, XMODE, 4, U>(w, x, M, y, ydt, nwaves, st);
+    if (M == 1) return launch_t<BITS, XMODE, 1, U, ONESHOT>(w, x, M, y, ydt, nwaves, st);
+    if (M == 2) return launch_t<BITS, XMODE, 2, U, ONESHOT>(w, x, M, y, ydt, nwaves, st);
+    return launch_t<BITS, XMODE, 4, U, ONESHOT>(w, x, M, y, ydt, nwaves, st);
 }
 
 template <int BITS, int XMODE>
 hipError_t launch_u(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, int unroll,
                     hipStream_t st)
 {
-    if (BITS == 4 && XMODE == XF16) {
-        if (unroll == 2) return launch_r<BITS, XMODE, 2>(w, x, M, y, ydt, nwaves, st);
-        if (unroll == 8) return launch_r<BITS, XMODE, 8>(w, x, M, y, ydt, nwaves, st);
+    const int planes = XMODE == XF32 ? 2 : 1;
+    const bool one_slab = (int64_t)M * (w.KT * kTileK + 8) * 2 * planes <= kLdsBudget;
+    const int per_wave = (w.KT + nwaves - 1) / nwaves;
+    if (one_slab && unroll == 0) {
+        if (per_wave <= 4) return launch_r<BITS, XMODE, 4, true>(w, x, M, y, ydt, nwaves, st);
+        if (per_wave <= 8) return launch_r<BITS, XMODE, 8, true>(w, x, M, y, ydt, nwaves, st);
+        if (per_wave <= 16) return launch_r<BITS, XMODE, 16, true>(w, x, M, y, ydt, nwaves, st);
     }
-    return launch_r<BITS, XMODE, 4>(w, x, M, y, ydt, nwaves, st);
+    if (unroll == 4) return launch_r<BITS, XMODE, 4, false>(w, x, M, y, ydt, nwaves, st);
+    return launch_r<BITS, XMODE, 2, false>(w, x, M, y, ydt, nwaves, st);
 }
 
 }  // namespace
@@ -294,7 +319,8 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
     }
     if (nwaves > 8) nwaves = 8;   // the kernel is compiled for at most 512 threads
     while (nwaves > 1 && nwaves > w.KT) nwaves >>= 1;
-    int unroll = g_tune_unroll > 0 ? g_tune_unroll : 4;
+    // 0: request a wave's whole share up front when it fits, else stream in batches of 2
+    int unroll = g_tune_unroll;
 
     if (w.bits == 4) {
         if (xdt == kF16) return launch_u<4, XF16>(w, x, M, y, ydt, nwaves, unroll, st);

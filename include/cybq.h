@@ -118,6 +118,16 @@ int cybq_weight_info(const cybq_weight* w, int* quant, int64_t* N, int64_t* K,
 int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt,
                 int64_t M, void* y, cybq_dtype ydt, void* stream);
 
+/* Replaces: the executor's walk over the quantised-matmul nodes of one decode
+ * step (7 linears per layer x layers + LM head - decide/pipeline.md:51): `count`
+ * independent invocations of cybq_matmul launched back to back on `stream`
+ * from native code, so the host cost per node is one kernel launch.
+ * w[i], x[i], y[i] as in cybq_matmul; all share M, xdt, ydt.  Stops at the
+ * first failing node and returns its status. */
+int cybq_matmul_many(cybq_ctx* ctx, int64_t count, const cybq_weight* const* w,
+                     const void* const* x, void* const* y, cybq_dtype xdt, int64_t M,
+                     cybq_dtype ydt, void* stream);
+
 /* Replaces: nothing the runtime calls per token; it is the verification hook
  * ("dequantised weights match bit-exactly"): out[N,K] f32 = f32(scale) * q. */
 int cybq_dequant(cybq_ctx* ctx, const cybq_weight* w, float* out, void* stream);
@@ -134,6 +144,13 @@ int cybq_quantize(cybq_ctx* ctx, cybq_quant quant, const float* src, int64_t N, 
 int cybq_weight_from_device(cybq_ctx* ctx, cybq_quant quant, int64_t N, int64_t K,
                             const void* q_dev, const void* scales_dev, void* stream,
                             cybq_weight** out);
+
+/* ---- diagnostics (not part of the operator interface) ------------------- */
+
+/* Overrides the decode kernel's launch heuristics for experiments: waves per
+ * workgroup (1..8), reserved, tiles in flight per wave (2, 4 or 8); 0 restores
+ * the automatic choice.  Process-wide. */
+int cybq_debug_set_gemv_tuning(int waves_per_group, int reserved, int unroll);
 
 #ifdef __cplusplus
 }
