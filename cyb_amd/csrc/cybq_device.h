@@ -55,11 +55,24 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t bits16)
 // nibble position of weight slot s inside a native Q4 word
 __host__ __device__ __forceinline__ int q4_nibble_pos(int s) { return (s >> 1) + 4 * (s & 1); }
 
+// The f16 magic constant 0x64006400 held in a vector register whose value the
+// compiler cannot see.  With it (w & mask) | magic compiles to one v_and_or_b32
+// (a gfx9 VOP3 encoding may read only one scalar, so with two visible constants
+// the compiler emits a separate and + or).  Call once at kernel entry, before
+// any MFMA is in flight: the hazard recogniser does not look inside asm.
+__device__ __forceinline__ uint32_t q4_magic_vgpr()
+{
+    uint32_t mv;
+    asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(mv));
+    return mv;
+}
+
 // One native Q4 word -> 8 exact f16 integers in MFMA operand order.
 // 0x6400 | u is the f16 number 1024 + u; 0x6400 | (u << 4) is 1024 + 16u.
-__device__ __forceinline__ void unpack_q4_f16(uint32_t w, uint32_t out[4])
+// `magic` = q4_magic_vgpr().
+__device__ __forceinline__ void unpack_q4_f16(uint32_t w, uint32_t magic, uint32_t out[4])
 {
-    const uint32_t lo = 0x000F000Fu, hi = 0x00F000F0u, magic = 0x64006400u;
+    const uint32_t lo = 0x000F000Fu, hi = 0x00F000F0u;
     const half2_t sub = {(_Float16)-1032.0f, (_Float16)-1032.0f};
     const half2_t mul = {(_Float16)0.0625f, (_Float16)0.0625f};
     const half2_t add = {(_Float16)-72.0f, (_Float16)-72.0f};

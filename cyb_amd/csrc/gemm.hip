@@ -44,6 +44,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(WeightView w, const uint16_t*
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     u32x4_t* xs = reinterpret_cast<u32x4_t*>(smem);                    // [MFRAGS][4][64]
     u32x4_t* ws = xs + MFRAGS * 4 * 64;                                // [NF][4][64]
+    const uint32_t magic = q4_magic_vgpr();
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -88,7 +89,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(WeightView w, const uint16_t*
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 uint32_t bw[4];
-                if (BITS == 4) unpack_q4_f16(q0[j], bw);
+                if (BITS == 4) unpack_q4_f16(q0[j], magic, bw);
                 else if (j < 2) unpack_q8_f16(q0[(j & 1) * 2], q0[(j & 1) * 2 + 1], bw);
                 else unpack_q8_f16(q1[(j & 1) * 2], q1[(j & 1) * 2 + 1], bw);
                 if (XBF) f16frag_to_bf16frag(bw);

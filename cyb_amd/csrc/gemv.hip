@@ -97,37 +97,81 @@ __device__ __forceinline__ void stage_x(uint16_t* xs, const void* x, int M, int 
     }
 }
 
-template <int BITS, int XMODE, int RMAX>
-__device__ __forceinline__ void compute_tile(const TileRegs<BITS>& t, const uint16_t* xrow,
-                                             int plane_elems, float acc[RMAX])
+// One tile = 4 scale groups.  tile_issue reads the four x operands from LDS,
+// unpacks the four weight operands and issues the four MFMAs back to back into
+// separate result registers; tile_accum folds the group scales in afterwards.
+// Callers run tile_accum one tile late, so the MFMA latency is covered by the
+// next tile's unpack instead of by wait states.
+template <int BITS, int XMODE>
+__device__ __forceinline__ void tile_issue(const TileRegs<BITS>& t, const uint16_t* xrow, int plane_elems,
+                                           uint32_t magic, float4_t d[4])
 {
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+    Frag16 a[4], al[4], b[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        Frag16 b;
+        a[j].u = *reinterpret_cast<const u32x4_t*>(xrow + j * 32);
+        if (XMODE == XF32) al[j].u = *reinterpret_cast<const u32x4_t*>(xrow + plane_elems + j * 32);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
         uint32_t bw[4];
-        if (BITS == 4) unpack_q4_f16(t.q[0][j], bw);
+        if (BITS == 4) unpack_q4_f16(t.q[0][j], magic, bw);
         else unpack_q8_f16(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
         if (XMODE == XBF16) f16frag_to_bf16frag(bw);
-        b.u = (u32x4_t){bw[0], bw[1], bw[2], bw[3]};
-        Frag16 a;
-        a.u = *reinterpret_cast<const u32x4_t*>(xrow + j * 32);
-        float4_t d;
+        b[j].u = (u32x4_t){bw[0], bw[1], bw[2], bw[3]};
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
         if (XMODE == XBF16) {
-            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, zero, 0, 0, 0);
+            d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].b, b[j].b, zero, 0, 0, 0);
         } else {
-            d = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, zero, 0, 0, 0);
-            if (XMODE == XF32) {
-                Frag16 al;
-                al.u = *reinterpret_cast<const u32x4_t*>(xrow + plane_elems + j * 32);
-                d = __builtin_amdgcn_mfma_f32_16x16x32_f16(al.h, b.h, d, 0, 0, 0);
-            }
+            d[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j].h, b[j].h, zero, 0, 0, 0);
+            if (XMODE == XF32) d[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al[j].h, b[j].h, d[j], 0, 0, 0);
         }
-        uint32_t sb = (j & 1) ? (t.s[j >> 1] >> 16) : (t.s[j >> 1] & 0xffffu);
+    }
+}
+
+template <int RMAX>
+__device__ __forceinline__ void tile_accum(u32x2_t s, const float4_t d[4], float acc[RMAX])
+{
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        uint32_t sb = (j & 1) ? (s[j >> 1] >> 16) : (s[j >> 1] & 0xffffu);
         float sc = f16_bits_to_f32(sb);
 #pragma unroll
-        for (int r = 0; r < RMAX; r++) acc[r] = __builtin_fmaf(sc, d[r], acc[r]);
+        for (int r = 0; r < RMAX; r++) acc[r] = __builtin_fmaf(sc, d[j][r], acc[r]);
     }
+}
+
+// Runs a batch of U tiles (tile index i0 + u * nwaves, valid while < limit).
+template <int BITS, int XMODE, int RMAX, int U>
+__device__ __forceinline__ void compute_batch(const TileRegs<BITS> (&buf)[U], int i0, int nwaves, int limit,
+                                              const uint16_t* xbase, int plane_elems, uint32_t magic,
+                                              float acc[RMAX])
+{
+    float4_t dprev[4];
+    u32x2_t sprev = {0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 4; j++) dprev[j] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int i = i0 + u * nwaves;
+        float4_t d[4];
+        u32x2_t sc = {0u, 0u};
+        if (i < limit) {
+            tile_issue<BITS, XMODE>(buf[u], xbase + i * kTileK, plane_elems, magic, d);
+            sc = buf[u].s;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) d[j] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        }
+        tile_accum<RMAX>(sprev, dprev, acc);
+#pragma unroll
+        for (int j = 0; j < 4; j++) dprev[j] = d[j];
+        sprev = sc;
+    }
+    tile_accum<RMAX>(sprev, dprev, acc);
 }
 
 // U = tiles a wave keeps in flight per batch.  ONESHOT: the wave's whole share
@@ -139,11 +183,12 @@ __global__ __launch_bounds__(512) void gemv_kernel(WeightView w, const void* __r
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t* xs = reinterpret_cast<uint16_t*>(smem);
+    const uint32_t magic = q4_magic_vgpr();
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const int lane = tid & 63;
-    const int wv = tid >> 6;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: tile guards become scalar branches
     const int nwaves = nthreads >> 6;
     const int nt = blockIdx.x;
     const int mrow = min(lane & 15, M - 1);
@@ -166,11 +211,7 @@ __global__ __launch_bounds__(512) void gemv_kernel(WeightView w, const void* __r
         stage_x<XMODE>(xs, x, M, w.K, 0, w.KT * kTileK, ldx, plane_elems, tid, nthreads);
         __syncthreads();
         const uint16_t* xbase = xs + mrow * ldx + oct * 8;
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            int i = wv + u * nwaves;
-            if (i < w.KT) compute_tile<BITS, XMODE, RMAX>(buf[u], xbase + i * kTileK, plane_elems, acc);
-        }
+        compute_batch<BITS, XMODE, RMAX, U>(buf, wv, nwaves, w.KT, xbase, plane_elems, magic, acc);
     } else {
     TileRegs<BITS> bufA[U], bufB[U];
 
@@ -196,11 +237,7 @@ __global__ __launch_bounds__(512) void gemv_kernel(WeightView w, const void* __r
                 int i = i1 + u * nwaves;
                 if (i < st) load_tile<BITS>(bufB[u], w, strip + slab0 + i, lane);
             }
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                int i = i0 + u * nwaves;
-                if (i < st) compute_tile<BITS, XMODE, RMAX>(bufA[u], xbase + i * kTileK, plane_elems, acc);
-            }
+            compute_batch<BITS, XMODE, RMAX, U>(bufA, i0, nwaves, st, xbase, plane_elems, magic, acc);
             // ---- bufB holds batch i1; fetch batch i1 + stride into bufA
             const int i2 = i1 + stride;
 #pragma unroll
@@ -208,11 +245,7 @@ __global__ __launch_bounds__(512) void gemv_kernel(WeightView w, const void* __r
                 int i = i2 + u * nwaves;
                 if (i < st) load_tile<BITS>(bufA[u], w, strip + slab0 + i, lane);
             }
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                int i = i1 + u * nwaves;
-                if (i < st) compute_tile<BITS, XMODE, RMAX>(bufB[u], xbase + i * kTileK, plane_elems, acc);
-            }
+            compute_batch<BITS, XMODE, RMAX, U>(bufB, i1, nwaves, st, xbase, plane_elems, magic, acc);
         }
     }
     }
@@ -292,7 +325,8 @@ hipError_t launch_u(const WeightView& w, const void* x, int M, void* y, int ydt,
     if (one_slab && unroll == 0) {
         if (per_wave <= 4) return launch_r<BITS, XMODE, 4, true>(w, x, M, y, ydt, nwaves, st);
         if (per_wave <= 8) return launch_r<BITS, XMODE, 8, true>(w, x, M, y, ydt, nwaves, st);
-        if (per_wave <= 16) return launch_r<BITS, XMODE, 16, true>(w, x, M, y, ydt, nwaves, st);
+        // 16 tiles in flight fit the register file only with one or two batch rows
+        if (per_wave <= 16 && M <= 2) return launch_r<BITS, XMODE, 16, true>(w, x, M, y, ydt, nwaves, st);
     }
     if (unroll == 4) return launch_r<BITS, XMODE, 4, false>(w, x, M, y, ydt, nwaves, st);
     return launch_r<BITS, XMODE, 2, false>(w, x, M, y, ydt, nwaves, st);

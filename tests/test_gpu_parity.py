@@ -113,6 +113,27 @@ def test_decode_long_k_uses_several_slabs(backend, oracle):
         assert oracle.rel_l2(y, oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+def test_decode_every_kernel_variant(backend, oracle, bits):
+    # the launch heuristics pick among one-shot (4 / 8 / 16 tiles in flight) and
+    # streaming (2 / 4 tiles per batch) variants; force each of them
+    N, K = 80, 4096
+    q, s = _quant(oracle, bits, N, K)
+    qw = backend.upload_quantized(q, s, bits)
+    try:
+        for M in (1, 2, 4, 9):
+            x = _x(M, K, "f16")
+            ref = oracle.matmul_f64(q, s, x.float().cpu().numpy())
+            for waves in (1, 2, 4, 8):
+                for unroll in (0, 2, 4):
+                    backend.set_gemv_tuning(waves, 0, unroll)
+                    y = _run(backend, qw, x).cpu().numpy()
+                    err = oracle.rel_l2(y, ref)
+                    assert err < TIGHT, (M, waves, unroll, err)
+    finally:
+        backend.set_gemv_tuning(0, 0, 0)
+
+
 def test_decode_batched_rows_equal_single_rows_bitwise(backend, oracle):
     N, K = 512, 4096
     q, s = _quant(oracle, 4, N, K)
