@@ -58,42 +58,86 @@ __device__ __forceinline__ void store_out(void* y, int ydt, int64_t idx, float v
 }
 
 // x rows of one K slab -> LDS (row stride ldx 16-bit elements; XF32: a second
-// plane of low halves follows the first at plane_elems).
+// plane of low halves follows the first at plane_elems).  Split in two so that
+// the global loads can be issued BEFORE the weight loads: vmcnt retires in
+// order, so an x load issued after them could only be waited for together with
+// every weight tile, and nothing would overlap the HBM stream.
+constexpr int kXChunks = 4;     // 8-element chunks of x a thread carries in registers
+
 template <int XMODE>
-__device__ __forceinline__ void stage_x(uint16_t* xs, const void* x, int M, int K, int k_begin,
-                                        int slab_k, int ldx, int plane_elems, int tid, int nthreads)
+struct XRegs {
+    u32x4_t v[kXChunks][XMODE == XF32 ? 2 : 1];
+};
+
+template <int XMODE>
+__device__ __forceinline__ void stage_x_load(XRegs<XMODE>& r, const void* x, int M, int K, int k_begin,
+                                             int slab_k, int first_chunk, int tid, int nthreads)
 {
     const int chunks_per_row = slab_k >> 3;
     const int total = M * chunks_per_row;
-    for (int c = tid; c < total; c += nthreads) {
-        int row = c / chunks_per_row;
-        int col = (c - row * chunks_per_row) << 3;
-        int k = k_begin + col;
-        u32x4_t* dst = reinterpret_cast<u32x4_t*>(xs + row * ldx + col);
+#pragma unroll
+    for (int c = 0; c < kXChunks; c++) {
+        const int idx = first_chunk + tid + c * nthreads;
+        const int row = idx / chunks_per_row;
+        const int k = k_begin + ((idx - row * chunks_per_row) << 3);
+        const bool live = idx < total && k < K;
         if (XMODE != XF32) {
             u32x4_t v = {0u, 0u, 0u, 0u};
-            if (k < K) v = *reinterpret_cast<const u32x4_t*>(
-                           reinterpret_cast<const uint16_t*>(x) + (int64_t)row * K + k);
-            *dst = v;
+            if (live) v = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const uint16_t*>(x) + (int64_t)row * K + k);
+            r.v[c][0] = v;
         } else {
-            float f[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (k < K) {
-                const float4* p = reinterpret_cast<const float4*>(
-                    reinterpret_cast<const float*>(x) + (int64_t)row * K + k);
-                float4 a = p[0], b = p[1];
-                f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w;
-                f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+            u32x4_t v0 = {0u, 0u, 0u, 0u}, v1 = v0;
+            if (live) {
+                const u32x4_t* p = reinterpret_cast<const u32x4_t*>(reinterpret_cast<const float*>(x) + (int64_t)row * K + k);
+                v0 = p[0];
+                v1 = p[1];
             }
+            r.v[c][0] = v0;
+            r.v[c][XMODE == XF32 ? 1 : 0] = v1;
+        }
+    }
+}
+
+template <int XMODE>
+__device__ __forceinline__ void stage_x_store(const XRegs<XMODE>& r, uint16_t* xs, int M, int slab_k, int ldx,
+                                              int plane_elems, int first_chunk, int tid, int nthreads)
+{
+    const int chunks_per_row = slab_k >> 3;
+    const int total = M * chunks_per_row;
+#pragma unroll
+    for (int c = 0; c < kXChunks; c++) {
+        const int idx = first_chunk + tid + c * nthreads;
+        if (idx >= total) continue;
+        const int row = idx / chunks_per_row;
+        const int col = (idx - row * chunks_per_row) << 3;
+        u32x4_t* dst = reinterpret_cast<u32x4_t*>(xs + row * ldx + col);
+        if (XMODE != XF32) {
+            *dst = r.v[c][0];
+        } else {
             Frag16 hi, lo;
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                _Float16 h = (_Float16)f[i];
+                float f = __builtin_bit_cast(float, (uint32_t)r.v[c][i >> 2][i & 3]);
+                _Float16 h = (_Float16)f;
                 hi.h[i] = h;
-                lo.h[i] = (_Float16)(f[i] - (float)h);
+                lo.h[i] = (_Float16)(f - (float)h);
             }
             *dst = hi.u;
             *reinterpret_cast<u32x4_t*>(xs + plane_elems + row * ldx + col) = lo.u;
         }
+    }
+}
+
+// chunks beyond the first kXChunks per thread (large M * slab): plain loop
+template <int XMODE>
+__device__ __forceinline__ void stage_x_rest(uint16_t* xs, const void* x, int M, int K, int k_begin, int slab_k,
+                                             int ldx, int plane_elems, int tid, int nthreads)
+{
+    const int total = M * (slab_k >> 3);
+    for (int first = kXChunks * nthreads; first < total; first += kXChunks * nthreads) {
+        XRegs<XMODE> r;
+        stage_x_load<XMODE>(r, x, M, K, k_begin, slab_k, first, tid, nthreads);
+        stage_x_store<XMODE>(r, xs, M, slab_k, ldx, plane_elems, first, tid, nthreads);
     }
 }
 
@@ -144,7 +188,20 @@ __device__ __forceinline__ void tile_accum(u32x2_t s, const float4_t d[4], float
     }
 }
 
-// Runs a batch of U tiles (tile index i0 + u * nwaves, valid while < limit).
+// The hot region is kept free of branches on purpose: vmcnt retires in order
+// and the compiler can only count outstanding loads along straight-line code;
+// a conditional load forces it to wait for everything (vmcnt(0)) and nothing
+// overlaps.  Tiles past the end of the slab are therefore clamped to the last
+// valid tile (a cache hit) and their scale is forced to zero.
+template <int BITS, int U>
+__device__ __forceinline__ void load_batch(TileRegs<BITS> (&buf)[U], const WeightView& w, int64_t base, int i0,
+                                           int nwaves, int limit, int lane)
+{
+#pragma unroll
+    for (int u = 0; u < U; u++) load_tile<BITS>(buf[u], w, base + min(i0 + u * nwaves, limit - 1), lane);
+}
+
+// Runs a batch of U tiles (tile index i0 + u * nwaves, contributing while < limit).
 template <int BITS, int XMODE, int RMAX, int U>
 __device__ __forceinline__ void compute_batch(const TileRegs<BITS> (&buf)[U], int i0, int nwaves, int limit,
                                               const uint16_t* xbase, int plane_elems, uint32_t magic,
@@ -157,15 +214,12 @@ __device__ __forceinline__ void compute_batch(const TileRegs<BITS> (&buf)[U], in
 #pragma unroll
     for (int u = 0; u < U; u++) {
         const int i = i0 + u * nwaves;
+        const bool valid = i < limit;
         float4_t d[4];
-        u32x2_t sc = {0u, 0u};
-        if (i < limit) {
-            tile_issue<BITS, XMODE>(buf[u], xbase + i * kTileK, plane_elems, magic, d);
-            sc = buf[u].s;
-        } else {
-#pragma unroll
-            for (int j = 0; j < 4; j++) d[j] = (float4_t){0.f, 0.f, 0.f, 0.f};
-        }
+        tile_issue<BITS, XMODE>(buf[u], xbase + min(i, limit - 1) * kTileK, plane_elems, magic, d);
+        u32x2_t sc = buf[u].s;
+        sc[0] = valid ? sc[0] : 0u;
+        sc[1] = valid ? sc[1] : 0u;
         tile_accum<RMAX>(sprev, dprev, acc);
 #pragma unroll
         for (int j = 0; j < 4; j++) dprev[j] = d[j];
@@ -178,7 +232,7 @@ __device__ __forceinline__ void compute_batch(const TileRegs<BITS> (&buf)[U], in
 // of the strip is at most U tiles, all requested before anything else happens
 // (one register set); otherwise two batches are live and ping-pong.
 template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT>
-__global__ __launch_bounds__(512) void gemv_kernel(WeightView w, const void* __restrict__ x, int M, void* __restrict__ y,
+__global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __restrict__ x, int M, void* __restrict__ y,
                             int ydt, int slab_tiles, int ldx)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -188,7 +242,7 @@ __global__ __launch_bounds__(512) void gemv_kernel(WeightView w, const void* __r
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const int lane = tid & 63;
-    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: tile guards become scalar branches
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nwaves = nthreads >> 6;
     const int nt = blockIdx.x;
     const int mrow = min(lane & 15, M - 1);
@@ -203,51 +257,38 @@ __global__ __launch_bounds__(512) void gemv_kernel(WeightView w, const void* __r
 
     if (ONESHOT) {
         TileRegs<BITS> buf[U];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            int i = wv + u * nwaves;
-            if (i < w.KT) load_tile<BITS>(buf[u], w, strip + i, lane);
-        }
-        stage_x<XMODE>(xs, x, M, w.K, 0, w.KT * kTileK, ldx, plane_elems, tid, nthreads);
+        XRegs<XMODE> xr;
+        stage_x_rest<XMODE>(xs, x, M, w.K, 0, w.KT * kTileK, ldx, plane_elems, tid, nthreads);
+        stage_x_load<XMODE>(xr, x, M, w.K, 0, w.KT * kTileK, 0, tid, nthreads);
+        load_batch<BITS, U>(buf, w, strip, wv, nwaves, w.KT, lane);
+        stage_x_store<XMODE>(xr, xs, M, w.KT * kTileK, ldx, plane_elems, 0, tid, nthreads);
         __syncthreads();
         const uint16_t* xbase = xs + mrow * ldx + oct * 8;
         compute_batch<BITS, XMODE, RMAX, U>(buf, wv, nwaves, w.KT, xbase, plane_elems, magic, acc);
     } else {
-    TileRegs<BITS> bufA[U], bufB[U];
+        TileRegs<BITS> bufA[U], bufB[U];
+        for (int slab0 = 0; slab0 < w.KT; slab0 += slab_tiles) {
+            const int st = min(slab_tiles, w.KT - slab0);
+            const int64_t base = strip + slab0;
+            if (slab0 > 0) __syncthreads();          // every wave is done with the previous slab of x
+            // x loads first, then the first weight batch of this slab: the HBM
+            // latency of the weights overlaps the staging and the barrier
+            XRegs<XMODE> xr;
+            stage_x_rest<XMODE>(xs, x, M, w.K, slab0 * kTileK, st * kTileK, ldx, plane_elems, tid, nthreads);
+            stage_x_load<XMODE>(xr, x, M, w.K, slab0 * kTileK, st * kTileK, 0, tid, nthreads);
+            load_batch<BITS, U>(bufA, w, base, wv, nwaves, st, lane);
+            stage_x_store<XMODE>(xr, xs, M, st * kTileK, ldx, plane_elems, 0, tid, nthreads);
+            __syncthreads();
 
-    for (int slab0 = 0; slab0 < w.KT; slab0 += slab_tiles) {
-        const int st = min(slab_tiles, w.KT - slab0);
-        // first batch of this slab goes out before x is staged: HBM latency
-        // overlaps the staging and the barrier
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            int i = wv + u * nwaves;
-            if (i < st) load_tile<BITS>(bufA[u], w, strip + slab0 + i, lane);
-        }
-        if (slab0 > 0) __syncthreads();
-        stage_x<XMODE>(xs, x, M, w.K, slab0 * kTileK, st * kTileK, ldx, plane_elems, tid, nthreads);
-        __syncthreads();
-
-        const uint16_t* xbase = xs + mrow * ldx + oct * 8;
-        for (int i0 = wv; i0 < st; i0 += 2 * stride) {
-            // ---- bufA holds batch i0; fetch batch i0 + stride into bufB
-            const int i1 = i0 + stride;
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                int i = i1 + u * nwaves;
-                if (i < st) load_tile<BITS>(bufB[u], w, strip + slab0 + i, lane);
+            const uint16_t* xbase = xs + mrow * ldx + oct * 8;
+            for (int i0 = wv; i0 < st; i0 += 2 * stride) {
+                // bufA holds batch i0; fetch batch i0 + stride into bufB, and so on
+                load_batch<BITS, U>(bufB, w, base, i0 + stride, nwaves, st, lane);
+                compute_batch<BITS, XMODE, RMAX, U>(bufA, i0, nwaves, st, xbase, plane_elems, magic, acc);
+                load_batch<BITS, U>(bufA, w, base, i0 + 2 * stride, nwaves, st, lane);
+                compute_batch<BITS, XMODE, RMAX, U>(bufB, i0 + stride, nwaves, st, xbase, plane_elems, magic, acc);
             }
-            compute_batch<BITS, XMODE, RMAX, U>(bufA, i0, nwaves, st, xbase, plane_elems, magic, acc);
-            // ---- bufB holds batch i1; fetch batch i1 + stride into bufA
-            const int i2 = i1 + stride;
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                int i = i2 + u * nwaves;
-                if (i < st) load_tile<BITS>(bufA[u], w, strip + slab0 + i, lane);
-            }
-            compute_batch<BITS, XMODE, RMAX, U>(bufB, i1, nwaves, st, xbase, plane_elems, magic, acc);
         }
-    }
     }
 
     // split-K partials -> LDS, summed in wave order by wave 0
@@ -323,12 +364,12 @@ hipError_t launch_u(const WeightView& w, const void* x, int M, void* y, int ydt,
     const bool one_slab = (int64_t)M * (w.KT * kTileK + 8) * 2 * planes <= kLdsBudget;
     const int per_wave = (w.KT + nwaves - 1) / nwaves;
     if (one_slab && unroll == 0) {
+        if (per_wave <= 2) return launch_r<BITS, XMODE, 2, true>(w, x, M, y, ydt, nwaves, st);
         if (per_wave <= 4) return launch_r<BITS, XMODE, 4, true>(w, x, M, y, ydt, nwaves, st);
-        if (per_wave <= 8) return launch_r<BITS, XMODE, 8, true>(w, x, M, y, ydt, nwaves, st);
-        // 16 tiles in flight fit the register file only with one or two batch rows
-        if (per_wave <= 16 && M <= 2) return launch_r<BITS, XMODE, 16, true>(w, x, M, y, ydt, nwaves, st);
+        // (fp32 activations carry two operand planes: 8 tiles in flight would spill)
+        if (per_wave <= 8 && XMODE != XF32) return launch_r<BITS, XMODE, 8, true>(w, x, M, y, ydt, nwaves, st);
     }
-    if (unroll == 4) return launch_r<BITS, XMODE, 4, false>(w, x, M, y, ydt, nwaves, st);
+    if (unroll == 4 && XMODE != XF32) return launch_r<BITS, XMODE, 4, false>(w, x, M, y, ydt, nwaves, st);
     return launch_r<BITS, XMODE, 2, false>(w, x, M, y, ydt, nwaves, st);
 }
 
@@ -344,14 +385,15 @@ void set_gemv_tuning(int waves_per_group, int strips_per_group, int unroll)
 hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
                        int num_cus, hipStream_t st)
 {
-    // enough waves to keep ~8 per CU in flight, never more than there are tiles
+    // Waves per workgroup (= split of a strip's K tiles).  Depends on the weight
+    // shape only, never on M, so that the summation order is the same for every
+    // batch size: enough waves for ~8 per CU, at most 8, never more than tiles.
     int nwaves = g_tune_waves;
     if (nwaves <= 0) {
-        int64_t want = (int64_t)num_cus * 8;
         nwaves = 2;
-        while (nwaves < 8 && (int64_t)w.NT * nwaves < want) nwaves *= 2;
+        while (nwaves < 8 && (int64_t)w.NT * nwaves < (int64_t)num_cus * 8) nwaves *= 2;
     }
-    if (nwaves > 8) nwaves = 8;   // the kernel is compiled for at most 512 threads
+    if (nwaves > 16) nwaves = 16;
     while (nwaves > 1 && nwaves > w.KT) nwaves >>= 1;
     // 0: request a wave's whole share up front when it fits, else stream in batches of 2
     int unroll = g_tune_unroll;

@@ -124,7 +124,7 @@ def test_decode_every_kernel_variant(backend, oracle, bits):
         for M in (1, 2, 4, 9):
             x = _x(M, K, "f16")
             ref = oracle.matmul_f64(q, s, x.float().cpu().numpy())
-            for waves in (1, 2, 4, 8):
+            for waves in (1, 2, 4, 8, 16):
                 for unroll in (0, 2, 4):
                     backend.set_gemv_tuning(waves, 0, unroll)
                     y = _run(backend, qw, x).cpu().numpy()
