@@ -77,6 +77,7 @@ def load_library() -> ctypes.CDLL:
     lib.cybq_weight_info.argtypes = [vp, ctypes.POINTER(ci), ctypes.POINTER(i64), ctypes.POINTER(i64),
                                      ctypes.POINTER(i64)]
     lib.cybq_matmul.argtypes = [vp, vp, vp, ci, i64, vp, ci, vp]
+    lib.cybq_set_prefill_mode.argtypes = [vp, ci]
     lib.cybq_matmul_many.argtypes = [vp, i64, vp, vp, vp, ci, i64, ci, vp]
     lib.cybq_dequant.argtypes = [vp, vp, vp, vp]
     lib.cybq_quantize.argtypes = [vp, ci, vp, i64, i64, vp, vp, vp]
@@ -282,6 +283,14 @@ class Backend:
         if (node.N and node.N != w.N) or (node.K and node.K != w.K) or node.quant != w.quant:
             raise CybqError(-2, "bad shape", f"node {node.w!r} does not match the loaded tensor")
         self.matmul(w, edges[node.x], edges[node.y], M=node.M, stream=stream)
+
+    def set_prefill_mode(self, mode: str) -> None:
+        """'fast' (default): one f16 MFMA per group, weights rounded once to f16;
+        'exact': lossless hi/lo split, two MFMAs per group."""
+        codes = {"fast": 0, "exact": 1}
+        if mode not in codes:
+            raise CybqError(-1, "invalid argument", f"prefill mode {mode!r}")
+        self._check(self._lib.cybq_set_prefill_mode(self._ctx, codes[mode]))
 
     def set_gemv_tuning(self, waves: int = 0, strips: int = 0, unroll: int = 0) -> None:
         self._lib.cybq_debug_set_gemv_tuning(waves, strips, unroll)

@@ -14,6 +14,7 @@
 struct cybq_ctx {
     int device = 0;
     int num_cus = 0;
+    bool prefill_exact = false;
     std::string last_error;
 };
 
@@ -292,7 +293,7 @@ int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype x
     if (M <= 16) {
         e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, st);
     } else if (xdt != CYBQ_F32) {
-        e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, st);
+        e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, st);
     } else {
         // fp32 activations keep full precision through the decode kernel's
         // hi/lo split; prefill in fp32 is walked 16 rows at a time.
@@ -305,6 +306,14 @@ int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype x
         }
     }
     if (e != hipSuccess) return fail_hip(ctx, e, "matmul launch");
+    return CYBQ_OK;
+}
+
+int cybq_set_prefill_mode(cybq_ctx* ctx, cybq_prefill_mode mode)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (mode != CYBQ_PREFILL_FAST && mode != CYBQ_PREFILL_EXACT) return fail(ctx, CYBQ_ERR_INVALID, "unknown prefill mode");
+    ctx->prefill_exact = mode == CYBQ_PREFILL_EXACT;
     return CYBQ_OK;
 }
 

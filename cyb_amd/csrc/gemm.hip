@@ -1,23 +1,47 @@
-// gemm.hip - prefill kernel: Y[M,N] = X[M,K] * W^T for M > 16, LDS-tiled MFMA.
+// gemm.hip - prefill kernel: Y[M,N] = X[M,K] * W^T for M > 16 on MFMA.
 //
-// A workgroup (4 waves) owns a BM x BN output tile and walks K in steps of 128
-// (one native weight tile column = 4 scale groups).  Per step
-//   - the NF = BN/16 native weight tiles are read once from HBM/L2 with 128-bit
-//     loads, unpacked to exact 16-bit integers (bf16 or f16, matching X) and
-//     written to LDS already in MFMA B-operand order;
-//   - the X tile is written to LDS in MFMA A-operand order (each wave-wide
-//     16 B load is one operand: 16 rows x 32 k);
-//   - every wave multiplies its 16*MF rows against all NF column blocks with
-//     v_mfma_f32_16x16x32, one scale group per instruction, and folds the f16
-//     group scale in fp32 into the accumulators.
-// The weight operand is an exact integer and the scale is applied in fp32, so
-// the result differs from the fp32 CPU path only by accumulation order.
+// Workgroup = 4 waves, output tile 256 rows x (16*NF) columns; wave w owns rows
+// [64w, 64w+64) of the tile (4 row blocks of 16) against all NF column blocks.
+//
+//   X  never touches LDS.  An MFMA A operand is 16 rows x 32 k with lane l
+//      holding row l%16, k 8*(l/16)..+8 - exactly a 16 B global load per lane -
+//      and every wave consumes only its own rows, so X streams global ->
+//      registers with a prefetch distance of two scale groups.
+//   W  is shared by the four waves: per K tile (128 k = 4 groups) the NF native
+//      weight tiles are read once with 128-bit loads and dequantised to
+//      w = f32(scale) * q, which is exact in fp32 (11-bit x 4-bit significand).
+//      A 16-bit MFMA operand cannot hold those 15 bits, so w is split without
+//      loss into hi = round16(w) and lo = w - hi (both exactly representable)
+//      and written to LDS as two operands, already in MFMA B-operand order.
+//      LDS is double buffered, one barrier per K tile.
+//   The inner loop is nothing but LDS operand reads and v_mfma_f32_16x16x32
+//      accumulating hi and lo products in fp32: no per-group scaling on the
+//      vector ALU, accumulators stay inside the matrix pipeline until the
+//      epilogue.  The price is two MFMAs per scale group; the gain is that the
+//      weights enter the contraction exactly, so the result differs from the
+//      fp32 CPU path only by accumulation order.  (Q8 weights need 18 bits; lo
+//      is then rounded and the split is exact to 2^-17 relative.)
+//
+// Two modes share this kernel:
+//   EXACT  as described above: two MFMAs per scale group in the type of X.
+//   FAST   one f16 MFMA per scale group.  The weight operand is round_f16(scale * q)
+//          (one rounding, relative error <= 2^-11, about 2e-4 relative L2 on Y -
+//          inside the operator's 1e-3 tolerance); bf16 activations are widened
+//          to f16 in registers after a 2^-4 prescale that is undone in the
+//          epilogue, exact for 2^-10 <= |x| < 2^20.
+//
+// Out-of-range rows / columns / k are clamped to valid addresses inside the hot
+// loop (their results are never stored, padded weights are zero); the loop has
+// no branches, so the compiler can count outstanding loads exactly.
 #include "cybq_device.h"
 #include "cybq_internal.h"
 
 namespace cybq {
 
 namespace {
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ uint16_t f32_to_bf16_rne_g(float f)
 {
@@ -34,26 +58,146 @@ __device__ __forceinline__ void store_out_g(void* y, int ydt, int64_t idx, float
     else reinterpret_cast<uint16_t*>(y)[idx] = f32_to_bf16_rne_g(v);
 }
 
-// XBF = 1: X is bf16 (bf16 MFMA), 0: X is f16 (f16 MFMA)
-template <int BITS, int XBF, int NF, int MF>
-__global__ __launch_bounds__(256) void gemm_kernel(WeightView w, const uint16_t* __restrict__ x, int M,
-                                                   void* __restrict__ y, int ydt)
+constexpr int MF = 4;        // row blocks (of 16) per wave
+constexpr int WAVES = 4;
+constexpr int BM = WAVES * MF * 16;
+
+template <int BITS>
+struct WRegs {               // one native weight tile as loaded by one lane, and its 4 group scales
+    u32x4_t q[BITS == 4 ? 1 : 2];
+    u32x2_t s;
+};
+
+template <int BITS>
+__device__ __forceinline__ void load_wtile(WRegs<BITS>& r, const u32x4_t* qp, const u32x2_t* sp, int64_t tile,
+                                           int lane)
 {
-    constexpr int WAVES = 4;
-    constexpr int MFRAGS = WAVES * MF;            // m-fragments per workgroup
+    if (BITS == 4) {
+        r.q[0] = qp[tile * 64 + lane];
+    } else {
+        r.q[0] = qp[tile * 128 + lane];
+        r.q[BITS == 4 ? 0 : 1] = qp[tile * 128 + 64 + lane];
+    }
+    r.s = sp[tile * 16 + (lane & 15)];
+}
+
+// (w0, w1) fp32 -> packed 16-bit hi pair and lo pair with hi + lo == w
+template <int XBF>
+__device__ __forceinline__ void split_pair(float w0, float w1, uint32_t& hi, uint32_t& lo)
+{
+    if (XBF) {
+        bf16x2_t h = __builtin_convertvector((float2_t){w0, w1}, bf16x2_t);
+        hi = __builtin_bit_cast(uint32_t, h);
+        float h0 = __builtin_bit_cast(float, hi << 16);
+        float h1 = __builtin_bit_cast(float, hi & 0xffff0000u);
+        bf16x2_t l = __builtin_convertvector((float2_t){w0 - h0, w1 - h1}, bf16x2_t);
+        lo = __builtin_bit_cast(uint32_t, l);
+    } else {
+        half2_t h = {(_Float16)w0, (_Float16)w1};
+        hi = as_u32(h);
+        half2_t l = {(_Float16)(w0 - (float)h.x), (_Float16)(w1 - (float)h.y)};
+        lo = as_u32(l);
+    }
+}
+
+// group j of a native tile -> B operand(s) in LDS: hi and lo (EXACT) or one rounded f16 operand
+template <int BITS, int XBF, bool EXACT>
+__device__ __forceinline__ void dequant_group_to_lds(const WRegs<BITS>& r, int j, uint32_t magic, u32x4_t* dst,
+                                                     int lane)
+{
+    uint32_t bw[4];
+    if (BITS == 4) unpack_q4_f16(r.q[0][j], magic, bw);
+    else unpack_q8_f16(r.q[(BITS == 4) ? 0 : (j >> 1)][(j & 1) * 2], r.q[(BITS == 4) ? 0 : (j >> 1)][(j & 1) * 2 + 1], bw);
+    const uint32_t sb = (j & 1) ? (r.s[j >> 1] >> 16) : (r.s[j >> 1] & 0xffffu);
+    if (!EXACT) {
+        const _Float16 sh = __builtin_bit_cast(_Float16, (uint16_t)sb);
+        const half2_t s2 = {sh, sh};
+        uint32_t o[4];
+#pragma unroll
+        for (int p = 0; p < 4; p++) o[p] = as_u32(as_h2(bw[p]) * s2);     // round_f16(scale * q)
+        dst[j * 64 + lane] = (u32x4_t){o[0], o[1], o[2], o[3]};
+        return;
+    }
+    const float sc = f16_bits_to_f32(sb);
+    uint32_t hi[4], lo[4];
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        half2_t qv = as_h2(bw[p]);
+        split_pair<XBF>(sc * (float)qv.x, sc * (float)qv.y, hi[p], lo[p]);
+    }
+    dst[(j * 2 + 0) * 64 + lane] = (u32x4_t){hi[0], hi[1], hi[2], hi[3]};
+    dst[(j * 2 + 1) * 64 + lane] = (u32x4_t){lo[0], lo[1], lo[2], lo[3]};
+}
+
+template <int XBF>
+__device__ __forceinline__ float4_t mma(const Frag16& a, const Frag16& b, float4_t c)
+{
+    if (XBF) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, c, 0, 0, 0);
+}
+
+// bf16 A operand -> f16 A operand, prescaled by 2^-4
+__device__ __forceinline__ Frag16 bf16_to_f16_frag(const Frag16& a)
+{
+    Frag16 o;
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        float f0 = __builtin_bit_cast(float, a.u[p] << 16);
+        float f1 = __builtin_bit_cast(float, a.u[p] & 0xffff0000u);
+        half2_t h = {(_Float16)(f0 * 0.0625f), (_Float16)(f1 * 0.0625f)};
+        o.u[p] = as_u32(h);
+    }
+    return o;
+}
+
+// XBF = 1: X is bf16, 0: X is f16.  EXACT: see the header comment.
+template <int BITS, int XBF, int NF, bool EXACT>
+__global__ __launch_bounds__(256) void gemm_kernel(WeightView w, const uint16_t* __restrict__ x, int M,
+                                                   void* __restrict__ y, int ydt, int n_tiles, int m_tiles)
+{
+    // Workgroups are handed to the 8 XCDs round-robin (id % 8) and every XCD has
+    // its own L2.  Give each XCD a contiguous run of tiles in row-block-major
+    // order, so the workgroups sharing an L2 read the same rows of X and X is
+    // fetched into every L2 once instead of once per column tile.
+    const int per_xcd = (int)gridDim.x >> 3;
+    const int item = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+    if (item >= n_tiles * m_tiles) return;
+    const int tile_m = item / n_tiles;
+    const int tile_n = item - tile_m * n_tiles;
+    constexpr int WT = (NF + WAVES - 1) / WAVES;      // weight tiles a wave stages per K tile
+    constexpr int OPS = EXACT ? 2 : 1;                // B operands per scale group
+    constexpr int TILE16 = 4 * OPS * 64;              // u32x4 per column block per buffer
+    constexpr int MMA_BF = EXACT ? XBF : 0;           // FAST always multiplies in f16
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    u32x4_t* xs = reinterpret_cast<u32x4_t*>(smem);                    // [MFRAGS][4][64]
-    u32x4_t* ws = xs + MFRAGS * 4 * 64;                                // [NF][4][64]
+    u32x4_t* ws = reinterpret_cast<u32x4_t*>(smem);   // [2][NF][4][2][64]
     const uint32_t magic = q4_magic_vgpr();
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wv = tid >> 6;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row16 = lane & 15;
     const int oct = lane >> 4;
-    const int nt0 = blockIdx.x * NF;
-    const int m0 = blockIdx.y * (MFRAGS * 16);
-    const int K = w.K;
+    const int nt0 = tile_n * NF;
+    const int m0 = tile_m * BM + wv * (MF * 16);
+    const int K = w.K, KT = w.KT;
+    const int kmax = K - 8 - oct * 8;                 // largest valid per-lane k offset
+
+    const u32x4_t* qp = reinterpret_cast<const u32x4_t*>(w.q);
+    const u32x2_t* sp = reinterpret_cast<const u32x2_t*>(w.s);
+
+    // per-lane row pointers of this wave's four row blocks (rows clamped to M-1)
+    const uint16_t* xrow[MF];
+#pragma unroll
+    for (int i = 0; i < MF; i++) xrow[i] = x + (int64_t)min(m0 + i * 16 + row16, M - 1) * K + oct * 8;
+
+    // the weight tiles this wave stages: column block f = wv + WAVES*t (clamped)
+    int64_t wtile[WT];
+    int wf[WT];
+#pragma unroll
+    for (int t = 0; t < WT; t++) {
+        wf[t] = min(wv + WAVES * t, NF - 1);
+        wtile[t] = (int64_t)min(nt0 + wf[t], w.NT - 1) * KT;
+    }
 
     float4_t acc[MF][NF];
 #pragma unroll
@@ -61,97 +205,92 @@ __global__ __launch_bounds__(256) void gemm_kernel(WeightView w, const uint16_t*
 #pragma unroll
         for (int f = 0; f < NF; f++) acc[i][f] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-    const float4_t zero = {0.f, 0.f, 0.f, 0.f};
-    const u32x4_t* qp = reinterpret_cast<const u32x4_t*>(w.q);
-    const u32x2_t* sp = reinterpret_cast<const u32x2_t*>(w.s);
+    // ---- prologue: first two groups of X, W tile 0 -> LDS buffer 0
+    Frag16 xa[2][MF];
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int i = 0; i < MF; i++)
+            xa[j][i].u = *reinterpret_cast<const u32x4_t*>(xrow[i] + min(j * 32, kmax));
+    WRegs<BITS> wr[WT];        // packed weights of the K tile that is dequantised next
+    {
+        WRegs<BITS> w0[WT];
+#pragma unroll
+        for (int t = 0; t < WT; t++) load_wtile<BITS>(w0[t], qp, sp, wtile[t], lane);
+#pragma unroll
+        for (int t = 0; t < WT; t++) load_wtile<BITS>(wr[t], qp, sp, wtile[t] + min(1, KT - 1), lane);
+#pragma unroll
+        for (int t = 0; t < WT; t++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                dequant_group_to_lds<BITS, XBF, EXACT>(w0[t], j, magic, ws + wf[t] * TILE16, lane);
+    }
+    __syncthreads();
 
-    for (int kt = 0; kt < w.KT; kt++) {
-        __syncthreads();
-        // ---- X tile -> LDS, A-operand order
-        for (int f = wv; f < MFRAGS * 4; f += WAVES) {
-            int i = f >> 2, j = f & 3;
-            int row = m0 + i * 16 + row16;
-            int k = kt * kTileK + j * 32 + oct * 8;
-            u32x4_t v = {0u, 0u, 0u, 0u};
-            if (row < M && k < K) v = *reinterpret_cast<const u32x4_t*>(x + (int64_t)row * K + k);
-            xs[f * 64 + lane] = v;
-        }
-        // ---- W tiles -> exact 16-bit integers -> LDS, B-operand order
-        for (int f = wv; f < NF; f += WAVES) {
-            int nt = nt0 + f;
-            u32x4_t q0 = {0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u}, q1 = q0;
-            if (BITS == 8) q0 = q1 = (u32x4_t){0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};
-            if (nt < w.NT) {
-                int64_t tile = (int64_t)nt * w.KT + kt;
-                if (BITS == 4) q0 = qp[tile * 64 + lane];
-                else { q0 = qp[tile * 128 + lane]; q1 = qp[tile * 128 + 64 + lane]; }
-            }
+    for (int kt = 0; kt < KT; kt++) {
+        const u32x4_t* wcur = ws + (kt & 1) * (NF * TILE16);
+        u32x4_t* wnxt = ws + ((kt + 1) & 1) * (NF * TILE16);
+        // wr holds K tile kt+1 (requested one iteration ago, so the HBM latency is
+        // behind us); request tile kt+2 now.  Past the end the index is clamped:
+        // the tile is staged again but never read.
+        const int ktn = min(kt + 2, KT - 1);
+        WRegs<BITS> wn[WT];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                uint32_t bw[4];
-                if (BITS == 4) unpack_q4_f16(q0[j], magic, bw);
-                else if (j < 2) unpack_q8_f16(q0[(j & 1) * 2], q0[(j & 1) * 2 + 1], bw);
-                else unpack_q8_f16(q1[(j & 1) * 2], q1[(j & 1) * 2 + 1], bw);
-                if (XBF) f16frag_to_bf16frag(bw);
-                ws[(f * 4 + j) * 64 + lane] = (u32x4_t){bw[0], bw[1], bw[2], bw[3]};
-            }
-        }
-        // ---- group scales of this step for every column block (registers)
-        float sc[NF][4];
-#pragma unroll
-        for (int f = 0; f < NF; f++) {
-            int nt = nt0 + f;
-            u32x2_t sv = {0u, 0u};
-            if (nt < w.NT) sv = sp[((int64_t)nt * w.KT + kt) * 16 + row16];
-            sc[f][0] = f16_bits_to_f32(sv[0] & 0xffffu);
-            sc[f][1] = f16_bits_to_f32(sv[0] >> 16);
-            sc[f][2] = f16_bits_to_f32(sv[1] & 0xffffu);
-            sc[f][3] = f16_bits_to_f32(sv[1] >> 16);
-        }
-        __syncthreads();
-        // ---- multiply
+        for (int t = 0; t < WT; t++) load_wtile<BITS>(wn[t], qp, sp, wtile[t] + ktn, lane);
+
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             Frag16 a[MF];
 #pragma unroll
-            for (int i = 0; i < MF; i++) a[i].u = xs[((wv * MF + i) * 4 + j) * 64 + lane];
+            for (int i = 0; i < MF; i++) a[i] = (!EXACT && XBF) ? bf16_to_f16_frag(xa[j & 1][i]) : xa[j & 1][i];
 #pragma unroll
             for (int f = 0; f < NF; f++) {
-                Frag16 b;
-                b.u = ws[(f * 4 + j) * 64 + lane];
-                const float s = sc[f][j];
+                Frag16 bh, bl;
+                bh.u = wcur[f * TILE16 + (j * OPS + 0) * 64 + lane];
+                if (EXACT) bl.u = wcur[f * TILE16 + (j * OPS + OPS - 1) * 64 + lane];
 #pragma unroll
-                for (int i = 0; i < MF; i++) {
-                    float4_t d;
-                    if (XBF) d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].b, b.b, zero, 0, 0, 0);
-                    else d = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i].h, b.h, zero, 0, 0, 0);
+                for (int i = 0; i < MF; i++) acc[i][f] = mma<MMA_BF>(a[i], bh, acc[i][f]);
+                if (EXACT) {
 #pragma unroll
-                    for (int r = 0; r < 4; r++) acc[i][f][r] = __builtin_fmaf(s, d[r], acc[i][f][r]);
+                    for (int i = 0; i < MF; i++) acc[i][f] = mma<MMA_BF>(a[i], bl, acc[i][f]);
                 }
             }
+            // group j is consumed: its registers take the X operands two groups ahead
+            const int kn = min(kt * kTileK + (j + 2) * 32, kmax);
+#pragma unroll
+            for (int i = 0; i < MF; i++) xa[j & 1][i].u = *reinterpret_cast<const u32x4_t*>(xrow[i] + kn);
+            // a quarter of the next tile's dequantisation rides along with every group
+            // (a wave whose second tile index is clamped rewrites a neighbour's
+            // block with identical values: no branch in the hot loop)
+#pragma unroll
+            for (int t = 0; t < WT; t++)
+                dequant_group_to_lds<BITS, XBF, EXACT>(wr[t], j, magic, wnxt + wf[t] * TILE16, lane);
         }
+#pragma unroll
+        for (int t = 0; t < WT; t++) wr[t] = wn[t];
+        __syncthreads();
     }
 
     // ---- epilogue
+    const float out_scale = (!EXACT && XBF) ? 16.0f : 1.0f;
 #pragma unroll
     for (int i = 0; i < MF; i++)
 #pragma unroll
         for (int f = 0; f < NF; f++) {
-            int n = (nt0 + f) * 16 + row16;
+            const int n = (nt0 + f) * 16 + row16;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                int m = m0 + (wv * MF + i) * 16 + oct * 4 + r;
-                if (m < M && n < w.N) store_out_g(y, ydt, (int64_t)m * w.N + n, acc[i][f][r]);
+                const int m = m0 + i * 16 + oct * 4 + r;
+                if (m < M && n < w.N) store_out_g(y, ydt, (int64_t)m * w.N + n, acc[i][f][r] * out_scale);
             }
         }
 }
 
-template <int BITS, int XBF, int NF, int MF>
+template <int BITS, int XBF, int NF, bool EXACT>
 hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, hipStream_t st)
 {
-    constexpr int BM = 4 * MF * 16;
-    size_t lds = (size_t)(4 * MF * 4 * 64 + NF * 4 * 64) * 16;
-    auto kern = gemm_kernel<BITS, XBF, NF, MF>;
+    const size_t lds = (size_t)2 * NF * (4 * (EXACT ? 2 : 1) * 64) * 16;     // 56 .. 128 KB
+    auto kern = gemm_kernel<BITS, XBF, NF, EXACT>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -159,33 +298,39 @@ hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt,
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    dim3 grid((unsigned)((w.NT + NF - 1) / NF), (unsigned)((M + BM - 1) / BM));
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, w, reinterpret_cast<const uint16_t*>(x), M, y, ydt);
+    const int n_tiles = (w.NT + NF - 1) / NF, m_tiles = (M + BM - 1) / BM;
+    const unsigned groups = (unsigned)(((int64_t)n_tiles * m_tiles + 7) / 8 * 8);
+    hipLaunchKernelGGL(kern, dim3(groups), dim3(256), lds, st, w, reinterpret_cast<const uint16_t*>(x), M, y, ydt,
+                       n_tiles, m_tiles);
     return hipGetLastError();
 }
 
 template <int BITS, int XBF>
-hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt, hipStream_t st)
+hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt, bool exact, hipStream_t st)
 {
     // 7 column blocks (BN = 112) tile N = 14336 = 128 * 112 exactly: with M = 512
     // that is 256 workgroups, one per CU; 8 column blocks otherwise
-    if (w.NT % 7 == 0) return launch_t<BITS, XBF, 7, 4>(w, x, M, y, ydt, st);
-    return launch_t<BITS, XBF, 8, 4>(w, x, M, y, ydt, st);
+    if (w.NT % 7 == 0) {
+        if (exact) return launch_t<BITS, XBF, 7, true>(w, x, M, y, ydt, st);
+        return launch_t<BITS, XBF, 7, false>(w, x, M, y, ydt, st);
+    }
+    if (exact) return launch_t<BITS, XBF, 8, true>(w, x, M, y, ydt, st);
+    return launch_t<BITS, XBF, 8, false>(w, x, M, y, ydt, st);
 }
 
 }  // namespace
 
 hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
-                       int num_cus, hipStream_t st)
+                       int num_cus, bool exact, hipStream_t st)
 {
     (void)num_cus;
-    if (xdt == kF32) return hipErrorNotSupported;   // api.hip routes f32 prefill elsewhere
+    if (xdt == kF32) return hipErrorNotSupported;   // api.hip walks fp32 prefill through the decode kernel
     if (w.bits == 4) {
-        if (xdt == kBF16) return launch_nf<4, 1>(w, x, M, y, ydt, st);
-        return launch_nf<4, 0>(w, x, M, y, ydt, st);
+        if (xdt == kBF16) return launch_nf<4, 1>(w, x, M, y, ydt, exact, st);
+        return launch_nf<4, 0>(w, x, M, y, ydt, exact, st);
     }
-    if (xdt == kBF16) return launch_nf<8, 1>(w, x, M, y, ydt, st);
-    return launch_nf<8, 0>(w, x, M, y, ydt, st);
+    if (xdt == kBF16) return launch_nf<8, 1>(w, x, M, y, ydt, exact, st);
+    return launch_nf<8, 0>(w, x, M, y, ydt, exact, st);
 }
 
 }  // namespace cybq

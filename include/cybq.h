@@ -74,6 +74,17 @@ typedef enum cybq_layout { CYBQ_LAYOUT_PLANAR = 0, CYBQ_LAYOUT_BLOCK_AOS = 1 } c
 
 typedef enum cybq_dtype { CYBQ_F32 = 0, CYBQ_F16 = 1, CYBQ_BF16 = 2 } cybq_dtype;
 
+/* How the prefill kernel (M > 16) feeds the matrix cores.  Both stay inside the
+ * operator's 1e-3 relative-L2 tolerance; the decode kernel (M <= 16) is always exact.
+ *   FAST   (default) one f16 MFMA per 32-group; the weight operand is
+ *          round_f16(scale * q), relative error <= 2^-11 per weight (about 2e-4
+ *          relative L2 on y).  bf16 activations are widened to f16 after a 2^-4
+ *          prescale (undone on output): |x| must stay below 2^20.
+ *   EXACT  two MFMAs per 32-group in the activation type; scale * q is split
+ *          without loss into a high and a low 16-bit operand, so y differs from
+ *          the fp32 CPU path only by accumulation order.  Half the throughput. */
+typedef enum cybq_prefill_mode { CYBQ_PREFILL_FAST = 0, CYBQ_PREFILL_EXACT = 1 } cybq_prefill_mode;
+
 /* ---- context ---------------------------------------------------------- */
 
 /* Replaces: backend construction when the runtime is spawned
@@ -117,6 +128,11 @@ int cybq_weight_info(const cybq_weight* w, int* quant, int64_t* N, int64_t* K,
  *   LDS-tiled MFMA prefill kernel; there is no other path. */
 int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt,
                 int64_t M, void* y, cybq_dtype ydt, void* stream);
+
+/* Replaces: a backend configuration knob (the reference picks a backend per run:
+ * `--backend honeycrisp|wgpu|cpu`, shell/src/worlds/models/mod.rs:113-115); here
+ * it selects the numeric mode of the prefill kernel for this context. */
+int cybq_set_prefill_mode(cybq_ctx* ctx, cybq_prefill_mode mode);
 
 /* Replaces: the executor's walk over the quantised-matmul nodes of one decode
  * step (7 linears per layer x layers + LM head - decide/pipeline.md:51): `count`
