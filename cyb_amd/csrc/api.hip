@@ -15,6 +15,8 @@ struct cybq_ctx {
     int device = 0;
     int num_cus = 0;
     bool prefill_exact = false;
+    void* workspace = nullptr;          // scratch for the prefill path, allocated once at init
+    size_t workspace_bytes = 0;
     std::string last_error;
 };
 
@@ -144,11 +146,24 @@ int cybq_init(int device, cybq_ctx** out)
     if (!ctx) return CYBQ_ERR_NOMEM;
     ctx->device = device;
     ctx->num_cus = prop.multiProcessorCount;
+    // 64 MiB of scratch (f16 copy of up to 2048 x 16384 activations); without it the
+    // prefill kernel converts in registers, so a failed allocation is not an error
+    ctx->workspace_bytes = (size_t)64 << 20;
+    if (hipMalloc(&ctx->workspace, ctx->workspace_bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        ctx->workspace = nullptr;
+        ctx->workspace_bytes = 0;
+    }
     *out = ctx;
     return CYBQ_OK;
 }
 
-void cybq_destroy(cybq_ctx* ctx) { delete ctx; }
+void cybq_destroy(cybq_ctx* ctx)
+{
+    if (!ctx) return;
+    if (ctx->workspace && hipSetDevice(ctx->device) == hipSuccess) (void)hipFree(ctx->workspace);
+    delete ctx;
+}
 
 int cybq_weight_upload(cybq_ctx* ctx, cybq_quant quant, cybq_layout layout, int64_t N, int64_t K,
                        const void* q, const void* scales, cybq_weight** out)
@@ -293,7 +308,7 @@ int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype x
     if (M <= 16) {
         e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, st);
     } else if (xdt != CYBQ_F32) {
-        e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, st);
+        e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, ctx->workspace, ctx->workspace_bytes, st);
     } else {
         // fp32 activations keep full precision through the decode kernel's
         // hi/lo split; prefill in fp32 is walked 16 rows at a time.

@@ -6,7 +6,7 @@
 //   X  never touches LDS.  An MFMA A operand is 16 rows x 32 k with lane l
 //      holding row l%16, k 8*(l/16)..+8 - exactly a 16 B global load per lane -
 //      and every wave consumes only its own rows, so X streams global ->
-//      registers with a prefetch distance of two scale groups.
+//      registers, one K tile (four scale groups) ahead of its use.
 //   W  is shared by the four waves: per K tile (128 k = 4 groups) the NF native
 //      weight tiles are read once with 128-bit loads and dequantised to
 //      w = f32(scale) * q, which is exact in fp32 (11-bit x 4-bit significand).
@@ -153,7 +153,7 @@ __device__ __forceinline__ Frag16 bf16_to_f16_frag(const Frag16& a)
 // XBF = 1: X is bf16, 0: X is f16.  EXACT: see the header comment.
 template <int BITS, int XBF, int NF, bool EXACT>
 __global__ __launch_bounds__(256) void gemm_kernel(WeightView w, const uint16_t* __restrict__ x, int M,
-                                                   void* __restrict__ y, int ydt, int n_tiles, int m_tiles)
+                                                   void* __restrict__ y, int ydt, int n_tiles, int m_tiles, float out_scale)
 {
     // Workgroups are handed to the 8 XCDs round-robin (id % 8) and every XCD has
     // its own L2.  Give each XCD a contiguous run of tiles in row-block-major
@@ -205,10 +205,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(WeightView w, const uint16_t*
 #pragma unroll
         for (int f = 0; f < NF; f++) acc[i][f] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-    // ---- prologue: first two groups of X, W tile 0 -> LDS buffer 0
-    Frag16 xa[2][MF];
+    // ---- prologue: first K tile of X, W tile 0 -> LDS buffer 0
+    Frag16 xa[4][MF];          // one K tile (four scale groups) of X in flight
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int j = 0; j < 4; j++)
 #pragma unroll
         for (int i = 0; i < MF; i++)
             xa[j][i].u = *reinterpret_cast<const u32x4_t*>(xrow[i] + min(j * 32, kmax));
@@ -242,23 +242,28 @@ __global__ __launch_bounds__(256) void gemm_kernel(WeightView w, const uint16_t*
         for (int j = 0; j < 4; j++) {
             Frag16 a[MF];
 #pragma unroll
-            for (int i = 0; i < MF; i++) a[i] = (!EXACT && XBF) ? bf16_to_f16_frag(xa[j & 1][i]) : xa[j & 1][i];
+            for (int i = 0; i < MF; i++) a[i] = (!EXACT && XBF) ? bf16_to_f16_frag(xa[j][i]) : xa[j][i];
 #pragma unroll
             for (int f = 0; f < NF; f++) {
-                Frag16 bh, bl;
-                bh.u = wcur[f * TILE16 + (j * OPS + 0) * 64 + lane];
-                if (EXACT) bl.u = wcur[f * TILE16 + (j * OPS + OPS - 1) * 64 + lane];
+                Frag16 b[OPS];
 #pragma unroll
-                for (int i = 0; i < MF; i++) acc[i][f] = mma<MMA_BF>(a[i], bh, acc[i][f]);
-                if (EXACT) {
+                for (int o = 0; o < OPS; o++) b[o].u = wcur[f * TILE16 + (j * OPS + o) * 64 + lane];
 #pragma unroll
-                    for (int i = 0; i < MF; i++) acc[i][f] = mma<MMA_BF>(a[i], bl, acc[i][f]);
+                for (int o = 0; o < OPS; o++)
+#pragma unroll
+                    for (int i = 0; i < MF; i++) acc[i][f] = mma<MMA_BF>(a[i], b[o], acc[i][f]);
+            }
+            // After an odd group its pair of operand sets is free: refill both with
+            // the same groups of the next K tile.  The two loads of a row hit the
+            // two halves of one 128 B line back to back.
+            if (j & 1) {
+#pragma unroll
+                for (int jj = j - 1; jj <= j; jj++) {
+                    const int kn = min((kt + 1) * kTileK + jj * 32, kmax);
+#pragma unroll
+                    for (int i = 0; i < MF; i++) xa[jj][i].u = *reinterpret_cast<const u32x4_t*>(xrow[i] + kn);
                 }
             }
-            // group j is consumed: its registers take the X operands two groups ahead
-            const int kn = min(kt * kTileK + (j + 2) * 32, kmax);
-#pragma unroll
-            for (int i = 0; i < MF; i++) xa[j & 1][i].u = *reinterpret_cast<const u32x4_t*>(xrow[i] + kn);
             // a quarter of the next tile's dequantisation rides along with every group
             // (a wave whose second tile index is clamped rewrites a neighbour's
             // block with identical values: no branch in the hot loop)
@@ -272,7 +277,6 @@ __global__ __launch_bounds__(256) void gemm_kernel(WeightView w, const uint16_t*
     }
 
     // ---- epilogue
-    const float out_scale = (!EXACT && XBF) ? 16.0f : 1.0f;
 #pragma unroll
     for (int i = 0; i < MF; i++)
 #pragma unroll
@@ -287,7 +291,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(WeightView w, const uint16_t*
 }
 
 template <int BITS, int XBF, int NF, bool EXACT>
-hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, hipStream_t st)
+hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, hipStream_t st)
 {
     const size_t lds = (size_t)2 * NF * (4 * (EXACT ? 2 : 1) * 64) * 16;     // 56 .. 128 KB
     auto kern = gemm_kernel<BITS, XBF, NF, EXACT>;
@@ -301,36 +305,63 @@ hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt,
     const int n_tiles = (w.NT + NF - 1) / NF, m_tiles = (M + BM - 1) / BM;
     const unsigned groups = (unsigned)(((int64_t)n_tiles * m_tiles + 7) / 8 * 8);
     hipLaunchKernelGGL(kern, dim3(groups), dim3(256), lds, st, w, reinterpret_cast<const uint16_t*>(x), M, y, ydt,
-                       n_tiles, m_tiles);
+                       n_tiles, m_tiles, out_scale);
     return hipGetLastError();
 }
 
 template <int BITS, int XBF>
-hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt, bool exact, hipStream_t st)
+hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt, bool exact, float out_scale,
+                     hipStream_t st)
 {
     // 7 column blocks (BN = 112) tile N = 14336 = 128 * 112 exactly: with M = 512
     // that is 256 workgroups, one per CU; 8 column blocks otherwise
     if (w.NT % 7 == 0) {
-        if (exact) return launch_t<BITS, XBF, 7, true>(w, x, M, y, ydt, st);
-        return launch_t<BITS, XBF, 7, false>(w, x, M, y, ydt, st);
+        if (exact) return launch_t<BITS, XBF, 7, true>(w, x, M, y, ydt, out_scale, st);
+        return launch_t<BITS, XBF, 7, false>(w, x, M, y, ydt, out_scale, st);
     }
-    if (exact) return launch_t<BITS, XBF, 8, true>(w, x, M, y, ydt, st);
-    return launch_t<BITS, XBF, 8, false>(w, x, M, y, ydt, st);
+    if (exact) return launch_t<BITS, XBF, 8, true>(w, x, M, y, ydt, out_scale, st);
+    return launch_t<BITS, XBF, 8, false>(w, x, M, y, ydt, out_scale, st);
+}
+
+// bf16 [n] -> f16 [n] scaled by 2^-4 (exact for 2^-10 <= |x| < 2^20); n % 8 == 0
+__global__ void widen_bf16_kernel(const u32x4_t* __restrict__ src, u32x4_t* __restrict__ dst, int64_t n8)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n8) return;
+    Frag16 a;
+    a.u = src[i];
+    dst[i] = bf16_to_f16_frag(a).u;
 }
 
 }  // namespace
 
 hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
-                       int num_cus, bool exact, hipStream_t st)
+                       int num_cus, bool exact, void* workspace, size_t workspace_bytes, hipStream_t st)
 {
     (void)num_cus;
     if (xdt == kF32) return hipErrorNotSupported;   // api.hip walks fp32 prefill through the decode kernel
-    if (w.bits == 4) {
-        if (xdt == kBF16) return launch_nf<4, 1>(w, x, M, y, ydt, exact, st);
-        return launch_nf<4, 0>(w, x, M, y, ydt, exact, st);
+    float out_scale = 1.0f;
+    if (!exact && xdt == kBF16) {
+        out_scale = 16.0f;                          // undoes the 2^-4 prescale of the f16 activations
+        const size_t need = (size_t)M * w.K * 2;
+        if (workspace && need <= workspace_bytes) {
+            // Widen X once instead of in every workgroup (each of the N/112 column
+            // tiles would redo it): one elementwise pass, then the f16 kernel.
+            const int64_t n8 = (int64_t)M * w.K / 8;
+            hipLaunchKernelGGL(widen_bf16_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, st,
+                               reinterpret_cast<const u32x4_t*>(x), reinterpret_cast<u32x4_t*>(workspace), n8);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return e;
+            x = workspace;
+            xdt = kF16;
+        }
     }
-    if (xdt == kBF16) return launch_nf<8, 1>(w, x, M, y, ydt, exact, st);
-    return launch_nf<8, 0>(w, x, M, y, ydt, exact, st);
+    if (w.bits == 4) {
+        if (xdt == kBF16) return launch_nf<4, 1>(w, x, M, y, ydt, exact, out_scale, st);
+        return launch_nf<4, 0>(w, x, M, y, ydt, exact, out_scale, st);
+    }
+    if (xdt == kBF16) return launch_nf<8, 1>(w, x, M, y, ydt, exact, out_scale, st);
+    return launch_nf<8, 0>(w, x, M, y, ydt, exact, out_scale, st);
 }
 
 }  // namespace cybq
