@@ -26,6 +26,10 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 MALL_BYTES = 256 << 20
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain
+# 256 MiB copy: FETCH x 1.9997, WRITE x 1.0000); profiles/decode_gemv_q4_4096x14336_m1.md
+TRAFFIC_DECODE_BYTES = 33_275_500
+TRAFFIC_PREFILL_M512_BYTES = 112_865_000
 
 
 def log(*a):
@@ -76,6 +80,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the prefill / sweep extras")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="no timing: a plain 256 MiB device copy (calibration), then the decode and prefill "
+                         "kernels, for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the op shards by rows of W; "
@@ -123,6 +130,20 @@ def main():
     def plan_of(n):
         return be.plan_many([ws[i % copies] for i in range(n)], [x] * n, [ys[i % 2] for i in range(n)])
 
+    if args.traffic_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)                      # plain copy kernel of known size: 256 MiB read, 256 MiB written
+        be.matmul_many(plan_of(100), M, stream)
+        xp = torch.from_numpy(synth.activations(4, 512, K)).to(dev).to(torch.bfloat16)
+        yp = torch.empty((512, N), dtype=torch.float32, device=dev)
+        for i in range(10):
+            be.matmul(ws[i % copies], xp, yp, stream=stream)
+        torch.cuda.synchronize()
+        log("traffic probe done")
+        return
+
     if args.warmup > 0:
         be.matmul_many(plan_of(args.warmup), M, stream)
     plan = plan_of(args.steps)
@@ -154,7 +175,7 @@ def main():
         "config": {"workload": "Q4 decode GEMV, K=4096 -> N=14336, M=1, x f16, y f32 (BASELINE configs[1])",
                    "weight_copies_rotated": int(copies), "algorithmic_bytes_per_step": int(alg_bytes)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_DECODE_BYTES},
         "parity_rel_l2": rel_l2,
         "single_launch_us": round(lat[len(lat) // 2], 2),
     }
@@ -179,7 +200,7 @@ def main():
             "workload": "Q4 prefill GEMM, M=512, K=4096 -> N=14336, X bf16, Y f32 (BASELINE configs[3])",
             "us": round(elp * 1e6, 1), "tflops": round(tfl, 1), "parity_rel_l2": relp,
             "roofline": {"bound": "mfma", "achieved": round(tfl, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
-                         "unit": "TFLOP/s", "frac": round(tfl / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}}
+                         "unit": "TFLOP/s", "frac": round(tfl / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": TRAFFIC_PREFILL_M512_BYTES}}
         log(f"prefill GEMM M=512: {elp * 1e6:.1f} us, {tfl:.1f} TFLOP/s, rel_l2 {relp:.2e}")
         # batch sweep of the decode kernel on the same shape
         sweep = {}
