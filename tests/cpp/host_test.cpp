@@ -1,0 +1,94 @@
+// host_test.cpp - exercises the C++ host layer (include/cybq.hpp, cybq_container.hpp)
+// end to end: map a .model container, load its tensors, run graph nodes, compare
+// with expected outputs written by the Python test (which gets them from the oracle).
+//
+//   host_test --parse FILE                     no GPU: print the tensor index
+//   host_test --run FILE X.bin Y.bin M [exact] GPU: X is f16 [M,K] (K of the first tensor),
+//                                              Y is f64 [tensors][M,N]; prints rel-L2 per tensor
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <vector>
+
+#include "cybq.hpp"
+#include "cybq_container.hpp"
+
+static std::vector<char> slurp(const char* path)
+{
+    std::ifstream f(path, std::ios::binary);
+    return std::vector<char>((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+}
+
+int main(int argc, char** argv)
+{
+    if (argc < 3) { std::fprintf(stderr, "usage: host_test --parse|--run FILE ...\n"); return 2; }
+    cybq::Container c;
+    cybq::Status s = c.open(argv[2]);
+    if (!s) { std::printf("ERROR %d %s\n", s.code, s.text.c_str()); return 1; }
+    if (!std::strcmp(argv[1], "--parse")) {
+        std::printf("name %s\n", c.name().c_str());
+        for (const auto& t : c.tensors())
+            std::printf("tensor %s q%d %s %lld %lld %lld\n", t.name.c_str(), (int)t.quant,
+                        t.layout == CYBQ_LAYOUT_PLANAR ? "planar" : "block_aos", (long long)t.N, (long long)t.K,
+                        (long long)(t.q - c.part("weights").first));
+        return 0;
+    }
+    if (argc < 6) { std::fprintf(stderr, "--run needs FILE X Y M\n"); return 2; }
+    const int64_t M = std::atoll(argv[5]);
+    const bool exact = argc > 6 && !std::strcmp(argv[6], "exact");
+    cybq::Backend be(0);
+    if (!be.ok()) { std::printf("ERROR %d %s\n", be.status().code, be.status().text.c_str()); return 1; }
+    be.set_prefill_mode(exact ? CYBQ_PREFILL_EXACT : CYBQ_PREFILL_FAST);
+    s = c.load_into(be);
+    if (!s) { std::printf("ERROR %d %s\n", s.code, s.text.c_str()); return 1; }
+
+    std::vector<char> xb = slurp(argv[3]), yb = slurp(argv[4]);
+    void* xd = nullptr;
+    if (hipMalloc(&xd, xb.size()) != hipSuccess || hipMemcpy(xd, xb.data(), xb.size(), hipMemcpyHostToDevice) != hipSuccess) {
+        std::printf("ERROR hip x\n"); return 1;
+    }
+    std::map<std::string, cybq::Edge> edges;
+    edges["x"] = cybq::Edge{xd, CYBQ_F16, M, c.tensors()[0].K};
+    std::vector<cybq::QMatMulNode> nodes;
+    std::vector<float*> outs;
+    for (size_t i = 0; i < c.tensors().size(); i++) {
+        const auto& t = c.tensors()[i];
+        float* yd = nullptr;
+        if (hipMalloc((void**)&yd, (size_t)M * t.N * 4) != hipSuccess) { std::printf("ERROR hip y\n"); return 1; }
+        outs.push_back(yd);
+        std::string yname = "y" + std::to_string(i);
+        edges[yname] = cybq::Edge{yd, CYBQ_F32, M, t.N};
+        cybq::QMatMulNode n;
+        n.w = t.name; n.x = "x"; n.y = yname; n.quant = t.quant; n.M = M; n.N = t.N; n.K = t.K;
+        nodes.push_back(n);
+    }
+    // first node through run(), all nodes through run_all(): both paths must agree
+    s = be.run(nodes[0], edges);
+    if (!s) { std::printf("ERROR %d %s\n", s.code, s.text.c_str()); return 1; }
+    s = be.run_all(nodes, edges);
+    if (!s) { std::printf("ERROR %d %s\n", s.code, s.text.c_str()); return 1; }
+    if (hipDeviceSynchronize() != hipSuccess) { std::printf("ERROR sync\n"); return 1; }
+    // error paths stay values
+    cybq::QMatMulNode bad = nodes[0];
+    bad.w = "no.such.tensor";
+    if (be.run(bad, edges).code != CYBQ_ERR_INVALID) { std::printf("ERROR missing tensor not reported\n"); return 1; }
+    bad = nodes[0];
+    bad.N += 16;
+    if (be.run(bad, edges).code != CYBQ_ERR_SHAPE) { std::printf("ERROR shape mismatch not reported\n"); return 1; }
+
+    const double* want = reinterpret_cast<const double*>(yb.data());
+    for (size_t i = 0; i < nodes.size(); i++) {
+        const int64_t cnt = M * nodes[i].N;
+        std::vector<float> got((size_t)cnt);
+        if (hipMemcpy(got.data(), outs[i], (size_t)cnt * 4, hipMemcpyDeviceToHost) != hipSuccess) { std::printf("ERROR copy\n"); return 1; }
+        double num = 0, den = 0;
+        for (int64_t j = 0; j < cnt; j++) { double d = got[j] - want[j]; num += d * d; den += want[j] * want[j]; }
+        std::printf("rel_l2 %s %.6e\n", nodes[i].w.c_str(), std::sqrt(num / den));
+        want += cnt;
+    }
+    std::printf("OK\n");
+    return 0;
+}
