@@ -214,6 +214,41 @@ def main():
             sweep[f"M{Mb}"] = {"us": round(e * 1e6, 2),
                                "GB/s": round(formats.matmul_bytes(bits, N, K, Mb, 2, 4) / e / 1e9, 1)}
         extra["decode_batch_sweep_4096x14336"] = sweep
+        # the reference-shaped decode step: 32 layers x (q,k,v,o,gate,up,down), Q4, random init,
+        # one native walk over the 224 linear nodes per step (BASELINE configs[4])
+        for t in ws[1:]:
+            t.free()
+        del ws[1:]
+        from cyb_amd import stack as stk
+        stack_out = {}
+        for label, shapes in (("per_linear_224_launches", None), ("qkv_and_gate_up_fused_128_launches", stk.fused_shapes())):
+            t0 = time.time()
+            st = stk.build(be, layers=32, seed=5, shapes=shapes, order=list(shapes) if shapes else None)
+            log(f"stack {label} built in {time.time() - t0:.1f}s: {st.weight_bytes} weight bytes")
+            res = {"weight_bytes": int(st.weight_bytes), "launches_per_step": len(st.nodes)}
+            for Ms in (1, 8):
+                edges = stk.edges_for(st, Ms, shapes=shapes)
+                pl = stk.plan(st, edges)
+                be.matmul_many(pl, Ms, stream)
+                reps = 20
+                torch.cuda.synchronize()
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                for _ in range(reps):
+                    be.matmul_many(pl, Ms, stream)
+                b.record()
+                torch.cuda.synchronize()
+                per = a.elapsed_time(b) * 1e-3 / reps
+                res[f"M{Ms}"] = {"us_per_step": round(per * 1e6, 1),
+                                 "GB/s": round(st.step_bytes(Ms) / per / 1e9, 1),
+                                 "frac_of_hbm_peak": round(st.step_bytes(Ms) / per / 1e9 / HBM_PEAK_GBS, 4),
+                                 "linear_stack_tok_per_s": round(Ms / per, 1)}
+                log(f"decode stack {label} M={Ms}: {per * 1e6:.0f} us/step")
+            stack_out[label] = res
+            for t in st.weights:
+                t.free()
+            del st, pl, edges
+        extra["decode_stack_llama3_8b_q4"] = stack_out
         result["extra"] = extra
 
     if not args.no_cpu:

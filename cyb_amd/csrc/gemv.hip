@@ -387,11 +387,13 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
 {
     // Waves per workgroup (= split of a strip's K tiles).  Depends on the weight
     // shape only, never on M, so that the summation order is the same for every
-    // batch size: enough waves for ~8 per CU, at most 8, never more than tiles.
+    // batch size: enough waves for ~8 per CU (at most 8), then 16 if that is what
+    // it takes to bring a wave's share down to 8 tiles, all requested up front.
     int nwaves = g_tune_waves;
     if (nwaves <= 0) {
         nwaves = 2;
         while (nwaves < 8 && (int64_t)w.NT * nwaves < (int64_t)num_cus * 8) nwaves *= 2;
+        while (nwaves < 16 && w.KT > 8 * nwaves) nwaves *= 2;
     }
     if (nwaves > 16) nwaves = 16;
     while (nwaves > 1 && nwaves > w.KT) nwaves >>= 1;

@@ -374,3 +374,54 @@ def test_error_codes(backend, oracle):
     backend.matmul(qw, x, y)
     torch.cuda.synchronize()
     assert oracle.rel_l2(y.cpu().numpy(), oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT
+
+
+# ------------------------------------------------------------ decode-step stack
+
+def test_decode_stack_small(backend, oracle):
+    """Config 5 in miniature: 2 layers x 7 linears of a scaled-down LlamaStyle model,
+    weights generated and quantised on the device, every linear checked on its own."""
+    from cyb_amd import stack
+    shapes = {"q_proj": (512, 512), "k_proj": (512, 128), "v_proj": (512, 128), "o_proj": (512, 512),
+              "gate_proj": (512, 1792), "up_proj": (512, 1792), "down_proj": (1792, 512)}
+    st = stack.build(backend, layers=2, seed=5, keep_planar=2, shapes=shapes)
+    assert len(st.nodes) == 14
+    for M in (1, 8):
+        edges = stack.edges_for(st, M, shapes=shapes)
+        pl = stack.plan(st, edges)
+        # run linear by linear so that every output can be read before it is overwritten
+        for i, node in enumerate(st.nodes):
+            node.M = M
+            backend.run(node, edges)
+            torch.cuda.synchronize()
+            qd, sd = st.planar[node.w]
+            q = formats.unpack_planar(qd.cpu().numpy(), 4, node.N, node.K)
+            s = sd.cpu().numpy().view(np.uint16).reshape(node.N, node.K // 32)
+            ref = oracle.matmul_f64(q, s, edges[node.x].float().cpu().numpy())
+            assert oracle.rel_l2(edges[node.y].cpu().numpy(), ref) < TIGHT, node.w
+        # and the whole step through the native node walk gives the last layer's outputs
+        backend.matmul_many(pl, M)
+        torch.cuda.synchronize()
+        last = st.nodes[-1]
+        qd, sd = st.planar[last.w]
+        q = formats.unpack_planar(qd.cpu().numpy(), 4, last.N, last.K)
+        s = sd.cpu().numpy().view(np.uint16).reshape(last.N, last.K // 32)
+        ref = oracle.matmul_f64(q, s, edges[last.x].float().cpu().numpy())
+        assert oracle.rel_l2(edges[last.y].cpu().numpy(), ref) < TIGHT
+    assert st.step_bytes(1) == sum(formats.matmul_bytes(4, n.N, n.K, 1, 2, 4) for n in st.nodes)
+    for w in st.weights:
+        w.free()
+
+
+def test_container_to_backend(backend, oracle, tmp_path):
+    from cyb_amd import container
+    q, s = _quant(oracle, 4, 64, 256)
+    path = str(tmp_path / "one.model")
+    container.write_container(path, "one", "", [container.tensor_entry("lm_head.weight", q, s, 4, formats.BLOCK_AOS)])
+    recs = container.load_into(backend, path)
+    assert [r.name for r in recs] == ["lm_head.weight"]
+    x = _x(3, 256, "f16")
+    y = torch.empty((3, 64), dtype=torch.float32, device="cuda")
+    backend.run(QMatMul(w="lm_head.weight", x="x", y="y", quant=4, M=3, N=64, K=256), {"x": x, "y": y})
+    torch.cuda.synchronize()
+    assert oracle.rel_l2(y.cpu().numpy(), oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT
