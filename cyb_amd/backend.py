@@ -292,5 +292,7 @@ class Backend:
             raise CybqError(-1, "invalid argument", f"prefill mode {mode!r}")
         self._check(self._lib.cybq_set_prefill_mode(self._ctx, codes[mode]))
 
-    def set_gemv_tuning(self, waves: int = 0, strips: int = 0, unroll: int = 0) -> None:
-        self._lib.cybq_debug_set_gemv_tuning(waves, strips, unroll)
+    def set_gemv_tuning(self, waves: int = 0, rows_kernel: int = 0, unroll: int = 0) -> None:
+        """Diagnostics: waves per workgroup; decode kernel choice (0 auto, 1 always the
+        x-in-registers kernel, 2 never); streaming batch size.  0 = automatic."""
+        self._lib.cybq_debug_set_gemv_tuning(waves, rows_kernel, unroll)

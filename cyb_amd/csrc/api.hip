@@ -376,9 +376,9 @@ int cybq_quantize(cybq_ctx* ctx, cybq_quant quant, const float* src, int64_t N, 
 
 /* Test and benchmark hook (not part of the operator interface): overrides the
  * decode kernel's launch heuristics; 0 restores the automatic choice. */
-int cybq_debug_set_gemv_tuning(int waves_per_group, int reserved, int unroll)
+int cybq_debug_set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll)
 {
-    cybq::set_gemv_tuning(waves_per_group, reserved, unroll);
+    cybq::set_gemv_tuning(waves_per_group, rows_kernel, unroll);
     return CYBQ_OK;
 }
 

@@ -31,6 +31,6 @@ hipError_t launch_quantize(int bits, const float* src, int N, int K, void* q_out
                            hipStream_t st);
 
 // test/bench hook: overrides the decode kernel's launch heuristics (0 = automatic)
-void set_gemv_tuning(int waves_per_group, int strips_per_group, int unroll);
+void set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll);
 
 }  // namespace cybq

@@ -309,7 +309,165 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
     }
 }
 
-int g_tune_waves = 0, g_tune_unroll = 0;
+// ---------------------------------------------------------------------------
+// Batch rows 5..16: x operands live in REGISTERS and are reused across strips.
+//
+// With more than a few batch rows the LDS kernel above spends its time moving
+// x: every 16-row strip's workgroup stages all M rows of x (128 KB at M = 16,
+// K = 4096, against 37 KB of weights).  Here a workgroup owns NS consecutive
+// strips; each wave loads the A operands of ITS K tiles once (lane = batch row
+// l%16, 8 k per lane: a 16 B global load per lane per scale group, no LDS, no
+// barrier), requests the weight tiles of all NS strips at once and walks over
+// the strips with the same operands.  Tile kt belongs
+// to wave kt % waves and partials are summed in wave order: deterministic, and a
+// row's bits do not depend on the batch it is part of (within this kernel; the
+// LDS kernel may split K over a different number of waves).
+template <int BITS, int XMODE>
+__device__ __forceinline__ void tile_issue_regs(const TileRegs<BITS>& t, const Frag16 (&a)[4], uint32_t magic,
+                                                float4_t d[4])
+{
+    const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+    Frag16 b[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        uint32_t bw[4];
+        if (BITS == 4) unpack_q4_f16(t.q[0][j], magic, bw);
+        else unpack_q8_f16(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
+        if (XMODE == XBF16) f16frag_to_bf16frag(bw);
+        b[j].u = (u32x4_t){bw[0], bw[1], bw[2], bw[3]};
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        if (XMODE == XBF16) d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].b, b[j].b, zero, 0, 0, 0);
+        else d[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j].h, b[j].h, zero, 0, 0, 0);
+    }
+}
+
+template <int BITS, int XMODE, int TS, int NS>
+// (waves_per_eu: the scheduler would otherwise trade the up-front loads for occupancy)
+__global__ __launch_bounds__(TS <= 2 ? 1024 : 512) __attribute__((amdgpu_waves_per_eu(2, TS <= 2 ? 4 : 2)))
+void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x,
+                                                                         int M, void* __restrict__ y, int ydt)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t magic = q4_magic_vgpr();
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nwaves = (int)blockDim.x >> 6;
+    const int oct = lane >> 4;
+    const int strip0 = blockIdx.x * NS;
+    const int KT = w.KT;
+    const int kmax = w.K - 8 - oct * 8;
+    const uint16_t* xrow = x + (int64_t)min(lane & 15, M - 1) * w.K + oct * 8;
+
+    float acc[NS][4];
+#pragma unroll
+    for (int s = 0; s < NS; s++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[s][r] = 0.f;
+
+    int64_t sbase[NS];
+#pragma unroll
+    for (int s = 0; s < NS; s++) sbase[s] = (int64_t)min(strip0 + s, w.NT - 1) * KT;
+
+    for (int slab0 = 0; slab0 < KT; slab0 += nwaves * TS) {
+        // my K tiles of this slab and their x operands (clamped past the end; such tiles get scale 0)
+        int kt[TS];
+        bool valid[TS];
+        Frag16 a[TS][4];
+#pragma unroll
+        for (int u = 0; u < TS; u++) {
+            const int t = slab0 + wv + nwaves * u;
+            valid[u] = t < KT;
+            kt[u] = min(t, KT - 1);
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                a[u][j].u = *reinterpret_cast<const u32x4_t*>(xrow + min(kt[u] * kTileK + j * 32, kmax));
+        }
+        // every weight tile of this slab (all strips) is requested before the first
+        // one is used: the whole slab is in flight while the wave works through it
+        TileRegs<BITS> buf[NS][TS];
+#pragma unroll
+        for (int s = 0; s < NS; s++)
+#pragma unroll
+            for (int u = 0; u < TS; u++) load_tile<BITS>(buf[s][u], w, sbase[s] + kt[u], lane);
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            float4_t dprev[4];
+            u32x2_t sprev = {0u, 0u};
+#pragma unroll
+            for (int j = 0; j < 4; j++) dprev[j] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < TS; u++) {
+                float4_t d[4];
+                tile_issue_regs<BITS, XMODE>(buf[s][u], a[u], magic, d);
+                u32x2_t sc = buf[s][u].s;
+                sc[0] = valid[u] ? sc[0] : 0u;
+                sc[1] = valid[u] ? sc[1] : 0u;
+                tile_accum<4>(sprev, dprev, acc[s]);
+#pragma unroll
+                for (int j = 0; j < 4; j++) dprev[j] = d[j];
+                sprev = sc;
+            }
+            tile_accum<4>(sprev, dprev, acc[s]);
+        }
+    }
+
+    // split-K partials -> LDS, summed in wave order
+    float* red = reinterpret_cast<float*>(smem);
+#pragma unroll
+    for (int s = 0; s < NS; s++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) red[((s * nwaves + wv) * 4 + r) * 64 + lane] = acc[s][r];
+    __syncthreads();
+    // wave v finishes strips v, v + waves, ...
+    for (int s = wv; s < NS; s += nwaves) {
+        const int nt = strip0 + s;
+        const int n = nt * 16 + (lane & 15);
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            float v = 0.f;
+            for (int k = 0; k < nwaves; k++) v += red[((s * nwaves + k) * 4 + r) * 64 + lane];
+            const int m = 4 * oct + r;
+            if (nt < w.NT && m < M && n < w.N) store_out(y, ydt, (int64_t)m * w.N + n, v);
+        }
+    }
+}
+
+template <int BITS, int XMODE, int TS, int NS>
+hipError_t launch_rows_t(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, hipStream_t st)
+{
+    const size_t lds = (size_t)NS * nwaves * 4 * 64 * sizeof(float);
+    const unsigned groups = (unsigned)((w.NT + NS - 1) / NS);
+    hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS>), dim3(groups), dim3(nwaves * 64), lds, st, w,
+                       reinterpret_cast<const uint16_t*>(x), M, y, ydt);
+    return hipGetLastError();
+}
+
+template <int BITS, int XMODE>
+hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int ydt, int tuned_waves, int num_cus,
+                       hipStream_t st)
+{
+    // strips per workgroup: as many as keeps about one workgroup per CU, at most 4;
+    // 8 waves split K (fewer when the strip has fewer tiles), 4 tiles of x per wave and slab
+    int ns = (w.NT + num_cus / 2) / num_cus;
+    ns = ns >= 3 ? 4 : (ns >= 2 ? 2 : 1);
+    int nwaves = tuned_waves > 0 ? tuned_waves : 8;
+    while (nwaves > 1 && nwaves * 2 > w.KT) nwaves >>= 1;
+    if (nwaves > 8) {          // 16 waves: 128 registers per lane, two tiles of x in flight
+        if (ns == 4) return launch_rows_t<BITS, XMODE, 2, 4>(w, x, M, y, ydt, nwaves, st);
+        if (ns == 2) return launch_rows_t<BITS, XMODE, 2, 2>(w, x, M, y, ydt, nwaves, st);
+        return launch_rows_t<BITS, XMODE, 2, 1>(w, x, M, y, ydt, nwaves, st);
+    }
+    if (ns == 4) return launch_rows_t<BITS, XMODE, 4, 4>(w, x, M, y, ydt, nwaves, st);
+    if (ns == 2) return launch_rows_t<BITS, XMODE, 4, 2>(w, x, M, y, ydt, nwaves, st);
+    // one strip per workgroup and a long K: eight tiles per wave and slab, fewer round trips
+    if (w.KT > nwaves * 4) return launch_rows_t<BITS, XMODE, 8, 1>(w, x, M, y, ydt, nwaves, st);
+    return launch_rows_t<BITS, XMODE, 4, 1>(w, x, M, y, ydt, nwaves, st);
+}
+
+int g_tune_waves = 0, g_tune_unroll = 0, g_tune_rows = 0;
 
 constexpr int kLdsBudget = 64 * 1024;
 
@@ -375,10 +533,10 @@ hipError_t launch_u(const WeightView& w, const void* x, int M, void* y, int ydt,
 
 }  // namespace
 
-void set_gemv_tuning(int waves_per_group, int strips_per_group, int unroll)
+void set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll)
 {
-    (void)strips_per_group;
     g_tune_waves = waves_per_group;
+    g_tune_rows = rows_kernel;       // 0 automatic, 1 always the register kernel, 2 never
     g_tune_unroll = unroll;
 }
 
@@ -399,6 +557,17 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
     while (nwaves > 1 && nwaves > w.KT) nwaves >>= 1;
     // 0: request a wave's whole share up front when it fits, else stream in batches of 2
     int unroll = g_tune_unroll;
+
+    // four or more batch rows (16-bit activations): x in registers, shared across strips
+    const bool rows_kernel = g_tune_rows == 1 || (g_tune_rows == 0 && M >= 4);
+    if (rows_kernel && xdt != kF32) {
+        if (w.bits == 4) {
+            if (xdt == kF16) return launch_rows<4, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, st);
+            return launch_rows<4, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, st);
+        }
+        if (xdt == kF16) return launch_rows<8, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, st);
+        return launch_rows<8, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, st);
+    }
 
     if (w.bits == 4) {
         if (xdt == kF16) return launch_u<4, XF16>(w, x, M, y, ydt, nwaves, unroll, st);

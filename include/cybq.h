@@ -164,9 +164,10 @@ int cybq_weight_from_device(cybq_ctx* ctx, cybq_quant quant, int64_t N, int64_t 
 /* ---- diagnostics (not part of the operator interface) ------------------- */
 
 /* Overrides the decode kernel's launch heuristics for experiments: waves per
- * workgroup (1..8), reserved, tiles in flight per wave (2, 4 or 8); 0 restores
- * the automatic choice.  Process-wide. */
-int cybq_debug_set_gemv_tuning(int waves_per_group, int reserved, int unroll);
+ * workgroup (1..16); which decode kernel runs (0 automatic, 1 always the
+ * x-in-registers kernel, 2 never); tiles in flight per wave of the streaming
+ * variant (2 or 4).  0 restores the automatic choice.  Process-wide. */
+int cybq_debug_set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll);
 
 #ifdef __cplusplus
 }

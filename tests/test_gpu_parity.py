@@ -138,25 +138,38 @@ def test_decode_every_kernel_variant(backend, oracle, bits):
             ref = oracle.matmul_f64(q, s, x.float().cpu().numpy())
             for waves in (1, 2, 4, 8, 16):
                 for unroll in (0, 2, 4):
-                    backend.set_gemv_tuning(waves, 0, unroll)
+                    backend.set_gemv_tuning(waves, 2, unroll)       # the LDS kernel, every variant
                     y = _run(backend, qw, x).cpu().numpy()
                     err = oracle.rel_l2(y, ref)
                     assert err < TIGHT, (M, waves, unroll, err)
+                backend.set_gemv_tuning(waves, 1, 0)                # the x-in-registers kernel
+                y2 = _run(backend, qw, x).cpu().numpy()
+                assert oracle.rel_l2(y2, ref) < TIGHT, (M, waves)
+                backend.set_gemv_tuning(waves, 2, 0)
+                assert np.array_equal(y2, _run(backend, qw, x).cpu().numpy()), (M, waves)   # same split, same bits
     finally:
         backend.set_gemv_tuning(0, 0, 0)
 
 
 def test_decode_batched_rows_equal_single_rows_bitwise(backend, oracle):
+    """Within one kernel a row's bits do not depend on the batch it travels in."""
     N, K = 512, 4096
     q, s = _quant(oracle, 4, N, K)
     qw = backend.upload_quantized(q, s, 4)
     x = _x(16, K, "f16")
-    yb = _run(backend, qw, x)
-    for m in (0, 5, 15):
-        y1 = _run(backend, qw, x[m:m + 1].contiguous())
-        assert torch.equal(y1[0], yb[m])
-    # and the kernel is deterministic run to run
-    assert torch.equal(_run(backend, qw, x), yb)
+    try:
+        for kernel, batch in ((2, 4), (2, 16), (1, 16), (1, 7)):      # LDS kernel, x-in-registers kernel
+            backend.set_gemv_tuning(0, kernel, 0)
+            yb = _run(backend, qw, x[:batch].contiguous())
+            for m in (0, batch // 2, batch - 1):
+                y1 = _run(backend, qw, x[m:m + 1].contiguous())
+                assert torch.equal(y1[0], yb[m]), (kernel, batch, m)
+            assert torch.equal(_run(backend, qw, x[:batch].contiguous()), yb)     # and run to run
+    finally:
+        backend.set_gemv_tuning(0, 0, 0)
+    # the automatic choice (LDS kernel up to 4 rows, registers beyond) is deterministic too
+    y16 = _run(backend, qw, x)
+    assert torch.equal(_run(backend, qw, x), y16)
 
 
 def test_decode_special_cases(backend, oracle):
