@@ -1,7 +1,7 @@
 // gemm.hip - prefill kernel: Y[M,N] = X[M,K] * W^T for M > 16 on MFMA.
 //
-// Workgroup = 4 waves, output tile 256 rows x (16*NF) columns; wave w owns rows
-// [64w, 64w+64) of the tile (4 row blocks of 16) against all NF column blocks.
+// Workgroup = 4 waves, output tile 256 or 128 rows x (16*NF) columns; wave w owns a
+// quarter of the rows (4 or 2 row blocks of 16) against all NF column blocks.
 //
 //   X  never touches LDS.  An MFMA A operand is 16 rows x 32 k with lane l
 //      holding row l%16, k 8*(l/16)..+8 - exactly a 16 B global load per lane -
@@ -58,9 +58,7 @@ __device__ __forceinline__ void store_out_g(void* y, int ydt, int64_t idx, float
     else reinterpret_cast<uint16_t*>(y)[idx] = f32_to_bf16_rne_g(v);
 }
 
-constexpr int MF = 4;        // row blocks (of 16) per wave
 constexpr int WAVES = 4;
-constexpr int BM = WAVES * MF * 16;
 
 template <int BITS>
 struct WRegs {               // one native weight tile as loaded by one lane, and its 4 group scales
@@ -151,8 +149,8 @@ __device__ __forceinline__ Frag16 bf16_to_f16_frag(const Frag16& a)
 }
 
 // XBF = 1: X is bf16, 0: X is f16.  EXACT: see the header comment.
-template <int BITS, int XBF, int NF, bool EXACT>
-__global__ __launch_bounds__(256) void gemm_kernel(WeightView w, const uint16_t* __restrict__ x, int M,
+template <int BITS, int XBF, int NF, bool EXACT, int MF>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MF == 4 ? 1 : 2, MF == 4 ? 1 : 2))) void gemm_kernel(WeightView w, const uint16_t* __restrict__ x, int M,
                                                    void* __restrict__ y, int ydt, int n_tiles, int m_tiles, float out_scale)
 {
     // Workgroups are handed to the 8 XCDs round-robin (id % 8) and every XCD has
@@ -164,6 +162,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(WeightView w, const uint16_t*
     if (item >= n_tiles * m_tiles) return;
     const int tile_m = item / n_tiles;
     const int tile_n = item - tile_m * n_tiles;
+    constexpr int BM = WAVES * MF * 16;               // MF = row blocks (of 16) per wave
     constexpr int WT = (NF + WAVES - 1) / WAVES;      // weight tiles a wave stages per K tile
     constexpr int OPS = EXACT ? 2 : 1;                // B operands per scale group
     constexpr int TILE16 = 4 * OPS * 64;              // u32x4 per column block per buffer
@@ -290,11 +289,12 @@ __global__ __launch_bounds__(256) void gemm_kernel(WeightView w, const uint16_t*
         }
 }
 
-template <int BITS, int XBF, int NF, bool EXACT>
-hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, hipStream_t st)
+template <int BITS, int XBF, int NF, bool EXACT, int MF>
+hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, hipStream_t st)
 {
+    constexpr int BM = WAVES * MF * 16;
     const size_t lds = (size_t)2 * NF * (4 * (EXACT ? 2 : 1) * 64) * 16;     // 56 .. 128 KB
-    auto kern = gemm_kernel<BITS, XBF, NF, EXACT>;
+    auto kern = gemm_kernel<BITS, XBF, NF, EXACT, MF>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -309,18 +309,32 @@ hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt,
     return hipGetLastError();
 }
 
+// Rows per workgroup.  256 (4 row blocks per wave, one workgroup per CU) halves the
+// LDS operand reads per MFMA; 128 (2 row blocks per wave) lets two workgroups share
+// a CU, so one's barrier and load stalls are covered by the other's MFMAs.  FAST has
+// LDS bandwidth to spare and prefers 128; EXACT reads two operands per group and
+// prefers 256 unless that leaves CUs without a tile.
+template <int BITS, int XBF, int NF, bool EXACT>
+hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, int num_cus,
+                    hipStream_t st)
+{
+    const int64_t tiles256 = (int64_t)((w.NT + NF - 1) / NF) * ((M + 255) / 256);
+    if (!EXACT || tiles256 < num_cus) return launch_m<BITS, XBF, NF, EXACT, 2>(w, x, M, y, ydt, out_scale, st);
+    return launch_m<BITS, XBF, NF, EXACT, 4>(w, x, M, y, ydt, out_scale, st);
+}
+
 template <int BITS, int XBF>
 hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt, bool exact, float out_scale,
-                     hipStream_t st)
+                     int num_cus, hipStream_t st)
 {
     // 7 column blocks (BN = 112) tile N = 14336 = 128 * 112 exactly: with M = 512
     // that is 256 workgroups, one per CU; 8 column blocks otherwise
     if (w.NT % 7 == 0) {
-        if (exact) return launch_t<BITS, XBF, 7, true>(w, x, M, y, ydt, out_scale, st);
-        return launch_t<BITS, XBF, 7, false>(w, x, M, y, ydt, out_scale, st);
+        if (exact) return launch_t<BITS, XBF, 7, true>(w, x, M, y, ydt, out_scale, num_cus, st);
+        return launch_t<BITS, XBF, 7, false>(w, x, M, y, ydt, out_scale, num_cus, st);
     }
-    if (exact) return launch_t<BITS, XBF, 8, true>(w, x, M, y, ydt, out_scale, st);
-    return launch_t<BITS, XBF, 8, false>(w, x, M, y, ydt, out_scale, st);
+    if (exact) return launch_t<BITS, XBF, 8, true>(w, x, M, y, ydt, out_scale, num_cus, st);
+    return launch_t<BITS, XBF, 8, false>(w, x, M, y, ydt, out_scale, num_cus, st);
 }
 
 // bf16 [n] -> f16 [n] scaled by 2^-4 (exact for 2^-10 <= |x| < 2^20); n % 8 == 0
@@ -338,7 +352,6 @@ __global__ void widen_bf16_kernel(const u32x4_t* __restrict__ src, u32x4_t* __re
 hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
                        int num_cus, bool exact, void* workspace, size_t workspace_bytes, hipStream_t st)
 {
-    (void)num_cus;
     if (xdt == kF32) return hipErrorNotSupported;   // api.hip walks fp32 prefill through the decode kernel
     float out_scale = 1.0f;
     if (!exact && xdt == kBF16) {
@@ -357,11 +370,11 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
         }
     }
     if (w.bits == 4) {
-        if (xdt == kBF16) return launch_nf<4, 1>(w, x, M, y, ydt, exact, out_scale, st);
-        return launch_nf<4, 0>(w, x, M, y, ydt, exact, out_scale, st);
+        if (xdt == kBF16) return launch_nf<4, 1>(w, x, M, y, ydt, exact, out_scale, num_cus, st);
+        return launch_nf<4, 0>(w, x, M, y, ydt, exact, out_scale, num_cus, st);
     }
-    if (xdt == kBF16) return launch_nf<8, 1>(w, x, M, y, ydt, exact, out_scale, st);
-    return launch_nf<8, 0>(w, x, M, y, ydt, exact, out_scale, st);
+    if (xdt == kBF16) return launch_nf<8, 1>(w, x, M, y, ydt, exact, out_scale, num_cus, st);
+    return launch_nf<8, 0>(w, x, M, y, ydt, exact, out_scale, num_cus, st);
 }
 
 }  // namespace cybq
