@@ -28,8 +28,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 MALL_BYTES = 256 << 20
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain
 # 256 MiB copy: FETCH x 1.9997, WRITE x 1.0000); profiles/decode_gemv_q4_4096x14336_m1.md
-TRAFFIC_DECODE_BYTES = 33_275_500
-TRAFFIC_PREFILL_M512_BYTES = 112_865_000
+TRAFFIC_DECODE_BYTES = 33_275_300
+TRAFFIC_PREFILL_M512_BYTES = 170_381_000
 
 
 def log(*a):
