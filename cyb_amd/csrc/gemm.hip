@@ -1,7 +1,7 @@
 // gemm.hip - prefill kernel: Y[M,N] = X[M,K] * W^T for M > 16 on MFMA.
 //
-// Workgroup = 4 waves, output tile 256 or 128 rows x (16*NF) columns; wave w owns a
-// quarter of the rows (4 or 2 row blocks of 16) against all NF column blocks.
+// Workgroup = 4 or 8 waves, output tile 256 or 128 rows x (16*NF) columns; wave w owns
+// its share of the rows (4 or 2 row blocks of 16) against all NF column blocks.
 //
 //   X  never touches LDS.  An MFMA A operand is 16 rows x 32 k with lane l
 //      holding row l%16, k 8*(l/16)..+8 - exactly a 16 B global load per lane -
@@ -58,7 +58,6 @@ __device__ __forceinline__ void store_out_g(void* y, int ydt, int64_t idx, float
     else reinterpret_cast<uint16_t*>(y)[idx] = f32_to_bf16_rne_g(v);
 }
 
-constexpr int WAVES = 4;
 
 template <int BITS>
 struct WRegs {               // one native weight tile as loaded by one lane, and its 4 group scales
@@ -149,8 +148,8 @@ __device__ __forceinline__ Frag16 bf16_to_f16_frag(const Frag16& a)
 }
 
 // XBF = 1: X is bf16, 0: X is f16.  EXACT: see the header comment.
-template <int BITS, int XBF, int NF, bool EXACT, int MF>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MF == 4 ? 1 : 2, MF == 4 ? 1 : 2))) void gemm_kernel(WeightView w, const uint16_t* __restrict__ x, int M,
+template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF == 4 ? 1 : 2, MF == 4 ? 1 : 2))) void gemm_kernel(WeightView w, const uint16_t* __restrict__ x, int M,
                                                    void* __restrict__ y, int ydt, int n_tiles, int m_tiles, float out_scale)
 {
     // Workgroups are handed to the 8 XCDs round-robin (id % 8) and every XCD has
@@ -289,12 +288,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MF == 4 ? 1
         }
 }
 
-template <int BITS, int XBF, int NF, bool EXACT, int MF>
+template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES>
 hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, hipStream_t st)
 {
     constexpr int BM = WAVES * MF * 16;
     const size_t lds = (size_t)2 * NF * (4 * (EXACT ? 2 : 1) * 64) * 16;     // 56 .. 128 KB
-    auto kern = gemm_kernel<BITS, XBF, NF, EXACT, MF>;
+    auto kern = gemm_kernel<BITS, XBF, NF, EXACT, MF, WAVES>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -304,23 +303,25 @@ hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt,
     }
     const int n_tiles = (w.NT + NF - 1) / NF, m_tiles = (M + BM - 1) / BM;
     const unsigned groups = (unsigned)(((int64_t)n_tiles * m_tiles + 7) / 8 * 8);
-    hipLaunchKernelGGL(kern, dim3(groups), dim3(256), lds, st, w, reinterpret_cast<const uint16_t*>(x), M, y, ydt,
+    hipLaunchKernelGGL(kern, dim3(groups), dim3(WAVES * 64), lds, st, w, reinterpret_cast<const uint16_t*>(x), M, y, ydt,
                        n_tiles, m_tiles, out_scale);
     return hipGetLastError();
 }
 
-// Rows per workgroup.  256 (4 row blocks per wave, one workgroup per CU) halves the
-// LDS operand reads per MFMA; 128 (2 row blocks per wave) lets two workgroups share
-// a CU, so one's barrier and load stalls are covered by the other's MFMAs.  FAST has
-// LDS bandwidth to spare and prefers 128; EXACT reads two operands per group and
-// prefers 256 unless that leaves CUs without a tile.
+// Workgroup shapes.
+//   4 waves x 4 row blocks (256 rows): fewest LDS operand reads per MFMA; one wave per SIMD.
+//   8 waves x 2 row blocks (256 rows): two waves per SIMD cover each other's stalls, the tile's
+//       weights are still loaded and dequantised once; every wave reads all B operands, so
+//       LDS reads per MFMA double - fine for FAST (one operand per group), too much for EXACT.
+//   4 waves x 2 row blocks (128 rows): twice the tiles, for grids that would leave CUs idle.
 template <int BITS, int XBF, int NF, bool EXACT>
 hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, int num_cus,
                     hipStream_t st)
 {
     const int64_t tiles256 = (int64_t)((w.NT + NF - 1) / NF) * ((M + 255) / 256);
-    if (!EXACT || tiles256 < num_cus) return launch_m<BITS, XBF, NF, EXACT, 2>(w, x, M, y, ydt, out_scale, st);
-    return launch_m<BITS, XBF, NF, EXACT, 4>(w, x, M, y, ydt, out_scale, st);
+    if (tiles256 < num_cus) return launch_m<BITS, XBF, NF, EXACT, 2, 4>(w, x, M, y, ydt, out_scale, st);
+    if (!EXACT) return launch_m<BITS, XBF, NF, EXACT, 2, 8>(w, x, M, y, ydt, out_scale, st);
+    return launch_m<BITS, XBF, NF, EXACT, 4, 4>(w, x, M, y, ydt, out_scale, st);
 }
 
 template <int BITS, int XBF>
