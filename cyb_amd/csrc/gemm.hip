@@ -33,6 +33,8 @@
 // Out-of-range rows / columns / k are clamped to valid addresses inside the hot
 // loop (their results are never stored, padded weights are zero); the loop has
 // no branches, so the compiler can count outstanding loads exactly.
+#include <type_traits>
+
 #include "cybq_device.h"
 #include "cybq_internal.h"
 
@@ -178,15 +180,27 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF =
     const int nt0 = tile_n * NF;
     const int m0 = tile_m * BM + wv * (MF * 16);
     const int K = w.K, KT = w.KT;
-    const int kmax = K - 8 - oct * 8;                 // largest valid per-lane k offset
 
     const u32x4_t* qp = reinterpret_cast<const u32x4_t*>(w.q);
     const u32x2_t* sp = reinterpret_cast<const u32x2_t*>(w.s);
 
-    // per-lane row pointers of this wave's four row blocks (rows clamped to M-1)
-    const uint16_t* xrow[MF];
+    // X addressing: a wave-uniform byte pointer (row block base + k) plus a 32-bit
+    // per-lane byte offset (row within the tile, k octet), so a load costs no vector
+    // ALU work.  Rows past M-1 are clamped to M-1 (never stored); a scale group past
+    // K (padding, zero weights) reads the last real group instead - K % 32 == 0, so
+    // the clamp is uniform.
+    const char* xtile = reinterpret_cast<const char*>(x + (int64_t)tile_m * BM * K);
+    uint32_t xoff[MF];
 #pragma unroll
-    for (int i = 0; i < MF; i++) xrow[i] = x + (int64_t)min(m0 + i * 16 + row16, M - 1) * K + oct * 8;
+    for (int i = 0; i < MF; i++) {
+        const int row = min(m0 + i * 16 + row16, M - 1) - tile_m * BM;
+        xoff[i] = (uint32_t)(((int64_t)row * K + oct * 8) * 2);
+    }
+    auto load_x = [&](Frag16 (&dst)[MF], int kstart) {
+        const char* base = xtile + (int64_t)min(kstart, K - 32) * 2;
+#pragma unroll
+        for (int i = 0; i < MF; i++) dst[i].u = *reinterpret_cast<const u32x4_t*>(base + xoff[i]);
+    };
 
     // the weight tiles this wave stages: column block f = wv + WAVES*t (clamped)
     int64_t wtile[WT];
@@ -203,20 +217,17 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF =
 #pragma unroll
         for (int f = 0; f < NF; f++) acc[i][f] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-    // ---- prologue: first K tile of X, W tile 0 -> LDS buffer 0
+    // ---- prologue: first K tile of X, W tile 0 -> LDS buffer 0, W tile 1 -> registers
     Frag16 xa[4][MF];          // one K tile (four scale groups) of X in flight
 #pragma unroll
-    for (int j = 0; j < 4; j++)
-#pragma unroll
-        for (int i = 0; i < MF; i++)
-            xa[j][i].u = *reinterpret_cast<const u32x4_t*>(xrow[i] + min(j * 32, kmax));
-    WRegs<BITS> wr[WT];        // packed weights of the K tile that is dequantised next
+    for (int j = 0; j < 4; j++) load_x(xa[j], j * 32);
+    WRegs<BITS> wreg[2][WT];   // packed weights: K tile t waits in wreg[t & 1]
     {
         WRegs<BITS> w0[WT];
 #pragma unroll
         for (int t = 0; t < WT; t++) load_wtile<BITS>(w0[t], qp, sp, wtile[t], lane);
 #pragma unroll
-        for (int t = 0; t < WT; t++) load_wtile<BITS>(wr[t], qp, sp, wtile[t] + min(1, KT - 1), lane);
+        for (int t = 0; t < WT; t++) load_wtile<BITS>(wreg[1][t], qp, sp, wtile[t] + min(1, KT - 1), lane);
 #pragma unroll
         for (int t = 0; t < WT; t++)
 #pragma unroll
@@ -225,22 +236,28 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF =
     }
     __syncthreads();
 
-    for (int kt = 0; kt < KT; kt++) {
-        const u32x4_t* wcur = ws + (kt & 1) * (NF * TILE16);
-        u32x4_t* wnxt = ws + ((kt + 1) & 1) * (NF * TILE16);
-        // wr holds K tile kt+1 (requested one iteration ago, so the HBM latency is
-        // behind us); request tile kt+2 now.  Past the end the index is clamped:
-        // the tile is staged again but never read.
+    // One K tile.  P = kt & 1 is a compile-time constant (the loop below is unrolled
+    // by two), so LDS buffers and register sets alternate without copies or selects:
+    //   multiply from LDS buffer P;  dequantise tile kt+1 (wreg[1-P], requested one
+    //   iteration ago: its HBM latency is behind us) into LDS buffer 1-P;  request
+    //   tile kt+2 into wreg[P].  Past the end indices are clamped: a tile is staged
+    //   again but never read.
+    auto k_tile = [&](int kt, auto parity) {
+        constexpr int P = decltype(parity)::value;
+        const u32x4_t* wcur = ws + P * (NF * TILE16);
+        u32x4_t* wnxt = ws + (1 - P) * (NF * TILE16);
         const int ktn = min(kt + 2, KT - 1);
-        WRegs<BITS> wn[WT];
 #pragma unroll
-        for (int t = 0; t < WT; t++) load_wtile<BITS>(wn[t], qp, sp, wtile[t] + ktn, lane);
+        for (int t = 0; t < WT; t++) load_wtile<BITS>(wreg[P][t], qp, sp, wtile[t] + ktn, lane);
 
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            Frag16 a[MF];
+            Frag16 cv[MF];
+            if (!EXACT && XBF) {
 #pragma unroll
-            for (int i = 0; i < MF; i++) a[i] = (!EXACT && XBF) ? bf16_to_f16_frag(xa[j][i]) : xa[j][i];
+                for (int i = 0; i < MF; i++) cv[i] = bf16_to_f16_frag(xa[j][i]);
+            }
+            const Frag16 (&a)[MF] = (!EXACT && XBF) ? cv : xa[j];
 #pragma unroll
             for (int f = 0; f < NF; f++) {
                 Frag16 b[OPS];
@@ -255,23 +272,21 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF =
             // the same groups of the next K tile.  The two loads of a row hit the
             // two halves of one 128 B line back to back.
             if (j & 1) {
-#pragma unroll
-                for (int jj = j - 1; jj <= j; jj++) {
-                    const int kn = min((kt + 1) * kTileK + jj * 32, kmax);
-#pragma unroll
-                    for (int i = 0; i < MF; i++) xa[jj][i].u = *reinterpret_cast<const u32x4_t*>(xrow[i] + kn);
-                }
+                load_x(xa[j - 1], (kt + 1) * kTileK + (j - 1) * 32);
+                load_x(xa[j], (kt + 1) * kTileK + j * 32);
             }
             // a quarter of the next tile's dequantisation rides along with every group
-            // (a wave whose second tile index is clamped rewrites a neighbour's
-            // block with identical values: no branch in the hot loop)
+            // (a wave whose tile index is clamped rewrites a neighbour's block with
+            // identical values: no branch in the hot loop)
 #pragma unroll
             for (int t = 0; t < WT; t++)
-                dequant_group_to_lds<BITS, XBF, EXACT>(wr[t], j, magic, wnxt + wf[t] * TILE16, lane);
+                dequant_group_to_lds<BITS, XBF, EXACT>(wreg[1 - P][t], j, magic, wnxt + wf[t] * TILE16, lane);
         }
-#pragma unroll
-        for (int t = 0; t < WT; t++) wr[t] = wn[t];
         __syncthreads();
+    };
+    for (int kt = 0; kt < KT; kt += 2) {
+        k_tile(kt, std::integral_constant<int, 0>{});
+        if (kt + 1 < KT) k_tile(kt + 1, std::integral_constant<int, 1>{});
     }
 
     // ---- epilogue
