@@ -33,6 +33,7 @@
 // Out-of-range rows / columns / k are clamped to valid addresses inside the hot
 // loop (their results are never stored, padded weights are zero); the loop has
 // no branches, so the compiler can count outstanding loads exactly.
+#include <cstdlib>
 #include <type_traits>
 
 #include "cybq_device.h"
@@ -150,10 +151,16 @@ __device__ __forceinline__ Frag16 bf16_to_f16_frag(const Frag16& a)
 }
 
 // XBF = 1: X is bf16, 0: X is f16.  EXACT: see the header comment.
-template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF == 4 ? 1 : 2, MF == 4 ? 1 : 2))) void gemm_kernel(WeightView w, const uint16_t* __restrict__ x, int M,
+// WAVES waves form MW = WAVES / KS row groups times KS K parts: wave (wm, kp) owns
+// MF row blocks of 16 against all NF column blocks and multiplies the K tiles
+// kt with kt % KS == kp.  KS = 2 lets two waves share a SIMD (they cover each
+// other's waits) while each still reuses a B operand read from LDS for MF = 4
+// MFMAs; the two partial sums are added once, through LDS, in the epilogue.
+template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES, int KS>
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF * WAVES <= 8 ? 2 : WAVES / 4, MF * WAVES <= 8 ? 2 : WAVES / 4))) void gemm_kernel(WeightView w, const u32x4_t* __restrict__ x, int x_row_blocks, int M,
                                                    void* __restrict__ y, int ydt, int n_tiles, int m_tiles, float out_scale)
 {
+    static_assert(KS == 1 || KS == 2, "K parts per workgroup");
     // Workgroups are handed to the 8 XCDs round-robin (id % 8) and every XCD has
     // its own L2.  Give each XCD a contiguous run of tiles in row-block-major
     // order, so the workgroups sharing an L2 read the same rows of X and X is
@@ -163,53 +170,88 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF =
     if (item >= n_tiles * m_tiles) return;
     const int tile_m = item / n_tiles;
     const int tile_n = item - tile_m * n_tiles;
-    constexpr int BM = WAVES * MF * 16;               // MF = row blocks (of 16) per wave
-    constexpr int WT = (NF + WAVES - 1) / WAVES;      // weight tiles a wave stages per K tile
+    constexpr int MW = WAVES / KS;                    // waves along M
+    constexpr int BM = MW * MF * 16;                  // MF = row blocks (of 16) per wave
+    constexpr int UNITS = KS * NF;                    // weight tiles staged per step
+    constexpr int WT = (UNITS + WAVES - 1) / WAVES;   // ... of which one wave stages WT
     constexpr int OPS = EXACT ? 2 : 1;                // B operands per scale group
-    constexpr int TILE16 = 4 * OPS * 64;              // u32x4 per column block per buffer
+    constexpr int TILE16 = 4 * OPS * 64;              // u32x4 per column block per K tile
+    constexpr int BUF16 = UNITS * TILE16;             // u32x4 per LDS buffer
     constexpr int MMA_BF = EXACT ? XBF : 0;           // FAST always multiplies in f16
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    u32x4_t* ws = reinterpret_cast<u32x4_t*>(smem);   // [2][NF][4][2][64]
+    u32x4_t* ws = reinterpret_cast<u32x4_t*>(smem);   // [2][KS][NF][4][OPS][64]
     const uint32_t magic = q4_magic_vgpr();
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kp = wv / MW, wm = wv - kp * MW;
     const int row16 = lane & 15;
     const int oct = lane >> 4;
     const int nt0 = tile_n * NF;
-    const int m0 = tile_m * BM + wv * (MF * 16);
+    const int m0 = tile_m * BM + wm * (MF * 16);
     const int K = w.K, KT = w.KT;
+    const int steps = (KT + KS - 1) / KS;
+    // Workgroups that run side by side share rows of X.  Walking K in the same order
+    // they would all ask the same few L2 channels for the same lines at the same
+    // moment (a row of X is a multiple of the channel interleave long), so each
+    // column tile starts its walk at a different K tile and wraps around.  The
+    // order depends on the column tile only: a row of Y does not depend on M.
+    const int kt0 = tile_n % KT;
+    auto rot = [&](int kt) {
+        const int r = min(kt, KT - 1) + kt0;
+        return r >= KT ? r - KT : r;
+    };
 
     const u32x4_t* qp = reinterpret_cast<const u32x4_t*>(w.q);
     const u32x2_t* sp = reinterpret_cast<const u32x2_t*>(w.s);
 
-    // X addressing: a wave-uniform byte pointer (row block base + k) plus a 32-bit
-    // per-lane byte offset (row within the tile, k octet), so a load costs no vector
-    // ALU work.  Rows past M-1 are clamped to M-1 (never stored); a scale group past
-    // K (padding, zero weights) reads the last real group instead - K % 32 == 0, so
-    // the clamp is uniform.
-    const char* xtile = reinterpret_cast<const char*>(x + (int64_t)tile_m * BM * K);
-    uint32_t xoff[MF];
+    // X arrives staged in A-operand order (stage_x_kernel): row block rb, scale group
+    // g is one contiguous KB, lane after lane, so a load is one wave-uniform base
+    // plus lane * 16 B and adjacent lanes read adjacent memory.  Row blocks past the
+    // last are clamped to it (never stored); a scale group past K (padding, zero
+    // weights) reads the last real group instead.
+    const int G = K / kGroup;
+    const u32x4_t* xb[MF];
 #pragma unroll
-    for (int i = 0; i < MF; i++) {
-        const int row = min(m0 + i * 16 + row16, M - 1) - tile_m * BM;
-        xoff[i] = (uint32_t)(((int64_t)row * K + oct * 8) * 2);
-    }
-    auto load_x = [&](Frag16 (&dst)[MF], int kstart) {
-        const char* base = xtile + (int64_t)min(kstart, K - 32) * 2;
+    for (int i = 0; i < MF; i++)
+        xb[i] = x + ((int64_t)min(m0 / 16 + i, x_row_blocks - 1) * G) * 64 + lane;
+    auto load_x = [&](Frag16 (&dst)[MF], int kt, int j) {
+        const int g = min(rot(kt) * 4 + j, G - 1);
 #pragma unroll
-        for (int i = 0; i < MF; i++) dst[i].u = *reinterpret_cast<const u32x4_t*>(base + xoff[i]);
+        for (int i = 0; i < MF; i++) dst[i].u = xb[i][g * 64];
     };
 
-    // the weight tiles this wave stages: column block f = wv + WAVES*t (clamped)
+    // The weight tiles this wave stages: unit u = wv + WAVES*t (clamped) is column
+    // block u % NF of K part u / NF.  wdst: where its operands go inside a buffer.
     int64_t wtile[WT];
-    int wf[WT];
+    int wkp[WT], wdst[WT];
 #pragma unroll
     for (int t = 0; t < WT; t++) {
-        wf[t] = min(wv + WAVES * t, NF - 1);
-        wtile[t] = (int64_t)min(nt0 + wf[t], w.NT - 1) * KT;
+        const int u = min(wv + WAVES * t, UNITS - 1);
+        wkp[t] = u / NF;
+        wdst[t] = u * TILE16;
+        wtile[t] = (int64_t)min(nt0 + (u - wkp[t] * NF), w.NT - 1) * KT;
     }
+    // K tile of unit t in step s is s*KS + wkp[t]; past KT-1 (only with KS > 1, in the
+    // last step) the last tile is loaded again and its scales are masked to zero,
+    // so the wave that multiplies it adds nothing.
+    auto load_units = [&](WRegs<BITS> (&dst)[WT], int step) {
+#pragma unroll
+        for (int t = 0; t < WT; t++)
+            load_wtile<BITS>(dst[t], qp, sp, wtile[t] + rot(step * KS + wkp[t]), lane);
+    };
+    auto stage_units = [&](WRegs<BITS> (&src)[WT], int step, int j, u32x4_t* buf) {
+#pragma unroll
+        for (int t = 0; t < WT; t++) {
+            if (KS > 1 && j == 0) {
+                const uint32_t keep = (step * KS + wkp[t] < KT) ? 0xffffffffu : 0u;
+                src[t].s[0] &= keep;
+                src[t].s[1] &= keep;
+            }
+            dequant_group_to_lds<BITS, XBF, EXACT>(src[t], j, magic, buf + wdst[t], lane);
+        }
+    };
 
     float4_t acc[MF][NF];
 #pragma unroll
@@ -217,47 +259,36 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF =
 #pragma unroll
         for (int f = 0; f < NF; f++) acc[i][f] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-    // ---- prologue: first K tile of X, W tile 0 -> LDS buffer 0, W tile 1 -> registers
+    // ---- prologue: first K tile of X, step 0 of W -> LDS buffer 0, step 1 -> registers
     Frag16 xa[4][MF];          // one K tile (four scale groups) of X in flight
 #pragma unroll
-    for (int j = 0; j < 4; j++) load_x(xa[j], j * 32);
-    WRegs<BITS> wreg[2][WT];   // packed weights: K tile t waits in wreg[t & 1]
+    for (int j = 0; j < 4; j++) load_x(xa[j], kp, j);
+    WRegs<BITS> wreg[2][WT];   // packed weights: step s waits in wreg[s & 1]
     {
         WRegs<BITS> w0[WT];
+        load_units(w0, 0);
+        load_units(wreg[1], 1);
 #pragma unroll
-        for (int t = 0; t < WT; t++) load_wtile<BITS>(w0[t], qp, sp, wtile[t], lane);
-#pragma unroll
-        for (int t = 0; t < WT; t++) load_wtile<BITS>(wreg[1][t], qp, sp, wtile[t] + min(1, KT - 1), lane);
-#pragma unroll
-        for (int t = 0; t < WT; t++)
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-                dequant_group_to_lds<BITS, XBF, EXACT>(w0[t], j, magic, ws + wf[t] * TILE16, lane);
+        for (int j = 0; j < 4; j++) stage_units(w0, 0, j, ws);
     }
     __syncthreads();
 
-    // One K tile.  P = kt & 1 is a compile-time constant (the loop below is unrolled
+    // One step.  P = step & 1 is a compile-time constant (the loop below is unrolled
     // by two), so LDS buffers and register sets alternate without copies or selects:
-    //   multiply from LDS buffer P;  dequantise tile kt+1 (wreg[1-P], requested one
-    //   iteration ago: its HBM latency is behind us) into LDS buffer 1-P;  request
-    //   tile kt+2 into wreg[P].  Past the end indices are clamped: a tile is staged
+    //   multiply from LDS buffer P;  dequantise step+1 (wreg[1-P], requested one
+    //   step ago: its HBM latency is behind us) into LDS buffer 1-P;  request
+    //   step+2 into wreg[P].  Past the end indices are clamped: tiles are staged
     //   again but never read.
-    auto k_tile = [&](int kt, auto parity) {
+    auto k_step = [&](int step, auto parity) {
         constexpr int P = decltype(parity)::value;
-        const u32x4_t* wcur = ws + P * (NF * TILE16);
-        u32x4_t* wnxt = ws + (1 - P) * (NF * TILE16);
-        const int ktn = min(kt + 2, KT - 1);
-#pragma unroll
-        for (int t = 0; t < WT; t++) load_wtile<BITS>(wreg[P][t], qp, sp, wtile[t] + ktn, lane);
+        const u32x4_t* wcur = ws + P * BUF16 + kp * (NF * TILE16);
+        u32x4_t* wnxt = ws + (1 - P) * BUF16;
+        load_units(wreg[P], step + 2);
+        const int kx = (step + 1) * KS + kp;              // this wave's next K tile of X
 
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            Frag16 cv[MF];
-            if (!EXACT && XBF) {
-#pragma unroll
-                for (int i = 0; i < MF; i++) cv[i] = bf16_to_f16_frag(xa[j][i]);
-            }
-            const Frag16 (&a)[MF] = (!EXACT && XBF) ? cv : xa[j];
+            const Frag16 (&a)[MF] = xa[j];
 #pragma unroll
             for (int f = 0; f < NF; f++) {
                 Frag16 b[OPS];
@@ -272,21 +303,37 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF =
             // the same groups of the next K tile.  The two loads of a row hit the
             // two halves of one 128 B line back to back.
             if (j & 1) {
-                load_x(xa[j - 1], (kt + 1) * kTileK + (j - 1) * 32);
-                load_x(xa[j], (kt + 1) * kTileK + j * 32);
+                load_x(xa[j - 1], kx, j - 1);
+                load_x(xa[j], kx, j);
             }
-            // a quarter of the next tile's dequantisation rides along with every group
-            // (a wave whose tile index is clamped rewrites a neighbour's block with
+            // a quarter of the next step's dequantisation rides along with every group
+            // (a wave whose unit index is clamped rewrites a neighbour's block with
             // identical values: no branch in the hot loop)
-#pragma unroll
-            for (int t = 0; t < WT; t++)
-                dequant_group_to_lds<BITS, XBF, EXACT>(wreg[1 - P][t], j, magic, wnxt + wf[t] * TILE16, lane);
+            stage_units(wreg[1 - P], step + 1, j, wnxt);
         }
         __syncthreads();
     };
-    for (int kt = 0; kt < KT; kt += 2) {
-        k_tile(kt, std::integral_constant<int, 0>{});
-        if (kt + 1 < KT) k_tile(kt + 1, std::integral_constant<int, 1>{});
+    for (int s = 0; s < steps; s += 2) {
+        k_step(s, std::integral_constant<int, 0>{});
+        if (s + 1 < steps) k_step(s + 1, std::integral_constant<int, 1>{});
+    }
+
+    // ---- K parts meet: part 1 parks its sums in LDS (all operand reads are behind the
+    // loop's last barrier), part 0 adds them
+    if (KS > 1) {
+        float4_t* park = reinterpret_cast<float4_t*>(smem) + wm * (MF * NF * 64) + lane;
+        if (kp == 1) {
+#pragma unroll
+            for (int i = 0; i < MF; i++)
+#pragma unroll
+                for (int f = 0; f < NF; f++) park[(i * NF + f) * 64] = acc[i][f];
+        }
+        __syncthreads();
+        if (kp != 0) return;
+#pragma unroll
+        for (int i = 0; i < MF; i++)
+#pragma unroll
+            for (int f = 0; f < NF; f++) acc[i][f] += park[(i * NF + f) * 64];
     }
 
     // ---- epilogue
@@ -303,12 +350,15 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF =
         }
 }
 
-template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES>
+template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES, int KS>
 hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, hipStream_t st)
 {
-    constexpr int BM = WAVES * MF * 16;
-    const size_t lds = (size_t)2 * NF * (4 * (EXACT ? 2 : 1) * 64) * 16;     // 56 .. 128 KB
-    auto kern = gemm_kernel<BITS, XBF, NF, EXACT, MF, WAVES>;
+    constexpr int BM = WAVES / KS * MF * 16;
+    // operand buffers: 2 x KS x NF x 4 KB (x 2 for EXACT), 56 .. 128 KB; with KS = 2 the
+    // parked partial sums (MW x MF x NF KB) fit in exactly the same space
+    const size_t lds = (size_t)2 * KS * NF * (4 * (EXACT ? 2 : 1) * 64) * 16;
+    static_assert(KS == 1 || (WAVES / KS) * MF <= 2 * KS * 4 * (EXACT ? 2 : 1), "parked sums must fit in the operand buffers");
+    auto kern = gemm_kernel<BITS, XBF, NF, EXACT, MF, WAVES, KS>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -318,25 +368,29 @@ hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt,
     }
     const int n_tiles = (w.NT + NF - 1) / NF, m_tiles = (M + BM - 1) / BM;
     const unsigned groups = (unsigned)(((int64_t)n_tiles * m_tiles + 7) / 8 * 8);
-    hipLaunchKernelGGL(kern, dim3(groups), dim3(WAVES * 64), lds, st, w, reinterpret_cast<const uint16_t*>(x), M, y, ydt,
-                       n_tiles, m_tiles, out_scale);
+    hipLaunchKernelGGL(kern, dim3(groups), dim3(WAVES * 64), lds, st, w, reinterpret_cast<const u32x4_t*>(x), (M + 15) / 16, M,
+                       y, ydt, n_tiles, m_tiles, out_scale);
     return hipGetLastError();
 }
 
-// Workgroup shapes.
-//   4 waves x 4 row blocks (256 rows): fewest LDS operand reads per MFMA; one wave per SIMD.
-//   8 waves x 2 row blocks (256 rows): two waves per SIMD cover each other's stalls, the tile's
-//       weights are still loaded and dequantised once; every wave reads all B operands, so
-//       LDS reads per MFMA double - fine for FAST (one operand per group), too much for EXACT.
+// Workgroup shapes (all 256 or 128 rows x 16*NF columns).
+//   FAST   8 waves = 4 row groups x 2 K parts, 4 row blocks per wave (256 rows): every B
+//          operand read from LDS feeds 4 MFMAs and two waves share a SIMD.
+//   EXACT  4 waves x 4 row blocks (256 rows), one wave per SIMD: two operands per group
+//          leave no LDS room for a second K part.
 //   4 waves x 2 row blocks (128 rows): twice the tiles, for grids that would leave CUs idle.
 template <int BITS, int XBF, int NF, bool EXACT>
 hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, int num_cus,
                     hipStream_t st)
 {
     const int64_t tiles256 = (int64_t)((w.NT + NF - 1) / NF) * ((M + 255) / 256);
-    if (tiles256 < num_cus) return launch_m<BITS, XBF, NF, EXACT, 2, 4>(w, x, M, y, ydt, out_scale, st);
-    if (!EXACT) return launch_m<BITS, XBF, NF, EXACT, 2, 8>(w, x, M, y, ydt, out_scale, st);
-    return launch_m<BITS, XBF, NF, EXACT, 4, 4>(w, x, M, y, ydt, out_scale, st);
+    if (tiles256 < num_cus) return launch_m<BITS, XBF, NF, EXACT, 2, 4, 1>(w, x, M, y, ydt, out_scale, st);
+    if (!EXACT) {
+        static const char* gv = getenv("CYBQ_GV");
+        if (gv && gv[0] == '1') return launch_m<BITS, XBF, NF, EXACT, 4, 8, 2>(w, x, M, y, ydt, out_scale, st);
+        return launch_m<BITS, XBF, NF, EXACT, 2, 8, 1>(w, x, M, y, ydt, out_scale, st);
+    }
+    return launch_m<BITS, XBF, NF, EXACT, 4, 4, 1>(w, x, M, y, ydt, out_scale, st);
 }
 
 template <int BITS, int XBF>
@@ -353,14 +407,39 @@ hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt
     return launch_t<BITS, XBF, 8, false>(w, x, M, y, ydt, out_scale, num_cus, st);
 }
 
-// bf16 [n] -> f16 [n] scaled by 2^-4 (exact for 2^-10 <= |x| < 2^20); n % 8 == 0
-__global__ void widen_bf16_kernel(const u32x4_t* __restrict__ src, u32x4_t* __restrict__ dst, int64_t n8)
+// X [M, K] row major -> A-operand order: for row block rb (16 rows, zero padded) and
+// scale group g, 64 x 16 B where slot (oct, r) = oct*16 + r holds row 16*rb + r,
+// k = 32*g + 8*oct .. +8.  WIDEN: bf16 -> f16 scaled by 2^-4 on the way (exact for
+// 2^-10 <= |x| < 2^20).  A workgroup moves one row block x 16 groups through LDS:
+// waves read 1 KB runs of a row and write whole 1 KB units.
+constexpr int kStageGroups = 16;                       // scale groups per workgroup
+constexpr int kStagePitch = kStageGroups * 4 + 1;      // 16 B slots per LDS row (odd: no bank conflicts)
+
+template <bool WIDEN>
+__global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict__ src, u32x4_t* __restrict__ dst, int M, int K8)
 {
-    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n8) return;
-    Frag16 a;
-    a.u = src[i];
-    dst[i] = bf16_to_f16_frag(a).u;
+    __shared__ u32x4_t tile[16 * kStagePitch];
+    const int rb = blockIdx.x;
+    const int c0 = blockIdx.y * (kStageGroups * 4);     // first 16 B chunk of the row handled here
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int r = it * 4 + (t >> 6), c = c0 + (t & 63);
+        const int row = rb * 16 + r;
+        Frag16 a;
+        a.u = (u32x4_t){0u, 0u, 0u, 0u};
+        if (row < M && c < K8) a.u = src[(int64_t)row * K8 + c];
+        if (WIDEN) a = bf16_to_f16_frag(a);
+        tile[r * kStagePitch + (t & 63)] = a.u;
+    }
+    __syncthreads();
+    const int G = K8 >> 2;
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int gl = it * 4 + (t >> 6), slot = t & 63;        // group within the workgroup, (oct, r)
+        const int g = blockIdx.y * kStageGroups + gl;
+        if (g < G) dst[((int64_t)rb * G + g) * 64 + slot] = tile[(slot & 15) * kStagePitch + gl * 4 + (slot >> 4)];
+    }
 }
 
 }  // namespace
@@ -369,28 +448,36 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
                        int num_cus, bool exact, void* workspace, size_t workspace_bytes, hipStream_t st)
 {
     if (xdt == kF32) return hipErrorNotSupported;   // api.hip walks fp32 prefill through the decode kernel
-    float out_scale = 1.0f;
-    if (!exact && xdt == kBF16) {
-        out_scale = 16.0f;                          // undoes the 2^-4 prescale of the f16 activations
-        const size_t need = (size_t)M * w.K * 2;
-        if (workspace && need <= workspace_bytes) {
-            // Widen X once instead of in every workgroup (each of the N/112 column
-            // tiles would redo it): one elementwise pass, then the f16 kernel.
-            const int64_t n8 = (int64_t)M * w.K / 8;
-            hipLaunchKernelGGL(widen_bf16_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, st,
-                               reinterpret_cast<const u32x4_t*>(x), reinterpret_cast<u32x4_t*>(workspace), n8);
-            hipError_t e = hipGetLastError();
-            if (e != hipSuccess) return e;
-            x = workspace;
-            xdt = kF16;
+    // FAST multiplies in f16: bf16 activations are widened (2^-4 prescale, undone in the epilogue)
+    const bool widen = !exact && xdt == kBF16;
+    const float out_scale = widen ? 16.0f : 1.0f;
+    const int kdt = widen ? kF16 : xdt;
+    // Rows are staged through the workspace in chunks that fit it; work on one stream is
+    // ordered, so a chunk's multiply is done before the next chunk overwrites the stage.
+    const int64_t row_bytes = (int64_t)w.K * 2;
+    const int64_t max_rows = (int64_t)(workspace_bytes / (size_t)row_bytes) / 256 * 256;
+    if (!workspace || max_rows < 256) return hipErrorOutOfMemory;
+    const size_t ysize = ydt == kF32 ? 4 : 2;
+    for (int64_t m_lo = 0; m_lo < M; m_lo += max_rows) {
+        const int mc = (int)((M - m_lo) < max_rows ? (M - m_lo) : max_rows);
+        const u32x4_t* xs = reinterpret_cast<const u32x4_t*>(static_cast<const char*>(x) + m_lo * row_bytes);
+        void* yc = static_cast<char*>(y) + (size_t)m_lo * w.N * ysize;
+        const int K8 = w.K / 8;
+        const dim3 grid((unsigned)((mc + 15) / 16), (unsigned)((K8 / 4 + kStageGroups - 1) / kStageGroups));
+        if (widen) hipLaunchKernelGGL(stage_x_kernel<true>, grid, dim3(256), 0, st, xs, reinterpret_cast<u32x4_t*>(workspace), mc, K8);
+        else hipLaunchKernelGGL(stage_x_kernel<false>, grid, dim3(256), 0, st, xs, reinterpret_cast<u32x4_t*>(workspace), mc, K8);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        if (w.bits == 4) {
+            e = kdt == kBF16 ? launch_nf<4, 1>(w, workspace, mc, yc, ydt, exact, out_scale, num_cus, st)
+                             : launch_nf<4, 0>(w, workspace, mc, yc, ydt, exact, out_scale, num_cus, st);
+        } else {
+            e = kdt == kBF16 ? launch_nf<8, 1>(w, workspace, mc, yc, ydt, exact, out_scale, num_cus, st)
+                             : launch_nf<8, 0>(w, workspace, mc, yc, ydt, exact, out_scale, num_cus, st);
         }
+        if (e != hipSuccess) return e;
     }
-    if (w.bits == 4) {
-        if (xdt == kBF16) return launch_nf<4, 1>(w, x, M, y, ydt, exact, out_scale, num_cus, st);
-        return launch_nf<4, 0>(w, x, M, y, ydt, exact, out_scale, num_cus, st);
-    }
-    if (xdt == kBF16) return launch_nf<8, 1>(w, x, M, y, ydt, exact, out_scale, num_cus, st);
-    return launch_nf<8, 0>(w, x, M, y, ydt, exact, out_scale, num_cus, st);
+    return hipSuccess;
 }
 
 }  // namespace cybq
