@@ -146,13 +146,13 @@ int cybq_init(int device, cybq_ctx** out)
     if (!ctx) return CYBQ_ERR_NOMEM;
     ctx->device = device;
     ctx->num_cus = prop.multiProcessorCount;
-    // 64 MiB of scratch (f16 copy of up to 2048 x 16384 activations); without it the
-    // prefill kernel converts in registers, so a failed allocation is not an error
-    ctx->workspace_bytes = (size_t)64 << 20;
+    // 256 MiB of scratch for the prefill path: the activations restaged in MFMA operand
+    // order (larger M is walked in row chunks) and the partial sums of a K split
+    ctx->workspace_bytes = (size_t)256 << 20;
     if (hipMalloc(&ctx->workspace, ctx->workspace_bytes) != hipSuccess) {
         (void)hipGetLastError();
-        ctx->workspace = nullptr;
-        ctx->workspace_bytes = 0;
+        delete ctx;
+        return CYBQ_ERR_NOMEM;
     }
     *out = ctx;
     return CYBQ_OK;

@@ -4,10 +4,14 @@
 // its share of the rows (4 or 2 row blocks of 16) against all NF column blocks.
 //
 //   X  never touches LDS.  An MFMA A operand is 16 rows x 32 k with lane l
-//      holding row l%16, k 8*(l/16)..+8 - exactly a 16 B global load per lane -
-//      and every wave consumes only its own rows, so X streams global ->
-//      registers, one K tile (four scale groups) ahead of its use.
-//   W  is shared by the four waves: per K tile (128 k = 4 groups) the NF native
+//      holding row l%16, k 8*(l/16)..+8.  Read straight from a row-major X that is
+//      64 separate 16 B accesses per load (neighbouring lanes are different rows),
+//      which saturates the address path long before the matrix cores.  So a small
+//      kernel first restages X once per call in operand order - row block, scale
+//      group, lane - and the multiply streams it global -> registers with
+//      contiguous 1 KB loads, one K tile (four scale groups) ahead of its use.
+//      The same pass widens bf16 to f16 for FAST mode.
+//   W  is shared by the waves of a workgroup: per K tile (128 k = 4 groups) the NF native
 //      weight tiles are read once with 128-bit loads and dequantised to
 //      w = f32(scale) * q, which is exact in fp32 (11-bit x 4-bit significand).
 //      A 16-bit MFMA operand cannot hold those 15 bits, so w is split without
@@ -27,13 +31,17 @@
 //   FAST   one f16 MFMA per scale group.  The weight operand is round_f16(scale * q)
 //          (one rounding, relative error <= 2^-11, about 2e-4 relative L2 on Y -
 //          inside the operator's 1e-3 tolerance); bf16 activations are widened
-//          to f16 in registers after a 2^-4 prescale that is undone in the
+//          to f16 by the staging pass after a 2^-4 prescale that is undone in the
 //          epilogue, exact for 2^-10 <= |x| < 2^20.
+//
+// Shapes with fewer tiles than CUs split K over workgroups: each split leaves fp32
+// partial sums in its own slab of the workspace and a last kernel adds the slabs in a
+// fixed order, so results are reproducible (no atomics).
 //
 // Out-of-range rows / columns / k are clamped to valid addresses inside the hot
 // loop (their results are never stored, padded weights are zero); the loop has
 // no branches, so the compiler can count outstanding loads exactly.
-#include <cstdlib>
+#include <algorithm>
 #include <type_traits>
 
 #include "cybq_device.h"
@@ -151,47 +159,44 @@ __device__ __forceinline__ Frag16 bf16_to_f16_frag(const Frag16& a)
 }
 
 // XBF = 1: X is bf16, 0: X is f16.  EXACT: see the header comment.
-// WAVES waves form MW = WAVES / KS row groups times KS K parts: wave (wm, kp) owns
-// MF row blocks of 16 against all NF column blocks and multiplies the K tiles
-// kt with kt % KS == kp.  KS = 2 lets two waves share a SIMD (they cover each
-// other's waits) while each still reuses a B operand read from LDS for MF = 4
-// MFMAs; the two partial sums are added once, through LDS, in the epilogue.
-template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES, int KS>
+// Wave wv of WAVES owns MF row blocks of 16 against all NF column blocks.
+template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF * WAVES <= 8 ? 2 : WAVES / 4, MF * WAVES <= 8 ? 2 : WAVES / 4))) void gemm_kernel(WeightView w, const u32x4_t* __restrict__ x, int x_row_blocks, int M,
-                                                   void* __restrict__ y, int ydt, int n_tiles, int m_tiles, float out_scale)
+                                                   void* __restrict__ y, int ydt, int n_tiles, int m_tiles, float out_scale,
+                                                   float* __restrict__ part, int splits, int kt_per_split)
 {
-    static_assert(KS == 1 || KS == 2, "K parts per workgroup");
     // Workgroups are handed to the 8 XCDs round-robin (id % 8) and every XCD has
     // its own L2.  Give each XCD a contiguous run of tiles in row-block-major
     // order, so the workgroups sharing an L2 read the same rows of X and X is
     // fetched into every L2 once instead of once per column tile.
     const int per_xcd = (int)gridDim.x >> 3;
     const int item = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
-    if (item >= n_tiles * m_tiles) return;
-    const int tile_m = item / n_tiles;
-    const int tile_n = item - tile_m * n_tiles;
-    constexpr int MW = WAVES / KS;                    // waves along M
-    constexpr int BM = MW * MF * 16;                  // MF = row blocks (of 16) per wave
-    constexpr int UNITS = KS * NF;                    // weight tiles staged per step
-    constexpr int WT = (UNITS + WAVES - 1) / WAVES;   // ... of which one wave stages WT
+    if (item >= n_tiles * m_tiles * splits) return;
+    // split-major: workgroups that run side by side share a K range of X
+    const int split = item / (n_tiles * m_tiles);
+    const int tile_m = (item - split * (n_tiles * m_tiles)) / n_tiles;
+    const int tile_n = item - (split * m_tiles + tile_m) * n_tiles;
+    constexpr int BM = WAVES * MF * 16;               // MF = row blocks (of 16) per wave
+    constexpr int WT = (NF + WAVES - 1) / WAVES;      // weight tiles a wave stages per K tile
     constexpr int OPS = EXACT ? 2 : 1;                // B operands per scale group
     constexpr int TILE16 = 4 * OPS * 64;              // u32x4 per column block per K tile
-    constexpr int BUF16 = UNITS * TILE16;             // u32x4 per LDS buffer
+    constexpr int BUF16 = NF * TILE16;                // u32x4 per LDS buffer
     constexpr int MMA_BF = EXACT ? XBF : 0;           // FAST always multiplies in f16
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    u32x4_t* ws = reinterpret_cast<u32x4_t*>(smem);   // [2][KS][NF][4][OPS][64]
+    u32x4_t* ws = reinterpret_cast<u32x4_t*>(smem);   // [2][NF][4][OPS][64]
     const uint32_t magic = q4_magic_vgpr();
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int kp = wv / MW, wm = wv - kp * MW;
     const int row16 = lane & 15;
     const int oct = lane >> 4;
     const int nt0 = tile_n * NF;
-    const int m0 = tile_m * BM + wm * (MF * 16);
-    const int K = w.K, KT = w.KT;
-    const int steps = (KT + KS - 1) / KS;
+    const int m0 = tile_m * BM + wv * (MF * 16);
+    const int K = w.K;
+    // this workgroup's K tiles: [kt_lo, kt_lo + KT) of the weight's w.KT (all of them unless K is split)
+    const int kt_lo = split * kt_per_split;
+    const int KT = min(kt_per_split, w.KT - kt_lo);
     // Workgroups that run side by side share rows of X.  Walking K in the same order
     // they would all ask the same few L2 channels for the same lines at the same
     // moment (a row of X is a multiple of the channel interleave long), so each
@@ -200,7 +205,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF *
     const int kt0 = tile_n % KT;
     auto rot = [&](int kt) {
         const int r = min(kt, KT - 1) + kt0;
-        return r >= KT ? r - KT : r;
+        return kt_lo + (r >= KT ? r - KT : r);
     };
 
     const u32x4_t* qp = reinterpret_cast<const u32x4_t*>(w.q);
@@ -222,35 +227,23 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF *
         for (int i = 0; i < MF; i++) dst[i].u = xb[i][g * 64];
     };
 
-    // The weight tiles this wave stages: unit u = wv + WAVES*t (clamped) is column
-    // block u % NF of K part u / NF.  wdst: where its operands go inside a buffer.
+    // The weight tiles this wave stages: column block f = wv + WAVES*t (clamped: a wave
+    // past the end stages a neighbour's block again with identical values, no branch).
     int64_t wtile[WT];
-    int wkp[WT], wdst[WT];
+    int wdst[WT];
 #pragma unroll
     for (int t = 0; t < WT; t++) {
-        const int u = min(wv + WAVES * t, UNITS - 1);
-        wkp[t] = u / NF;
-        wdst[t] = u * TILE16;
-        wtile[t] = (int64_t)min(nt0 + (u - wkp[t] * NF), w.NT - 1) * KT;
+        const int f = min(wv + WAVES * t, NF - 1);
+        wdst[t] = f * TILE16;
+        wtile[t] = (int64_t)min(nt0 + f, w.NT - 1) * w.KT;
     }
-    // K tile of unit t in step s is s*KS + wkp[t]; past KT-1 (only with KS > 1, in the
-    // last step) the last tile is loaded again and its scales are masked to zero,
-    // so the wave that multiplies it adds nothing.
-    auto load_units = [&](WRegs<BITS> (&dst)[WT], int step) {
+    auto load_units = [&](WRegs<BITS> (&dst)[WT], int kt) {
 #pragma unroll
-        for (int t = 0; t < WT; t++)
-            load_wtile<BITS>(dst[t], qp, sp, wtile[t] + rot(step * KS + wkp[t]), lane);
+        for (int t = 0; t < WT; t++) load_wtile<BITS>(dst[t], qp, sp, wtile[t] + rot(kt), lane);
     };
-    auto stage_units = [&](WRegs<BITS> (&src)[WT], int step, int j, u32x4_t* buf) {
+    auto stage_units = [&](WRegs<BITS> (&src)[WT], int j, u32x4_t* buf) {
 #pragma unroll
-        for (int t = 0; t < WT; t++) {
-            if (KS > 1 && j == 0) {
-                const uint32_t keep = (step * KS + wkp[t] < KT) ? 0xffffffffu : 0u;
-                src[t].s[0] &= keep;
-                src[t].s[1] &= keep;
-            }
-            dequant_group_to_lds<BITS, XBF, EXACT>(src[t], j, magic, buf + wdst[t], lane);
-        }
+        for (int t = 0; t < WT; t++) dequant_group_to_lds<BITS, XBF, EXACT>(src[t], j, magic, buf + wdst[t], lane);
     };
 
     float4_t acc[MF][NF];
@@ -259,32 +252,31 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF *
 #pragma unroll
         for (int f = 0; f < NF; f++) acc[i][f] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-    // ---- prologue: first K tile of X, step 0 of W -> LDS buffer 0, step 1 -> registers
+    // ---- prologue: first K tile of X, W tile 0 -> LDS buffer 0, W tile 1 -> registers
     Frag16 xa[4][MF];          // one K tile (four scale groups) of X in flight
 #pragma unroll
-    for (int j = 0; j < 4; j++) load_x(xa[j], kp, j);
-    WRegs<BITS> wreg[2][WT];   // packed weights: step s waits in wreg[s & 1]
+    for (int j = 0; j < 4; j++) load_x(xa[j], 0, j);
+    WRegs<BITS> wreg[2][WT];   // packed weights: K tile t waits in wreg[t & 1]
     {
         WRegs<BITS> w0[WT];
         load_units(w0, 0);
         load_units(wreg[1], 1);
 #pragma unroll
-        for (int j = 0; j < 4; j++) stage_units(w0, 0, j, ws);
+        for (int j = 0; j < 4; j++) stage_units(w0, j, ws);
     }
     __syncthreads();
 
-    // One step.  P = step & 1 is a compile-time constant (the loop below is unrolled
+    // One K tile.  P = kt & 1 is a compile-time constant (the loop below is unrolled
     // by two), so LDS buffers and register sets alternate without copies or selects:
-    //   multiply from LDS buffer P;  dequantise step+1 (wreg[1-P], requested one
-    //   step ago: its HBM latency is behind us) into LDS buffer 1-P;  request
-    //   step+2 into wreg[P].  Past the end indices are clamped: tiles are staged
+    //   multiply from LDS buffer P;  dequantise tile kt+1 (wreg[1-P], requested one
+    //   iteration ago: its HBM latency is behind us) into LDS buffer 1-P;  request
+    //   tile kt+2 into wreg[P].  Past the end indices are clamped: a tile is staged
     //   again but never read.
-    auto k_step = [&](int step, auto parity) {
+    auto k_tile = [&](int kt, auto parity) {
         constexpr int P = decltype(parity)::value;
-        const u32x4_t* wcur = ws + P * BUF16 + kp * (NF * TILE16);
+        const u32x4_t* wcur = ws + P * BUF16;
         u32x4_t* wnxt = ws + (1 - P) * BUF16;
-        load_units(wreg[P], step + 2);
-        const int kx = (step + 1) * KS + kp;              // this wave's next K tile of X
+        load_units(wreg[P], kt + 2);
 
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -300,43 +292,37 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF *
                     for (int i = 0; i < MF; i++) acc[i][f] = mma<MMA_BF>(a[i], b[o], acc[i][f]);
             }
             // After an odd group its pair of operand sets is free: refill both with
-            // the same groups of the next K tile.  The two loads of a row hit the
-            // two halves of one 128 B line back to back.
+            // the same groups of the next K tile.
             if (j & 1) {
-                load_x(xa[j - 1], kx, j - 1);
-                load_x(xa[j], kx, j);
+                load_x(xa[j - 1], kt + 1, j - 1);
+                load_x(xa[j], kt + 1, j);
             }
-            // a quarter of the next step's dequantisation rides along with every group
-            // (a wave whose unit index is clamped rewrites a neighbour's block with
-            // identical values: no branch in the hot loop)
-            stage_units(wreg[1 - P], step + 1, j, wnxt);
+            // a quarter of the next tile's dequantisation rides along with every group
+            stage_units(wreg[1 - P], j, wnxt);
         }
         __syncthreads();
     };
-    for (int s = 0; s < steps; s += 2) {
-        k_step(s, std::integral_constant<int, 0>{});
-        if (s + 1 < steps) k_step(s + 1, std::integral_constant<int, 1>{});
+    for (int kt = 0; kt < KT; kt += 2) {
+        k_tile(kt, std::integral_constant<int, 0>{});
+        if (kt + 1 < KT) k_tile(kt + 1, std::integral_constant<int, 1>{});
     }
 
-    // ---- K parts meet: part 1 parks its sums in LDS (all operand reads are behind the
-    // loop's last barrier), part 0 adds them
-    if (KS > 1) {
-        float4_t* park = reinterpret_cast<float4_t*>(smem) + wm * (MF * NF * 64) + lane;
-        if (kp == 1) {
-#pragma unroll
-            for (int i = 0; i < MF; i++)
-#pragma unroll
-                for (int f = 0; f < NF; f++) park[(i * NF + f) * 64] = acc[i][f];
-        }
-        __syncthreads();
-        if (kp != 0) return;
+    // ---- epilogue: a K split leaves its partial sums in fp32 for splitk_reduce_kernel
+    if (splits > 1) {
+        float* dst = part + (int64_t)split * M * w.N;
 #pragma unroll
         for (int i = 0; i < MF; i++)
 #pragma unroll
-            for (int f = 0; f < NF; f++) acc[i][f] += park[(i * NF + f) * 64];
+            for (int f = 0; f < NF; f++) {
+                const int n = (nt0 + f) * 16 + row16;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int m = m0 + i * 16 + oct * 4 + r;
+                    if (m < M && n < w.N) dst[(int64_t)m * w.N + n] = acc[i][f][r];
+                }
+            }
+        return;
     }
-
-    // ---- epilogue
 #pragma unroll
     for (int i = 0; i < MF; i++)
 #pragma unroll
@@ -350,15 +336,24 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF *
         }
 }
 
-template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES, int KS>
-hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, hipStream_t st)
+// y = out_scale * (part[0] + part[1] + ... + part[splits-1]), added in that order
+__global__ void splitk_reduce_kernel(const float* __restrict__ part, int splits, int64_t total, void* __restrict__ y, int ydt,
+                                     float out_scale)
 {
-    constexpr int BM = WAVES / KS * MF * 16;
-    // operand buffers: 2 x KS x NF x 4 KB (x 2 for EXACT), 56 .. 128 KB; with KS = 2 the
-    // parked partial sums (MW x MF x NF KB) fit in exactly the same space
-    const size_t lds = (size_t)2 * KS * NF * (4 * (EXACT ? 2 : 1) * 64) * 16;
-    static_assert(KS == 1 || (WAVES / KS) * MF <= 2 * KS * 4 * (EXACT ? 2 : 1), "parked sums must fit in the operand buffers");
-    auto kern = gemm_kernel<BITS, XBF, NF, EXACT, MF, WAVES, KS>;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    float v = part[i];
+    for (int s = 1; s < splits; s++) v += part[(int64_t)s * total + i];
+    store_out_g(y, ydt, i, v * out_scale);
+}
+
+template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES>
+hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, float* part,
+                    size_t part_bytes, int num_cus, hipStream_t st)
+{
+    constexpr int BM = WAVES * MF * 16;
+    const size_t lds = (size_t)2 * NF * (4 * (EXACT ? 2 : 1) * 64) * 16;     // operand buffers, 56 .. 128 KB
+    auto kern = gemm_kernel<BITS, XBF, NF, EXACT, MF, WAVES>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -367,44 +362,55 @@ hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt,
         attr_set = true;
     }
     const int n_tiles = (w.NT + NF - 1) / NF, m_tiles = (M + BM - 1) / BM;
-    const unsigned groups = (unsigned)(((int64_t)n_tiles * m_tiles + 7) / 8 * 8);
+    // Too few tiles to fill the chip: split K over workgroups.  Every split adds its
+    // K range in fp32 into its own slab of `part`; a second kernel adds the slabs in
+    // a fixed order (no atomics: results are reproducible).
+    const int64_t tiles = (int64_t)n_tiles * m_tiles;
+    int splits = (int)std::min<int64_t>(8, num_cus / tiles);
+    splits = std::min(splits, w.KT / 4);                         // at least 4 K tiles per split
+    while (splits > 1 && (size_t)splits * M * w.N * 4 > part_bytes) splits--;
+    if (splits < 1) splits = 1;
+    const int kt_per_split = (w.KT + splits - 1) / splits;
+    splits = (w.KT + kt_per_split - 1) / kt_per_split;          // no empty split
+    const unsigned groups = (unsigned)((tiles * splits + 7) / 8 * 8);
     hipLaunchKernelGGL(kern, dim3(groups), dim3(WAVES * 64), lds, st, w, reinterpret_cast<const u32x4_t*>(x), (M + 15) / 16, M,
-                       y, ydt, n_tiles, m_tiles, out_scale);
+                       y, ydt, n_tiles, m_tiles, out_scale, part, splits, kt_per_split);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || splits == 1) return e;
+    const int64_t total = (int64_t)M * w.N;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, part, splits, total, y, ydt,
+                       out_scale);
     return hipGetLastError();
 }
 
-// Workgroup shapes (all 256 or 128 rows x 16*NF columns).
-//   FAST   8 waves = 4 row groups x 2 K parts, 4 row blocks per wave (256 rows): every B
-//          operand read from LDS feeds 4 MFMAs and two waves share a SIMD.
-//   EXACT  4 waves x 4 row blocks (256 rows), one wave per SIMD: two operands per group
-//          leave no LDS room for a second K part.
+// Workgroup shapes.
+//   FAST   8 waves x 2 row blocks (256 rows): two waves per SIMD cover each other's waits and
+//          the tile's weights are dequantised once for all eight.
+//   EXACT  4 waves x 4 row blocks (256 rows), one wave per SIMD: with two operands per group
+//          every LDS read must feed four MFMAs.
 //   4 waves x 2 row blocks (128 rows): twice the tiles, for grids that would leave CUs idle.
 template <int BITS, int XBF, int NF, bool EXACT>
-hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, int num_cus,
-                    hipStream_t st)
+hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, float* part,
+                    size_t part_bytes, int num_cus, hipStream_t st)
 {
     const int64_t tiles256 = (int64_t)((w.NT + NF - 1) / NF) * ((M + 255) / 256);
-    if (tiles256 < num_cus) return launch_m<BITS, XBF, NF, EXACT, 2, 4, 1>(w, x, M, y, ydt, out_scale, st);
-    if (!EXACT) {
-        static const char* gv = getenv("CYBQ_GV");
-        if (gv && gv[0] == '1') return launch_m<BITS, XBF, NF, EXACT, 4, 8, 2>(w, x, M, y, ydt, out_scale, st);
-        return launch_m<BITS, XBF, NF, EXACT, 2, 8, 1>(w, x, M, y, ydt, out_scale, st);
-    }
-    return launch_m<BITS, XBF, NF, EXACT, 4, 4, 1>(w, x, M, y, ydt, out_scale, st);
+    if (tiles256 < num_cus) return launch_m<BITS, XBF, NF, EXACT, 2, 4>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
+    if constexpr (!EXACT) return launch_m<BITS, XBF, NF, EXACT, 2, 8>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
+    else return launch_m<BITS, XBF, NF, EXACT, 4, 4>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
 }
 
 template <int BITS, int XBF>
 hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt, bool exact, float out_scale,
-                     int num_cus, hipStream_t st)
+                     float* part, size_t part_bytes, int num_cus, hipStream_t st)
 {
     // 7 column blocks (BN = 112) tile N = 14336 = 128 * 112 exactly: with M = 512
     // that is 256 workgroups, one per CU; 8 column blocks otherwise
     if (w.NT % 7 == 0) {
-        if (exact) return launch_t<BITS, XBF, 7, true>(w, x, M, y, ydt, out_scale, num_cus, st);
-        return launch_t<BITS, XBF, 7, false>(w, x, M, y, ydt, out_scale, num_cus, st);
+        if (exact) return launch_t<BITS, XBF, 7, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
+        return launch_t<BITS, XBF, 7, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
     }
-    if (exact) return launch_t<BITS, XBF, 8, true>(w, x, M, y, ydt, out_scale, num_cus, st);
-    return launch_t<BITS, XBF, 8, false>(w, x, M, y, ydt, out_scale, num_cus, st);
+    if (exact) return launch_t<BITS, XBF, 8, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
+    return launch_t<BITS, XBF, 8, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
 }
 
 // X [M, K] row major -> A-operand order: for row block rb (16 rows, zero padded) and
@@ -454,8 +460,11 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
     const int kdt = widen ? kF16 : xdt;
     // Rows are staged through the workspace in chunks that fit it; work on one stream is
     // ordered, so a chunk's multiply is done before the next chunk overwrites the stage.
+    // First half of the workspace: staged X; second half: partial sums of a K split.
+    const size_t half = workspace_bytes / 2;
+    float* part = reinterpret_cast<float*>(static_cast<char*>(workspace) + half);
     const int64_t row_bytes = (int64_t)w.K * 2;
-    const int64_t max_rows = (int64_t)(workspace_bytes / (size_t)row_bytes) / 256 * 256;
+    const int64_t max_rows = (int64_t)(half / (size_t)row_bytes) / 256 * 256;
     if (!workspace || max_rows < 256) return hipErrorOutOfMemory;
     const size_t ysize = ydt == kF32 ? 4 : 2;
     for (int64_t m_lo = 0; m_lo < M; m_lo += max_rows) {
@@ -469,11 +478,11 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         if (w.bits == 4) {
-            e = kdt == kBF16 ? launch_nf<4, 1>(w, workspace, mc, yc, ydt, exact, out_scale, num_cus, st)
-                             : launch_nf<4, 0>(w, workspace, mc, yc, ydt, exact, out_scale, num_cus, st);
+            e = kdt == kBF16 ? launch_nf<4, 1>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, st)
+                             : launch_nf<4, 0>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, st);
         } else {
-            e = kdt == kBF16 ? launch_nf<8, 1>(w, workspace, mc, yc, ydt, exact, out_scale, num_cus, st)
-                             : launch_nf<8, 0>(w, workspace, mc, yc, ydt, exact, out_scale, num_cus, st);
+            e = kdt == kBF16 ? launch_nf<8, 1>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, st)
+                             : launch_nf<8, 0>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, st);
         }
         if (e != hipSuccess) return e;
     }

@@ -297,6 +297,45 @@ def test_prefill_rows_agree_with_decode_rows(backend, oracle, prefill_mode):
     assert torch.equal(_run(backend, qw, x), yp)            # deterministic
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("shape", [(200, 4352), (37, 8192 + 96), (500, 2048)])
+def test_prefill_few_tiles_split_k(backend, oracle, prefill_mode, bits, shape):
+    # fewer output tiles than CUs and a long K: the K range is split over workgroups
+    # (K tiles not divisible by the split, ragged N and M) and the partial sums are
+    # added by a second kernel, which also does the output conversion
+    N, K = shape
+    q, s = _quant(oracle, bits, N, K)
+    qw = backend.upload_quantized(q, s, bits)
+    for M in (17, 130, 300):
+        x = _x(M, K, "bf16")
+        y = _run(backend, qw, x)
+        assert not torch.isnan(y).any()
+        err = oracle.rel_l2(y.cpu().numpy(), oracle.matmul_f64(q, s, x.float().cpu().numpy()))
+        assert err < _bar(prefill_mode), (M, err)
+        assert torch.equal(_run(backend, qw, x), y)                       # fixed summation order
+        for ydt in ("f16", "bf16"):
+            assert torch.equal(_run(backend, qw, x, ydt), y.to(TDT[ydt]))   # rounded once
+
+
+def test_prefill_more_rows_than_the_stage_holds(backend, oracle, prefill_mode):
+    # 4200 x 16384 activations are 131 MiB: they pass through the 128 MiB staging area
+    # in two row chunks
+    N, K, M = 48, 16384, 4200
+    q, s = _quant(oracle, 4, N, K)
+    qw = backend.upload_quantized(q, s, 4)
+    x = _x(M, K, "bf16")
+    y = _run(backend, qw, x)
+    assert not torch.isnan(y).any()
+    wd = torch.from_numpy(oracle.dequant(q, s)).cuda().double()
+    full = x.double() @ wd.T
+    for lo, hi in ((0, 1000), (3900, 4096), (4096, M)):                     # rows of both chunks
+        err = ((y[lo:hi].double() - full[lo:hi]).norm() / full[lo:hi].norm()).item()
+        assert err < _bar(prefill_mode), (lo, err)
+    rows = [0, 4095, 4096, M - 1]
+    ref = oracle.matmul_f64(q, s, x[rows].float().cpu().numpy())
+    assert oracle.rel_l2(y[rows].cpu().numpy(), ref) < _bar(prefill_mode)
+
+
 @pytest.mark.parametrize("M", [128, 512])
 @pytest.mark.parametrize("shape", [(4096, 14336), (14336, 4096)])
 def test_config4_full_size(backend, oracle, prefill_mode, M, shape):
