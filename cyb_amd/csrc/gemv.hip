@@ -231,6 +231,23 @@ __device__ __forceinline__ void compute_batch(const TileRegs<BITS> (&buf)[U], in
 // U = tiles a wave keeps in flight per batch.  ONESHOT: the wave's whole share
 // of the strip is at most U tiles, all requested before anything else happens
 // (one register set); otherwise two batches are live and ping-pong.
+// Sum of the waves' partial sums red[k * stride], k = 0 .. nwaves-1, added in wave
+// order.  The reads go out eight at a time: one LDS round trip per eight waves
+// instead of one per wave.  (Slots past nwaves add +0, which changes nothing: a sum
+// that starts from +0 is never -0.)
+__device__ __forceinline__ float sum_partials(const float* red, int nwaves, int stride)
+{
+    float v = 0.f;
+    for (int k0 = 0; k0 < nwaves; k0 += 8) {
+        float t[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) t[i] = red[min(k0 + i, nwaves - 1) * stride];
+#pragma unroll
+        for (int i = 0; i < 8; i++) v += (k0 + i < nwaves) ? t[i] : 0.f;
+    }
+    return v;
+}
+
 template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT>
 __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __restrict__ x, int M, void* __restrict__ y,
                             int ydt, int slab_tiles, int ldx)
@@ -291,21 +308,17 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
         }
     }
 
-    // split-K partials -> LDS, summed in wave order by wave 0
+    // split-K partials -> LDS, summed in wave order; wave r finishes output register r
     __syncthreads();
     float* red = reinterpret_cast<float*>(smem);
 #pragma unroll
     for (int r = 0; r < RMAX; r++) red[(wv * RMAX + r) * 64 + lane] = acc[r];
     __syncthreads();
-    if (wv == 0) {
-        const int n = nt * 16 + (lane & 15);
-#pragma unroll
-        for (int r = 0; r < RMAX; r++) {
-            float v = 0.f;
-            for (int k = 0; k < nwaves; k++) v += red[(k * RMAX + r) * 64 + lane];
-            int m = 4 * oct + r;
-            if (m < M && n < w.N) store_out(y, ydt, (int64_t)m * w.N + n, v);
-        }
+    const int n = nt * 16 + (lane & 15);
+    for (int r = wv; r < RMAX; r += nwaves) {
+        const float v = sum_partials(red + r * 64 + lane, nwaves, RMAX * 64);
+        const int m = 4 * oct + r;
+        if (m < M && n < w.N) store_out(y, ydt, (int64_t)m * w.N + n, v);
     }
 }
 
@@ -358,8 +371,12 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x,
     const int oct = lane >> 4;
     const int strip0 = blockIdx.x * NS;
     const int KT = w.KT;
-    const int kmax = w.K - 8 - oct * 8;
-    const uint16_t* xrow = x + (int64_t)min(lane & 15, M - 1) * w.K + oct * 8;
+    // x is read the way memory likes it - lane l takes 16 B number l%4 of row l/4, so
+    // four neighbouring lanes cover 64 contiguous bytes - and then moved across lanes
+    // into MFMA A-operand order (lane l: row l%16, k octet l/16).  Reading in operand
+    // order directly costs 64 separate accesses per load instead of 16.
+    const uint16_t* xrow = x + (int64_t)min(lane >> 2, M - 1) * w.K + (lane & 3) * 8;
+    const int from_lane = (((lane & 15) << 2) | oct) << 2;       // byte address for ds_bpermute
 
     float acc[NS][4];
 #pragma unroll
@@ -383,7 +400,7 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x,
             kt[u] = min(t, KT - 1);
 #pragma unroll
             for (int j = 0; j < 4; j++)
-                a[u][j].u = *reinterpret_cast<const u32x4_t*>(xrow + min(kt[u] * kTileK + j * 32, kmax));
+                a[u][j].u = *reinterpret_cast<const u32x4_t*>(xrow + min(kt[u] * kTileK + j * 32, w.K - 32));
         }
         // every weight tile of this slab (all strips) is requested before the first
         // one is used: the whole slab is in flight while the wave works through it
@@ -392,6 +409,13 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x,
         for (int s = 0; s < NS; s++)
 #pragma unroll
             for (int u = 0; u < TS; u++) load_tile<BITS>(buf[s][u], w, sbase[s] + kt[u], lane);
+#pragma unroll
+        for (int u = 0; u < TS; u++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int p = 0; p < 4; p++)
+                    a[u][j].u[p] = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane, (int)a[u][j].u[p]);
 #pragma unroll
         for (int s = 0; s < NS; s++) {
             float4_t dprev[4];
@@ -421,17 +445,14 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x,
 #pragma unroll
         for (int r = 0; r < 4; r++) red[((s * nwaves + wv) * 4 + r) * 64 + lane] = acc[s][r];
     __syncthreads();
-    // wave v finishes strips v, v + waves, ...
-    for (int s = wv; s < NS; s += nwaves) {
+    // wave v finishes (strip, output register) pairs v, v + waves, ...
+    for (int p = wv; p < NS * 4; p += nwaves) {
+        const int s = p >> 2, r = p & 3;
         const int nt = strip0 + s;
         const int n = nt * 16 + (lane & 15);
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            float v = 0.f;
-            for (int k = 0; k < nwaves; k++) v += red[((s * nwaves + k) * 4 + r) * 64 + lane];
-            const int m = 4 * oct + r;
-            if (nt < w.NT && m < M && n < w.N) store_out(y, ydt, (int64_t)m * w.N + n, v);
-        }
+        const float v = sum_partials(red + (s * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64);
+        const int m = 4 * oct + r;
+        if (nt < w.NT && m < M && n < w.N) store_out(y, ydt, (int64_t)m * w.N + n, v);
     }
 }
 
