@@ -1,7 +1,7 @@
 // gemm.hip - prefill kernel: Y[M,N] = X[M,K] * W^T for M > 16 on MFMA.
 //
-// Workgroup = 4 or 8 waves, output tile 256 or 128 rows x (16*NF) columns; wave w owns
-// its share of the rows (4 or 2 row blocks of 16) against all NF column blocks.
+// Workgroup = 8 or 4 waves, output tile 256 or 128 rows x (16*NF) columns; wave w owns
+// two row blocks of 16 against all NF column blocks.
 //
 //   X  never touches LDS.  An MFMA A operand is 16 rows x 32 k with lane l
 //      holding row l%16, k 8*(l/16)..+8.  Read straight from a row-major X that is
@@ -161,7 +161,7 @@ __device__ __forceinline__ Frag16 bf16_to_f16_frag(const Frag16& a)
 // XBF = 1: X is bf16, 0: X is f16.  EXACT: see the header comment.
 // Wave wv of WAVES owns MF row blocks of 16 against all NF column blocks.
 template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF * WAVES <= 8 ? 2 : WAVES / 4, MF * WAVES <= 8 ? 2 : WAVES / 4))) void gemm_kernel(WeightView w, const u32x4_t* __restrict__ x, int x_row_blocks, int M,
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kernel(WeightView w, const u32x4_t* __restrict__ x, int x_row_blocks, int M,
                                                    void* __restrict__ y, int ydt, int n_tiles, int m_tiles, float out_scale,
                                                    float* __restrict__ part, int splits, int kt_per_split)
 {
@@ -252,31 +252,38 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF *
 #pragma unroll
         for (int f = 0; f < NF; f++) acc[i][f] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-    // ---- prologue: first K tile of X, W tile 0 -> LDS buffer 0, W tile 1 -> registers
+    // ---- prologue: first K tile of X, W tile 0 -> LDS buffer 0, W tiles 1 .. SETS-1 -> registers
     Frag16 xa[4][MF];          // one K tile (four scale groups) of X in flight
 #pragma unroll
     for (int j = 0; j < 4; j++) load_x(xa[j], 0, j);
-    WRegs<BITS> wreg[2][WT];   // packed weights: K tile t waits in wreg[t & 1]
+    // Packed weights wait in registers: K tile t sits in wreg[t % SETS], requested SETS - 1
+    // iterations before it is dequantised.  Loads retire in order and every iteration
+    // also requests X, so two sets leave a weight tile one iteration (about 2 us) to
+    // arrive - enough from cache, short for a first touch in HBM; Q4 FAST has the
+    // registers for four.
+    constexpr int SETS = (BITS == 4 && !EXACT) ? 4 : 2;
+    WRegs<BITS> wreg[SETS][WT];
     {
         WRegs<BITS> w0[WT];
         load_units(w0, 0);
-        load_units(wreg[1], 1);
+#pragma unroll
+        for (int t = 1; t < SETS; t++) load_units(wreg[t], t);
 #pragma unroll
         for (int j = 0; j < 4; j++) stage_units(w0, j, ws);
     }
     __syncthreads();
 
-    // One K tile.  P = kt & 1 is a compile-time constant (the loop below is unrolled
-    // by two), so LDS buffers and register sets alternate without copies or selects:
-    //   multiply from LDS buffer P;  dequantise tile kt+1 (wreg[1-P], requested one
-    //   iteration ago: its HBM latency is behind us) into LDS buffer 1-P;  request
-    //   tile kt+2 into wreg[P].  Past the end indices are clamped: a tile is staged
-    //   again but never read.
-    auto k_tile = [&](int kt, auto parity) {
-        constexpr int P = decltype(parity)::value;
+    // One K tile.  R = kt % SETS is a compile-time constant (the loop below is unrolled
+    // SETS times), so LDS buffers (R & 1) and register sets alternate without copies
+    // or selects:  multiply from LDS buffer R & 1;  dequantise tile kt+1 from its
+    // register set into the other buffer;  request tile kt+SETS into the set tile kt
+    // left free.  Past the end indices are clamped: a tile is staged again but never read.
+    auto k_tile = [&](int kt, auto residue) {
+        constexpr int R = decltype(residue)::value;
+        constexpr int P = R & 1;
         const u32x4_t* wcur = ws + P * BUF16;
         u32x4_t* wnxt = ws + (1 - P) * BUF16;
-        load_units(wreg[P], kt + 2);
+        load_units(wreg[R], kt + SETS);
 
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -298,13 +305,17 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MF *
                 load_x(xa[j], kt + 1, j);
             }
             // a quarter of the next tile's dequantisation rides along with every group
-            stage_units(wreg[1 - P], j, wnxt);
+            stage_units(wreg[(R + 1) % SETS], j, wnxt);
         }
         __syncthreads();
     };
-    for (int kt = 0; kt < KT; kt += 2) {
+    for (int kt = 0; kt < KT; kt += SETS) {
         k_tile(kt, std::integral_constant<int, 0>{});
         if (kt + 1 < KT) k_tile(kt + 1, std::integral_constant<int, 1>{});
+        if constexpr (SETS == 4) {
+            if (kt + 2 < KT) k_tile(kt + 2, std::integral_constant<int, 2>{});
+            if (kt + 3 < KT) k_tile(kt + 3, std::integral_constant<int, 3>{});
+        }
     }
 
     // ---- epilogue: a K split leaves its partial sums in fp32 for splitk_reduce_kernel
@@ -383,20 +394,18 @@ hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt,
     return hipGetLastError();
 }
 
-// Workgroup shapes.
-//   FAST   8 waves x 2 row blocks (256 rows): two waves per SIMD cover each other's waits and
-//          the tile's weights are dequantised once for all eight.
-//   EXACT  4 waves x 4 row blocks (256 rows), one wave per SIMD: with two operands per group
-//          every LDS read must feed four MFMAs.
-//   4 waves x 2 row blocks (128 rows): twice the tiles, for grids that would leave CUs idle.
+// Workgroup shapes: every wave owns 2 row blocks.
+//   8 waves (256 rows): two waves per SIMD cover each other's waits and the tile's
+//       weights are dequantised once for all eight.
+//   4 waves (128 rows), two workgroups per CU: twice the tiles, for grids that would
+//       leave CUs idle.
 template <int BITS, int XBF, int NF, bool EXACT>
 hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, float* part,
                     size_t part_bytes, int num_cus, hipStream_t st)
 {
     const int64_t tiles256 = (int64_t)((w.NT + NF - 1) / NF) * ((M + 255) / 256);
     if (tiles256 < num_cus) return launch_m<BITS, XBF, NF, EXACT, 2, 4>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
-    if constexpr (!EXACT) return launch_m<BITS, XBF, NF, EXACT, 2, 8>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
-    else return launch_m<BITS, XBF, NF, EXACT, 4, 4>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
+    return launch_m<BITS, XBF, NF, EXACT, 2, 8>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
 }
 
 template <int BITS, int XBF>
@@ -405,12 +414,16 @@ hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt
 {
     // 7 column blocks (BN = 112) tile N = 14336 = 128 * 112 exactly: with M = 512
     // that is 256 workgroups, one per CU; 8 column blocks otherwise
-    if (w.NT % 7 == 0) {
-        if (exact) return launch_t<BITS, XBF, 7, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
-        return launch_t<BITS, XBF, 7, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
+    const bool nf7 = w.NT % 7 == 0;
+    if (exact) {
+        if (nf7) return launch_t<BITS, XBF, 7, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
+        return launch_t<BITS, XBF, 8, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
     }
-    if (exact) return launch_t<BITS, XBF, 8, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
-    return launch_t<BITS, XBF, 8, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
+    if constexpr (XBF == 0) {       // FAST multiplies in f16: bf16 activations were widened by the staging pass
+        if (nf7) return launch_t<BITS, 0, 7, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
+        return launch_t<BITS, 0, 8, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
+    }
+    return hipErrorInvalidValue;
 }
 
 // X [M, K] row major -> A-operand order: for row block rb (16 rows, zero padded) and
