@@ -228,9 +228,6 @@ __device__ __forceinline__ void compute_batch(const TileRegs<BITS> (&buf)[U], in
     tile_accum<RMAX>(sprev, dprev, acc);
 }
 
-// U = tiles a wave keeps in flight per batch.  ONESHOT: the wave's whole share
-// of the strip is at most U tiles, all requested before anything else happens
-// (one register set); otherwise two batches are live and ping-pong.
 // Sum of the waves' partial sums red[k * stride], k = 0 .. nwaves-1, added in wave
 // order.  The reads go out eight at a time: one LDS round trip per eight waves
 // instead of one per wave.  (Slots past nwaves add +0, which changes nothing: a sum
@@ -248,6 +245,9 @@ __device__ __forceinline__ float sum_partials(const float* red, int nwaves, int 
     return v;
 }
 
+// U = tiles a wave keeps in flight per batch.  ONESHOT: the wave's whole share
+// of the strip is at most U tiles, all requested before anything else happens
+// (one register set); otherwise two batches are live and ping-pong.
 template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT>
 __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __restrict__ x, int M, void* __restrict__ y,
                             int ydt, int slab_tiles, int ldx)
