@@ -28,8 +28,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 MALL_BYTES = 256 << 20
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain
 # 256 MiB copy: FETCH x 1.9997, WRITE x 1.0000); profiles/decode_gemv_q4_4096x14336_m1.md
-TRAFFIC_DECODE_BYTES = 33_275_300
-TRAFFIC_PREFILL_M512_BYTES = 170_381_000
+TRAFFIC_DECODE_BYTES = 33_280_700
+TRAFFIC_PREFILL_M512_BYTES = 121_787_300     # multiply 113.4 MB + activation staging pass 8.4 MB
 
 
 def log(*a):
@@ -244,6 +244,28 @@ def main():
                                  "frac_of_hbm_peak": round(st.step_bytes(Ms) / per / 1e9 / HBM_PEAK_GBS, 4),
                                  "linear_stack_tok_per_s": round(Ms / per, 1)}
                 log(f"decode stack {label} M={Ms}: {per * 1e6:.0f} us/step")
+            if shapes is not None:
+                # prefill of one 512-token chunk through the same stack (bf16 activations), and both
+                # phases in the units the reference's UI reports (tok_in_s / tok_out_s,
+                # /root/reference/shell/src/worlds/models/mod.rs:44-52): linears only, no attention
+                Mp2 = 512
+                edges = stk.edges_for(st, Mp2, shapes=shapes, xdtype=torch.bfloat16)
+                pl = stk.plan(st, edges)
+                be.matmul_many(pl, Mp2, stream)
+                torch.cuda.synchronize()
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                for _ in range(3):
+                    be.matmul_many(pl, Mp2, stream)
+                b.record()
+                torch.cuda.synchronize()
+                per = a.elapsed_time(b) * 1e-3 / 3
+                flops = sum(2.0 * Mp2 * w.N * w.K for w in st.weights)
+                res["prefill_M512"] = {"ms_per_chunk": round(per * 1e3, 3), "TFLOP/s": round(flops / per / 1e12, 1),
+                                       "frac_of_mfma_peak": round(flops / per / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+                res["linear_stack_tok_in_s"] = round(Mp2 / per, 1)
+                res["linear_stack_tok_out_s"] = res["M1"]["linear_stack_tok_per_s"]
+                log(f"prefill stack {label} M={Mp2}: {per * 1e3:.2f} ms/chunk, {flops / per / 1e12:.0f} TFLOP/s")
             stack_out[label] = res
             for t in st.weights:
                 t.free()

@@ -88,13 +88,14 @@ def build(backend: Backend, layers: int = 32, bits: int = formats.Q4, seed: int 
     return st
 
 
-def edges_for(stack: LinearStack, M: int, seed: int = 5, shapes: Dict[str, tuple] = None):
-    """Fresh seeded f16 inputs (one per input width) and f32 outputs (one per linear kind)."""
+def edges_for(stack: LinearStack, M: int, seed: int = 5, shapes: Dict[str, tuple] = None, xdtype=None):
+    """Fresh seeded inputs (one per input width; f16 unless `xdtype` says otherwise) and f32
+    outputs (one per linear kind)."""
     import torch
     shapes = shapes or synth.LLAMA3_8B_LINEARS
     edges = {}
     for i, K in enumerate(sorted({k for k, _ in shapes.values()})):
-        x = torch.from_numpy(synth.activations(seed, M, K, stream=i)).cuda().to(torch.float16)
+        x = torch.from_numpy(synth.activations(seed, M, K, stream=i)).cuda().to(xdtype or torch.float16)
         edges[f"in.{K}"] = x
     for lin in shapes:
         edges[f"out.{lin}"] = torch.empty((M, shapes[lin][1]), dtype=torch.float32, device="cuda")
