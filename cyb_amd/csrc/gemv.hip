@@ -69,7 +69,8 @@ struct XRegs {
     u32x4_t v[kXChunks][XMODE == XF32 ? 2 : 1];
 };
 
-template <int XMODE>
+// ONEROW (M == 1): chunk index = column, no division on the way to the first load.
+template <int XMODE, bool ONEROW>
 __device__ __forceinline__ void stage_x_load(XRegs<XMODE>& r, const void* x, int M, int K, int k_begin,
                                              int slab_k, int first_chunk, int tid, int nthreads)
 {
@@ -78,7 +79,7 @@ __device__ __forceinline__ void stage_x_load(XRegs<XMODE>& r, const void* x, int
 #pragma unroll
     for (int c = 0; c < kXChunks; c++) {
         const int idx = first_chunk + tid + c * nthreads;
-        const int row = idx / chunks_per_row;
+        const int row = ONEROW ? 0 : idx / chunks_per_row;
         const int k = k_begin + ((idx - row * chunks_per_row) << 3);
         const bool live = idx < total && k < K;
         if (XMODE != XF32) {
@@ -98,7 +99,7 @@ __device__ __forceinline__ void stage_x_load(XRegs<XMODE>& r, const void* x, int
     }
 }
 
-template <int XMODE>
+template <int XMODE, bool ONEROW>
 __device__ __forceinline__ void stage_x_store(const XRegs<XMODE>& r, uint16_t* xs, int M, int slab_k, int ldx,
                                               int plane_elems, int first_chunk, int tid, int nthreads)
 {
@@ -108,7 +109,7 @@ __device__ __forceinline__ void stage_x_store(const XRegs<XMODE>& r, uint16_t* x
     for (int c = 0; c < kXChunks; c++) {
         const int idx = first_chunk + tid + c * nthreads;
         if (idx >= total) continue;
-        const int row = idx / chunks_per_row;
+        const int row = ONEROW ? 0 : idx / chunks_per_row;
         const int col = (idx - row * chunks_per_row) << 3;
         u32x4_t* dst = reinterpret_cast<u32x4_t*>(xs + row * ldx + col);
         if (XMODE != XF32) {
@@ -129,15 +130,15 @@ __device__ __forceinline__ void stage_x_store(const XRegs<XMODE>& r, uint16_t* x
 }
 
 // chunks beyond the first kXChunks per thread (large M * slab): plain loop
-template <int XMODE>
+template <int XMODE, bool ONEROW>
 __device__ __forceinline__ void stage_x_rest(uint16_t* xs, const void* x, int M, int K, int k_begin, int slab_k,
                                              int ldx, int plane_elems, int tid, int nthreads)
 {
     const int total = M * (slab_k >> 3);
     for (int first = kXChunks * nthreads; first < total; first += kXChunks * nthreads) {
         XRegs<XMODE> r;
-        stage_x_load<XMODE>(r, x, M, K, k_begin, slab_k, first, tid, nthreads);
-        stage_x_store<XMODE>(r, xs, M, slab_k, ldx, plane_elems, first, tid, nthreads);
+        stage_x_load<XMODE, ONEROW>(r, x, M, K, k_begin, slab_k, first, tid, nthreads);
+        stage_x_store<XMODE, ONEROW>(r, xs, M, slab_k, ldx, plane_elems, first, tid, nthreads);
     }
 }
 
@@ -250,7 +251,7 @@ __device__ __forceinline__ float sum_partials(const float* red, int nwaves, int 
 // (one register set); otherwise two batches are live and ping-pong.
 template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT>
 __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __restrict__ x, int M, void* __restrict__ y,
-                            int ydt, int slab_tiles, int ldx)
+                            int ydt, int slab_tiles, int ldx, int red_offset)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t* xs = reinterpret_cast<uint16_t*>(smem);
@@ -275,10 +276,10 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
     if (ONESHOT) {
         TileRegs<BITS> buf[U];
         XRegs<XMODE> xr;
-        stage_x_rest<XMODE>(xs, x, M, w.K, 0, w.KT * kTileK, ldx, plane_elems, tid, nthreads);
-        stage_x_load<XMODE>(xr, x, M, w.K, 0, w.KT * kTileK, 0, tid, nthreads);
+        stage_x_rest<XMODE, RMAX == 1>(xs, x, M, w.K, 0, w.KT * kTileK, ldx, plane_elems, tid, nthreads);
+        stage_x_load<XMODE, RMAX == 1>(xr, x, M, w.K, 0, w.KT * kTileK, 0, tid, nthreads);
         load_batch<BITS, U>(buf, w, strip, wv, nwaves, w.KT, lane);
-        stage_x_store<XMODE>(xr, xs, M, w.KT * kTileK, ldx, plane_elems, 0, tid, nthreads);
+        stage_x_store<XMODE, RMAX == 1>(xr, xs, M, w.KT * kTileK, ldx, plane_elems, 0, tid, nthreads);
         __syncthreads();
         const uint16_t* xbase = xs + mrow * ldx + oct * 8;
         compute_batch<BITS, XMODE, RMAX, U>(buf, wv, nwaves, w.KT, xbase, plane_elems, magic, acc);
@@ -291,10 +292,10 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
             // x loads first, then the first weight batch of this slab: the HBM
             // latency of the weights overlaps the staging and the barrier
             XRegs<XMODE> xr;
-            stage_x_rest<XMODE>(xs, x, M, w.K, slab0 * kTileK, st * kTileK, ldx, plane_elems, tid, nthreads);
-            stage_x_load<XMODE>(xr, x, M, w.K, slab0 * kTileK, st * kTileK, 0, tid, nthreads);
+            stage_x_rest<XMODE, RMAX == 1>(xs, x, M, w.K, slab0 * kTileK, st * kTileK, ldx, plane_elems, tid, nthreads);
+            stage_x_load<XMODE, RMAX == 1>(xr, x, M, w.K, slab0 * kTileK, st * kTileK, 0, tid, nthreads);
             load_batch<BITS, U>(bufA, w, base, wv, nwaves, st, lane);
-            stage_x_store<XMODE>(xr, xs, M, st * kTileK, ldx, plane_elems, 0, tid, nthreads);
+            stage_x_store<XMODE, RMAX == 1>(xr, xs, M, st * kTileK, ldx, plane_elems, 0, tid, nthreads);
             __syncthreads();
 
             const uint16_t* xbase = xs + mrow * ldx + oct * 8;
@@ -308,9 +309,9 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
         }
     }
 
-    // split-K partials -> LDS, summed in wave order; wave r finishes output register r
-    __syncthreads();
-    float* red = reinterpret_cast<float*>(smem);
+    // split-K partials -> LDS (their own area behind x: no barrier to wait for the last
+    // reader of x), summed in wave order; wave r finishes output register r
+    float* red = reinterpret_cast<float*>(smem + red_offset);
 #pragma unroll
     for (int r = 0; r < RMAX; r++) red[(wv * RMAX + r) * 64 + lane] = acc[r];
     __syncthreads();
@@ -510,19 +511,18 @@ hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt,
         if (slab_tiles < nwaves) slab_tiles = nwaves;
     }
     int ldx = slab_tiles * kTileK + 8;
-    size_t lds = (size_t)M * ldx * 2 * planes;
-    size_t red = (size_t)nwaves * RMAX * 64 * sizeof(float);
-    if (lds < red) lds = red;
+    const size_t xbytes = ((size_t)M * ldx * 2 * planes + 255) & ~(size_t)255;
+    const size_t lds = xbytes + (size_t)nwaves * RMAX * 64 * sizeof(float);     // x, then the waves' partial sums
     auto kern = gemv_kernel<BITS, XMODE, RMAX, U, ONESHOT>;
     static bool attr_set = false;
     if (!attr_set) {
         // M = 16 fp32 activations with 8 waves need 66 KB, just over the default cap
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    hipLaunchKernelGGL(kern, dim3(w.NT), dim3(nwaves * 64), lds, st, w, x, M, y, ydt, slab_tiles, ldx);
+    hipLaunchKernelGGL(kern, dim3(w.NT), dim3(nwaves * 64), lds, st, w, x, M, y, ydt, slab_tiles, ldx, (int)xbytes);
     return hipGetLastError();
 }
 
