@@ -221,9 +221,11 @@ def main():
         del ws[1:]
         from cyb_amd import stack as stk
         stack_out = {}
-        for label, shapes in (("per_linear_224_launches", None), ("qkv_and_gate_up_fused_128_launches", stk.fused_shapes())):
+        for label, shapes, epis in (("per_linear_224_launches", None, False),
+                                    ("qkv_and_gate_up_fused_128_launches", stk.fused_shapes(), False),
+                                    ("fused_128_launches_swiglu_and_residual_epilogues", stk.fused_shapes(), True)):
             t0 = time.time()
-            st = stk.build(be, layers=32, seed=5, shapes=shapes, order=list(shapes) if shapes else None)
+            st = stk.build(be, layers=32, seed=5, shapes=shapes, order=list(shapes) if shapes else None, epilogues=epis)
             log(f"stack {label} built in {time.time() - t0:.1f}s: {st.weight_bytes} weight bytes")
             res = {"weight_bytes": int(st.weight_bytes), "launches_per_step": len(st.nodes)}
             for Ms in (1, 8):
@@ -244,7 +246,7 @@ def main():
                                  "frac_of_hbm_peak": round(st.step_bytes(Ms) / per / 1e9 / HBM_PEAK_GBS, 4),
                                  "linear_stack_tok_per_s": round(Ms / per, 1)}
                 log(f"decode stack {label} M={Ms}: {per * 1e6:.0f} us/step")
-            if shapes is not None:
+            if shapes is not None and not epis:
                 # prefill of one 512-token chunk through the same stack (bf16 activations), and both
                 # phases in the units the reference's UI reports (tok_in_s / tok_out_s,
                 # /root/reference/shell/src/worlds/models/mod.rs:44-52): linears only, no attention

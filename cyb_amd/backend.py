@@ -32,6 +32,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "lib", "libcybq.so")
 
 F32, F16, BF16 = 0, 1, 2
+EPILOGUES = {"none": 0, "add": 1, "swiglu": 2}      # enum cybq_epilogue
 _DTYPE_CODES = {"torch.float32": F32, "torch.float16": F16, "torch.bfloat16": BF16,
                 "float32": F32, "float16": F16}
 _ITEMSIZE = {F32: 4, F16: 2, BF16: 2}
@@ -77,6 +78,9 @@ def load_library() -> ctypes.CDLL:
     lib.cybq_weight_info.argtypes = [vp, ctypes.POINTER(ci), ctypes.POINTER(i64), ctypes.POINTER(i64),
                                      ctypes.POINTER(i64)]
     lib.cybq_matmul.argtypes = [vp, vp, vp, ci, i64, vp, ci, vp]
+    lib.cybq_matmul_ex.argtypes = [vp, vp, vp, ci, i64, vp, ci, ci, vp, vp]
+    lib.cybq_weight_fuse_pairs.argtypes = [vp, vp, vp, ctypes.POINTER(vp)]
+    lib.cybq_matmul_many_ex.argtypes = [vp, i64, vp, vp, vp, vp, vp, ci, i64, ci, vp]
     lib.cybq_set_prefill_mode.argtypes = [vp, ci]
     lib.cybq_matmul_many.argtypes = [vp, i64, vp, vp, vp, ci, i64, ci, vp]
     lib.cybq_dequant.argtypes = [vp, vp, vp, vp]
@@ -162,18 +166,24 @@ class QWeight:
 class MatmulPlan:
     """Pointer arrays of a fixed node list (one decode step's linears)."""
 
-    def __init__(self, backend: "Backend", weights, xs, ys):
+    def __init__(self, backend: "Backend", weights, xs, ys, epilogues=None, residuals=None):
         n = len(weights)
         if not (n == len(xs) == len(ys)):
             raise CybqError(-1, "invalid argument", "weights / xs / ys differ in length")
         self.count = n
-        self.keep = (list(weights), list(xs), list(ys))      # keeps tensors and handles alive
+        self.keep = (list(weights), list(xs), list(ys), list(residuals or []))      # keeps tensors and handles alive
         arr = ctypes.c_void_p * n
         self.w = arr(*[w.handle.value for w in weights])
         self.x = arr(*[_ptr(t) for t in xs])
         self.y = arr(*[_ptr(t) for t in ys])
         self.xdt = _dtype_code(xs[0], None) if n else F16
         self.ydt = _dtype_code(ys[0], None) if n else F32
+        self.epi = self.res = None
+        if epilogues is not None:
+            if len(epilogues) != n or (residuals is not None and len(residuals) != n):
+                raise CybqError(-1, "invalid argument", "epilogues / residuals differ in length from the node list")
+            self.epi = (ctypes.c_int * n)(*[EPILOGUES[e] for e in epilogues])
+            self.res = arr(*[_ptr(r) for r in (residuals or [None] * n)])
 
 
 class Backend:
@@ -256,11 +266,35 @@ class Backend:
         self._check(self._lib.cybq_matmul(self._ctx, w.handle, _ptr(x), _dtype_code(x, xdt), M, _ptr(y),
                                           _dtype_code(y, ydt), stream))
 
-    def plan_many(self, weights, xs, ys) -> "MatmulPlan":
-        """Freezes a list of (weight, x, y) nodes into pointer arrays for matmul_many."""
-        return MatmulPlan(self, weights, xs, ys)
+    def matmul_ex(self, w: QWeight, x, y, epilogue: str = "none", residual=None, M: Optional[int] = None,
+                  stream: int = 0) -> None:
+        """cybq_matmul_ex: epilogue "none", "add" (y = residual + x W^T) or "swiglu" (w from
+        fuse_pairs; y has half as many columns as w has rows)."""
+        if epilogue not in EPILOGUES:
+            raise CybqError(-1, "invalid argument", f"unknown epilogue {epilogue!r}")
+        if M is None:
+            M = int(x.shape[0]) if x.dim() == 2 else 1
+        self._check(self._lib.cybq_matmul_ex(self._ctx, w.handle, _ptr(x), _dtype_code(x, None), M, _ptr(y),
+                                             _dtype_code(y, None), EPILOGUES[epilogue], _ptr(residual), stream))
+
+    def fuse_pairs(self, gate: QWeight, up: QWeight, name: Optional[str] = None) -> QWeight:
+        """One weight holding gate and up projections interleaved by 16-row strip (device to device)."""
+        out = ctypes.c_void_p()
+        self._check(self._lib.cybq_weight_fuse_pairs(self._ctx, gate.handle, up.handle, ctypes.byref(out)))
+        w = QWeight(self, out.value)
+        if name is not None:
+            self.weights[name] = w
+        return w
+
+    def plan_many(self, weights, xs, ys, epilogues=None, residuals=None) -> "MatmulPlan":
+        """Freezes a list of (weight, x, y[, epilogue, residual]) nodes into pointer arrays for matmul_many."""
+        return MatmulPlan(self, weights, xs, ys, epilogues, residuals)
 
     def matmul_many(self, plan: "MatmulPlan", M: int, stream: int = 0) -> None:
+        if plan.epi is not None:
+            self._check(self._lib.cybq_matmul_many_ex(self._ctx, plan.count, plan.w, plan.x, plan.y, plan.epi, plan.res,
+                                                      plan.xdt, M, plan.ydt, stream))
+            return
         self._check(self._lib.cybq_matmul_many(self._ctx, plan.count, plan.w, plan.x, plan.y, plan.xdt, M,
                                                plan.ydt, stream))
 

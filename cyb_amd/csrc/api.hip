@@ -28,6 +28,7 @@ struct cybq_weight {
     uint32_t* q = nullptr;
     uint16_t* s = nullptr;
     size_t q_bytes = 0, s_bytes = 0;
+    bool paired = false;                // made by cybq_weight_fuse_pairs: strips alternate gate / up
 };
 
 namespace {
@@ -264,6 +265,7 @@ int cybq_weight_clone(cybq_ctx* ctx, const cybq_weight* src, cybq_weight** out)
         delete w;
         return fail_hip(ctx, e, "weight clone");
     }
+    w->paired = src->paired;
     *out = w;
     return CYBQ_OK;
 }
@@ -290,8 +292,8 @@ int cybq_weight_info(const cybq_weight* w, int* quant, int64_t* N, int64_t* K, i
     return CYBQ_OK;
 }
 
-int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M, void* y,
-                cybq_dtype ydt, void* stream)
+int cybq_matmul_ex(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M, void* y,
+                   cybq_dtype ydt, cybq_epilogue epilogue, const void* residual, void* stream)
 {
     if (!ctx) return CYBQ_ERR_INVALID;
     if (!w || !x || !y) return fail(ctx, CYBQ_ERR_INVALID, "w / x / y is NULL");
@@ -300,15 +302,28 @@ int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype x
     if (w->device != ctx->device) return fail(ctx, CYBQ_ERR_INVALID, "weight lives on another device");
     if (!aligned16(x)) return fail(ctx, CYBQ_ERR_ALIGN, "x must be 16-byte aligned");
     if (reinterpret_cast<uintptr_t>(y) % dtype_size(ydt)) return fail(ctx, CYBQ_ERR_ALIGN, "y is not aligned to its element size");
+    cybq::Epilogue epi = {cybq::kEpiNone, nullptr};
+    if (epilogue == CYBQ_EPI_ADD) {
+        if (!residual) return fail(ctx, CYBQ_ERR_INVALID, "CYBQ_EPI_ADD needs a residual");
+        if (reinterpret_cast<uintptr_t>(residual) % dtype_size(ydt)) return fail(ctx, CYBQ_ERR_ALIGN, "residual is not aligned to its element size");
+        epi = {cybq::kEpiAdd, residual};
+    } else if (epilogue == CYBQ_EPI_SWIGLU) {
+        if (!w->paired) return fail(ctx, CYBQ_ERR_INVALID, "CYBQ_EPI_SWIGLU needs a weight made by cybq_weight_fuse_pairs");
+        if (xdt == CYBQ_F32 && M > 16) return fail(ctx, CYBQ_ERR_INVALID, "CYBQ_EPI_SWIGLU with fp32 activations is limited to M <= 16");
+        epi = {cybq::kEpiSwiglu, nullptr};
+    } else if (epilogue != CYBQ_EPI_NONE) {
+        return fail(ctx, CYBQ_ERR_INVALID, "unknown epilogue");
+    }
     DeviceGuard guard(ctx->device);
     if (guard.err != hipSuccess) return fail_hip(ctx, guard.err, "hipSetDevice");
     hipStream_t st = static_cast<hipStream_t>(stream);
     cybq::WeightView v = view_of(w);
     hipError_t e;
     if (M <= 16) {
-        e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, st);
+        e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, epi, st);
     } else if (xdt != CYBQ_F32) {
-        e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, ctx->workspace, ctx->workspace_bytes, st);
+        e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, ctx->workspace, ctx->workspace_bytes,
+                              epi, st);
     } else {
         // fp32 activations keep full precision through the decode kernel's
         // hi/lo split; prefill in fp32 is walked 16 rows at a time.
@@ -316,11 +331,51 @@ int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype x
         for (int64_t m0 = 0; m0 < M && e == hipSuccess; m0 += 16) {
             int mm = (int)((M - m0) < 16 ? (M - m0) : 16);
             const char* xp = static_cast<const char*>(x) + (size_t)m0 * w->K * 4;
-            char* yp = static_cast<char*>(y) + (size_t)m0 * w->N * dtype_size(ydt);
-            e = cybq::launch_gemv(v, xp, xdt, mm, yp, ydt, ctx->num_cus, st);
+            const size_t yoff = (size_t)m0 * w->N * dtype_size(ydt);
+            cybq::Epilogue ec = epi;
+            if (epi.kind == cybq::kEpiAdd) ec.residual = static_cast<const char*>(residual) + yoff;
+            e = cybq::launch_gemv(v, xp, xdt, mm, static_cast<char*>(y) + yoff, ydt, ctx->num_cus, ec, st);
         }
     }
     if (e != hipSuccess) return fail_hip(ctx, e, "matmul launch");
+    return CYBQ_OK;
+}
+
+int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M, void* y,
+                cybq_dtype ydt, void* stream)
+{
+    return cybq_matmul_ex(ctx, w, x, xdt, M, y, ydt, CYBQ_EPI_NONE, nullptr, stream);
+}
+
+int cybq_weight_fuse_pairs(cybq_ctx* ctx, const cybq_weight* gate, const cybq_weight* up, cybq_weight** out)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (!gate || !up || !out) return fail(ctx, CYBQ_ERR_INVALID, "gate / up / out is NULL");
+    *out = nullptr;
+    if (gate->device != ctx->device || up->device != ctx->device) return fail(ctx, CYBQ_ERR_INVALID, "weight lives on another device");
+    if (gate->bits != up->bits || gate->N != up->N || gate->K != up->K) return fail(ctx, CYBQ_ERR_SHAPE, "gate and up differ in quant or shape");
+    if (gate->N % cybq::kTileN) return fail(ctx, CYBQ_ERR_SHAPE, "N must be a multiple of 16");
+    if (gate->paired || up->paired) return fail(ctx, CYBQ_ERR_INVALID, "inputs are already fused");
+    DeviceGuard guard(ctx->device);
+    if (guard.err != hipSuccess) return fail_hip(ctx, guard.err, "hipSetDevice");
+    cybq_weight* w = nullptr;
+    int rc = alloc_weight(ctx, gate->bits, 2 * gate->N, gate->K, &w);
+    if (rc) return rc;
+    // the native layout is strip-major: output strip 2i is gate strip i, 2i+1 is up strip i
+    const size_t qs = (size_t)gate->KT * (gate->bits == 4 ? 1024 : 2048), ss = (size_t)gate->KT * 128;
+    hipError_t e = hipMemcpy2D(w->q, 2 * qs, gate->q, qs, qs, gate->NT, hipMemcpyDeviceToDevice);
+    if (e == hipSuccess) e = hipMemcpy2D(reinterpret_cast<char*>(w->q) + qs, 2 * qs, up->q, qs, qs, up->NT, hipMemcpyDeviceToDevice);
+    if (e == hipSuccess) e = hipMemcpy2D(w->s, 2 * ss, gate->s, ss, ss, gate->NT, hipMemcpyDeviceToDevice);
+    if (e == hipSuccess) e = hipMemcpy2D(reinterpret_cast<char*>(w->s) + ss, 2 * ss, up->s, ss, ss, up->NT, hipMemcpyDeviceToDevice);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (e != hipSuccess) {
+        (void)hipFree(w->q);
+        (void)hipFree(w->s);
+        delete w;
+        return fail_hip(ctx, e, "weight fuse");
+    }
+    w->paired = true;
+    *out = w;
     return CYBQ_OK;
 }
 
@@ -339,6 +394,20 @@ int cybq_matmul_many(cybq_ctx* ctx, int64_t count, const cybq_weight* const* w, 
     if (count < 0 || (count > 0 && (!w || !x || !y))) return fail(ctx, CYBQ_ERR_INVALID, "bad node list");
     for (int64_t i = 0; i < count; i++) {
         int rc = cybq_matmul(ctx, w[i], x[i], xdt, M, y[i], ydt, stream);
+        if (rc) return rc;
+    }
+    return CYBQ_OK;
+}
+
+int cybq_matmul_many_ex(cybq_ctx* ctx, int64_t count, const cybq_weight* const* w, const void* const* x,
+                        void* const* y, const int* epilogue, const void* const* residual, cybq_dtype xdt, int64_t M,
+                        cybq_dtype ydt, void* stream)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (count < 0 || (count > 0 && (!w || !x || !y))) return fail(ctx, CYBQ_ERR_INVALID, "bad node list");
+    for (int64_t i = 0; i < count; i++) {
+        const cybq_epilogue e = epilogue ? static_cast<cybq_epilogue>(epilogue[i]) : CYBQ_EPI_NONE;
+        int rc = cybq_matmul_ex(ctx, w[i], x[i], xdt, M, y[i], ydt, e, residual ? residual[i] : nullptr, stream);
         if (rc) return rc;
     }
     return CYBQ_OK;

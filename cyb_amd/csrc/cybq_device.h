@@ -129,6 +129,19 @@ __device__ __forceinline__ int q8_slot_value(uint32_t w0, uint32_t w1, int s)
     return (int)((w >> (8 * (s & 3))) & 255u) - 128;
 }
 
+// What happens to an output element on its way to memory.
+//   kEpiAdd     y = residual + x W^T   (residual: same shape and element type as y)
+//   kEpiSwiglu  the weight holds gate and up projections interleaved by 16-row strip
+//               (strip 2i = gate strip i, strip 2i+1 = up strip i); y[:, n] =
+//               silu(gate_n) * up_n has half as many columns as the weight has rows
+constexpr int kEpiNone = 0, kEpiAdd = 1, kEpiSwiglu = 2;
+struct Epilogue {
+    int kind;
+    const void* residual;
+};
+
+__device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+
 struct WeightView {       // what kernels need to know about an uploaded tensor
     const uint32_t* q;    // native q plane
     const uint16_t* s;    // native scale plane

@@ -19,13 +19,14 @@ hipError_t launch_dequant(const WeightView& w, float* out, hipStream_t st);
 
 // decode path, 1 <= M <= 16
 hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
-                       int num_cus, hipStream_t st);
+                       int num_cus, const Epilogue& epi, hipStream_t st);
 // prefill path, M > 16
 // exact: two MFMAs per group with losslessly split weights; otherwise one f16 MFMA
 // per group with weights rounded once to f16
 // workspace: device scratch owned by the context (FAST mode widens bf16 X into it)
 hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
-                       int num_cus, bool exact, void* workspace, size_t workspace_bytes, hipStream_t st);
+                       int num_cus, bool exact, void* workspace, size_t workspace_bytes, const Epilogue& epi,
+                       hipStream_t st);
 
 hipError_t launch_quantize(int bits, const float* src, int N, int K, void* q_out, void* s_out,
                            hipStream_t st);

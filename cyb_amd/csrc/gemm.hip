@@ -70,6 +70,13 @@ __device__ __forceinline__ void store_out_g(void* y, int ydt, int64_t idx, float
 }
 
 
+__device__ __forceinline__ float load_out_g(const void* p, int dt, int64_t idx)
+{
+    if (dt == kF32) return reinterpret_cast<const float*>(p)[idx];
+    if (dt == kF16) return (float)reinterpret_cast<const _Float16*>(p)[idx];
+    return __builtin_bit_cast(float, (uint32_t)reinterpret_cast<const uint16_t*>(p)[idx] << 16);
+}
+
 template <int BITS>
 struct WRegs {               // one native weight tile as loaded by one lane, and its 4 group scales
     u32x4_t q[BITS == 4 ? 1 : 2];
@@ -163,7 +170,7 @@ __device__ __forceinline__ Frag16 bf16_to_f16_frag(const Frag16& a)
 template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kernel(WeightView w, const u32x4_t* __restrict__ x, int x_row_blocks, int M,
                                                    void* __restrict__ y, int ydt, int n_tiles, int m_tiles, float out_scale,
-                                                   float* __restrict__ part, int splits, int kt_per_split)
+                                                   float* __restrict__ part, int splits, int kt_per_split, Epilogue epi)
 {
     // Workgroups are handed to the 8 XCDs round-robin (id % 8) and every XCD has
     // its own L2.  Give each XCD a contiguous run of tiles in row-block-major
@@ -334,6 +341,23 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
             }
         return;
     }
+    if (epi.kind == kEpiSwiglu) {      // column blocks 2p / 2p+1 are gate / up of output block (nt0 >> 1) + p
+        const int n_out = w.N >> 1;
+#pragma unroll
+        for (int i = 0; i < MF; i++)
+#pragma unroll
+            for (int p = 0; p < NF / 2; p++) {
+                const int n = ((nt0 >> 1) + p) * 16 + row16;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int m = m0 + i * 16 + oct * 4 + r;
+                    if (m < M && n < n_out)
+                        store_out_g(y, ydt, (int64_t)m * n_out + n,
+                                    silu_mul(acc[i][2 * p][r] * out_scale, acc[i][2 * p + 1][r] * out_scale));
+                }
+            }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < MF; i++)
 #pragma unroll
@@ -342,25 +366,46 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const int m = m0 + i * 16 + oct * 4 + r;
-                if (m < M && n < w.N) store_out_g(y, ydt, (int64_t)m * w.N + n, acc[i][f][r] * out_scale);
+                if (m < M && n < w.N) {
+                    float v = acc[i][f][r] * out_scale;
+                    if (epi.kind == kEpiAdd) v += load_out_g(epi.residual, ydt, (int64_t)m * w.N + n);
+                    store_out_g(y, ydt, (int64_t)m * w.N + n, v);
+                }
             }
         }
 }
 
-// y = out_scale * (part[0] + part[1] + ... + part[splits-1]), added in that order
-__global__ void splitk_reduce_kernel(const float* __restrict__ part, int splits, int64_t total, void* __restrict__ y, int ydt,
-                                     float out_scale)
+// y = epilogue(out_scale * (part[0] + part[1] + ... + part[splits-1])), slabs added in that order.
+// One thread per output element; N = columns of a slab (for SwiGLU y has N / 2).
+__global__ void splitk_reduce_kernel(const float* __restrict__ part, int splits, int M, int N, void* __restrict__ y, int ydt,
+                                     float out_scale, Epilogue epi)
 {
+    const int64_t slab = (int64_t)M * N;
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= total) return;
+    if (epi.kind == kEpiSwiglu) {
+        const int n_out = N >> 1;
+        if (i >= (int64_t)M * n_out) return;
+        const int m = (int)(i / n_out), n = (int)(i - (int64_t)m * n_out);
+        const int64_t ig = (int64_t)m * N + (n >> 4) * 32 + (n & 15);
+        float g = part[ig], u = part[ig + 16];
+        for (int s = 1; s < splits; s++) {
+            g += part[s * slab + ig];
+            u += part[s * slab + ig + 16];
+        }
+        store_out_g(y, ydt, i, silu_mul(g * out_scale, u * out_scale));
+        return;
+    }
+    if (i >= slab) return;
     float v = part[i];
-    for (int s = 1; s < splits; s++) v += part[(int64_t)s * total + i];
-    store_out_g(y, ydt, i, v * out_scale);
+    for (int s = 1; s < splits; s++) v += part[s * slab + i];
+    v *= out_scale;
+    if (epi.kind == kEpiAdd) v += load_out_g(epi.residual, ydt, i);
+    store_out_g(y, ydt, i, v);
 }
 
 template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES>
 hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, float* part,
-                    size_t part_bytes, int num_cus, hipStream_t st)
+                    size_t part_bytes, int num_cus, const Epilogue& epi, hipStream_t st)
 {
     constexpr int BM = WAVES * MF * 16;
     const size_t lds = (size_t)2 * NF * (4 * (EXACT ? 2 : 1) * 64) * 16;     // operand buffers, 56 .. 128 KB
@@ -385,12 +430,12 @@ hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt,
     splits = (w.KT + kt_per_split - 1) / kt_per_split;          // no empty split
     const unsigned groups = (unsigned)((tiles * splits + 7) / 8 * 8);
     hipLaunchKernelGGL(kern, dim3(groups), dim3(WAVES * 64), lds, st, w, reinterpret_cast<const u32x4_t*>(x), (M + 15) / 16, M,
-                       y, ydt, n_tiles, m_tiles, out_scale, part, splits, kt_per_split);
+                       y, ydt, n_tiles, m_tiles, out_scale, part, splits, kt_per_split, epi);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || splits == 1) return e;
     const int64_t total = (int64_t)M * w.N;
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, part, splits, total, y, ydt,
-                       out_scale);
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, part, splits, M, w.N, y, ydt,
+                       out_scale, epi);
     return hipGetLastError();
 }
 
@@ -401,27 +446,27 @@ hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt,
 //       leave CUs idle.
 template <int BITS, int XBF, int NF, bool EXACT>
 hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, float* part,
-                    size_t part_bytes, int num_cus, hipStream_t st)
+                    size_t part_bytes, int num_cus, const Epilogue& epi, hipStream_t st)
 {
     const int64_t tiles256 = (int64_t)((w.NT + NF - 1) / NF) * ((M + 255) / 256);
-    if (tiles256 < num_cus) return launch_m<BITS, XBF, NF, EXACT, 2, 4>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
-    return launch_m<BITS, XBF, NF, EXACT, 2, 8>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
+    if (tiles256 < num_cus) return launch_m<BITS, XBF, NF, EXACT, 2, 4>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, st);
+    return launch_m<BITS, XBF, NF, EXACT, 2, 8>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, st);
 }
 
 template <int BITS, int XBF>
 hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt, bool exact, float out_scale,
-                     float* part, size_t part_bytes, int num_cus, hipStream_t st)
+                     float* part, size_t part_bytes, int num_cus, const Epilogue& epi, hipStream_t st)
 {
     // 7 column blocks (BN = 112) tile N = 14336 = 128 * 112 exactly: with M = 512
     // that is 256 workgroups, one per CU; 8 column blocks otherwise
-    const bool nf7 = w.NT % 7 == 0;
+    const bool nf7 = w.NT % 7 == 0 && epi.kind != kEpiSwiglu;      // gate / up pairs need an even number of column blocks
     if (exact) {
-        if (nf7) return launch_t<BITS, XBF, 7, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
-        return launch_t<BITS, XBF, 8, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
+        if (nf7) return launch_t<BITS, XBF, 7, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, st);
+        return launch_t<BITS, XBF, 8, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, st);
     }
     if constexpr (XBF == 0) {       // FAST multiplies in f16: bf16 activations were widened by the staging pass
-        if (nf7) return launch_t<BITS, 0, 7, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
-        return launch_t<BITS, 0, 8, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, st);
+        if (nf7) return launch_t<BITS, 0, 7, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, st);
+        return launch_t<BITS, 0, 8, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, st);
     }
     return hipErrorInvalidValue;
 }
@@ -464,7 +509,8 @@ __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict_
 }  // namespace
 
 hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
-                       int num_cus, bool exact, void* workspace, size_t workspace_bytes, hipStream_t st)
+                       int num_cus, bool exact, void* workspace, size_t workspace_bytes, const Epilogue& epi,
+                       hipStream_t st)
 {
     if (xdt == kF32) return hipErrorNotSupported;   // api.hip walks fp32 prefill through the decode kernel
     // FAST multiplies in f16: bf16 activations are widened (2^-4 prescale, undone in the epilogue)
@@ -483,7 +529,10 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
     for (int64_t m_lo = 0; m_lo < M; m_lo += max_rows) {
         const int mc = (int)((M - m_lo) < max_rows ? (M - m_lo) : max_rows);
         const u32x4_t* xs = reinterpret_cast<const u32x4_t*>(static_cast<const char*>(x) + m_lo * row_bytes);
-        void* yc = static_cast<char*>(y) + (size_t)m_lo * w.N * ysize;
+        const int64_t n_out = epi.kind == kEpiSwiglu ? w.N / 2 : w.N;
+        void* yc = static_cast<char*>(y) + (size_t)m_lo * n_out * ysize;
+        Epilogue ec = epi;                 // this row chunk's slice of the residual
+        if (epi.kind == kEpiAdd) ec.residual = static_cast<const char*>(epi.residual) + (size_t)m_lo * n_out * ysize;
         const int K8 = w.K / 8;
         const dim3 grid((unsigned)((mc + 15) / 16), (unsigned)((K8 / 4 + kStageGroups - 1) / kStageGroups));
         if (widen) hipLaunchKernelGGL(stage_x_kernel<true>, grid, dim3(256), 0, st, xs, reinterpret_cast<u32x4_t*>(workspace), mc, K8);
@@ -491,11 +540,11 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         if (w.bits == 4) {
-            e = kdt == kBF16 ? launch_nf<4, 1>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, st)
-                             : launch_nf<4, 0>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, st);
+            e = kdt == kBF16 ? launch_nf<4, 1>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, ec, st)
+                             : launch_nf<4, 0>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, ec, st);
         } else {
-            e = kdt == kBF16 ? launch_nf<8, 1>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, st)
-                             : launch_nf<8, 0>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, st);
+            e = kdt == kBF16 ? launch_nf<8, 1>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, ec, st)
+                             : launch_nf<8, 0>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, ec, st);
         }
         if (e != hipSuccess) return e;
     }

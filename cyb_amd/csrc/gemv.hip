@@ -57,6 +57,20 @@ __device__ __forceinline__ void store_out(void* y, int ydt, int64_t idx, float v
     else reinterpret_cast<uint16_t*>(y)[idx] = f32_to_bf16_rne(v);
 }
 
+__device__ __forceinline__ float load_out(const void* p, int dt, int64_t idx)
+{
+    if (dt == kF32) return reinterpret_cast<const float*>(p)[idx];
+    if (dt == kF16) return (float)reinterpret_cast<const _Float16*>(p)[idx];
+    return __builtin_bit_cast(float, (uint32_t)reinterpret_cast<const uint16_t*>(p)[idx] << 16);
+}
+
+// one finished output element: residual add (fp32, before the single rounding to ydt), store
+__device__ __forceinline__ void emit(void* y, int ydt, const Epilogue& epi, int64_t idx, float v)
+{
+    if (epi.kind == kEpiAdd) v += load_out(epi.residual, ydt, idx);
+    store_out(y, ydt, idx, v);
+}
+
 // x rows of one K slab -> LDS (row stride ldx 16-bit elements; XF32: a second
 // plane of low halves follows the first at plane_elems).  Split in two so that
 // the global loads can be issued BEFORE the weight loads: vmcnt retires in
@@ -249,9 +263,9 @@ __device__ __forceinline__ float sum_partials(const float* red, int nwaves, int 
 // U = tiles a wave keeps in flight per batch.  ONESHOT: the wave's whole share
 // of the strip is at most U tiles, all requested before anything else happens
 // (one register set); otherwise two batches are live and ping-pong.
-template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT>
+template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT, int PAIR>
 __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __restrict__ x, int M, void* __restrict__ y,
-                            int ydt, int slab_tiles, int ldx, int red_offset)
+                            int ydt, int slab_tiles, int ldx, int red_offset, Epilogue epi)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t* xs = reinterpret_cast<uint16_t*>(smem);
@@ -260,9 +274,14 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const int lane = tid & 63;
-    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nwaves = nthreads >> 6;
-    const int nt = blockIdx.x;
+    // SwiGLU: the workgroup owns a gate strip and its up strip; the first half of its
+    // waves splits the K tiles of one, the second half those of the other, x is staged once
+    // (PAIR = 2)
+    const int wv_all = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nwaves = (nthreads >> 6) / PAIR;                 // waves per strip
+    const int sub = (PAIR == 2 && wv_all >= nwaves) ? 1 : 0;
+    const int wv = wv_all - sub * nwaves;
+    const int nt = blockIdx.x * PAIR + sub;
     const int mrow = min(lane & 15, M - 1);
     const int oct = lane >> 4;
     const int plane_elems = M * ldx;
@@ -313,13 +332,24 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
     // reader of x), summed in wave order; wave r finishes output register r
     float* red = reinterpret_cast<float*>(smem + red_offset);
 #pragma unroll
-    for (int r = 0; r < RMAX; r++) red[(wv * RMAX + r) * 64 + lane] = acc[r];
+    for (int r = 0; r < RMAX; r++) red[(wv_all * RMAX + r) * 64 + lane] = acc[r];
     __syncthreads();
+    if (PAIR == 2) {
+        const int n_out = w.N >> 1;
+        const int n = blockIdx.x * 16 + (lane & 15);
+        for (int r = wv_all; r < RMAX; r += 2 * nwaves) {
+            const float g = sum_partials(red + r * 64 + lane, nwaves, RMAX * 64);
+            const float u = sum_partials(red + (nwaves * RMAX + r) * 64 + lane, nwaves, RMAX * 64);
+            const int m = 4 * oct + r;
+            if (m < M && n < n_out) store_out(y, ydt, (int64_t)m * n_out + n, silu_mul(g, u));
+        }
+        return;
+    }
     const int n = nt * 16 + (lane & 15);
     for (int r = wv; r < RMAX; r += nwaves) {
         const float v = sum_partials(red + r * 64 + lane, nwaves, RMAX * 64);
         const int m = 4 * oct + r;
-        if (m < M && n < w.N) store_out(y, ydt, (int64_t)m * w.N + n, v);
+        if (m < M && n < w.N) emit(y, ydt, epi, (int64_t)m * w.N + n, v);
     }
 }
 
@@ -360,8 +390,7 @@ __device__ __forceinline__ void tile_issue_regs(const TileRegs<BITS>& t, const F
 template <int BITS, int XMODE, int TS, int NS>
 // (waves_per_eu: the scheduler would otherwise trade the up-front loads for occupancy)
 __global__ __launch_bounds__(TS <= 2 ? 1024 : 512) __attribute__((amdgpu_waves_per_eu(2, TS <= 2 ? 4 : 2)))
-void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x,
-                                                                         int M, void* __restrict__ y, int ydt)
+void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void* __restrict__ y, int ydt, Epilogue epi)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t magic = q4_magic_vgpr();
@@ -447,54 +476,69 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x,
         for (int r = 0; r < 4; r++) red[((s * nwaves + wv) * 4 + r) * 64 + lane] = acc[s][r];
     __syncthreads();
     // wave v finishes (strip, output register) pairs v, v + waves, ...
+    if (NS >= 2 && epi.kind == kEpiSwiglu) {       // strips 2j / 2j+1 of the group are gate / up of output strip (strip0 >> 1) + j
+        const int n_out = w.N >> 1;
+        for (int p = wv; p < NS * 2; p += nwaves) {
+            const int j = p >> 2, r = p & 3;
+            const int nt = (strip0 >> 1) + j;
+            const int n = nt * 16 + (lane & 15);
+            const float g = sum_partials(red + ((2 * j) * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64);
+            const float u = sum_partials(red + ((2 * j + 1) * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64);
+            const int m = 4 * oct + r;
+            if (m < M && n < n_out) store_out(y, ydt, (int64_t)m * n_out + n, silu_mul(g, u));
+        }
+        return;
+    }
     for (int p = wv; p < NS * 4; p += nwaves) {
         const int s = p >> 2, r = p & 3;
         const int nt = strip0 + s;
         const int n = nt * 16 + (lane & 15);
         const float v = sum_partials(red + (s * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64);
         const int m = 4 * oct + r;
-        if (nt < w.NT && m < M && n < w.N) store_out(y, ydt, (int64_t)m * w.N + n, v);
+        if (nt < w.NT && m < M && n < w.N) emit(y, ydt, epi, (int64_t)m * w.N + n, v);
     }
 }
 
 template <int BITS, int XMODE, int TS, int NS>
-hipError_t launch_rows_t(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, hipStream_t st)
+hipError_t launch_rows_t(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
+                         hipStream_t st)
 {
     const size_t lds = (size_t)NS * nwaves * 4 * 64 * sizeof(float);
     const unsigned groups = (unsigned)((w.NT + NS - 1) / NS);
     hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS>), dim3(groups), dim3(nwaves * 64), lds, st, w,
-                       reinterpret_cast<const uint16_t*>(x), M, y, ydt);
+                       reinterpret_cast<const uint16_t*>(x), M, y, ydt, epi);
     return hipGetLastError();
 }
 
 template <int BITS, int XMODE>
 hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int ydt, int tuned_waves, int num_cus,
-                       hipStream_t st)
+                       const Epilogue& epi, hipStream_t st)
 {
     // strips per workgroup: as many as keeps about one workgroup per CU, at most 4;
     // 8 waves split K (fewer when the strip has fewer tiles), 4 tiles of x per wave and slab
     int ns = (w.NT + num_cus / 2) / num_cus;
     ns = ns >= 3 ? 4 : (ns >= 2 ? 2 : 1);
+    if (epi.kind == kEpiSwiglu && ns < 2) ns = 2;          // a gate strip and its up strip share a workgroup
     int nwaves = tuned_waves > 0 ? tuned_waves : 8;
     while (nwaves > 1 && nwaves * 2 > w.KT) nwaves >>= 1;
     if (nwaves > 8) {          // 16 waves: 128 registers per lane, two tiles of x in flight
-        if (ns == 4) return launch_rows_t<BITS, XMODE, 2, 4>(w, x, M, y, ydt, nwaves, st);
-        if (ns == 2) return launch_rows_t<BITS, XMODE, 2, 2>(w, x, M, y, ydt, nwaves, st);
-        return launch_rows_t<BITS, XMODE, 2, 1>(w, x, M, y, ydt, nwaves, st);
+        if (ns == 4) return launch_rows_t<BITS, XMODE, 2, 4>(w, x, M, y, ydt, nwaves, epi, st);
+        if (ns == 2) return launch_rows_t<BITS, XMODE, 2, 2>(w, x, M, y, ydt, nwaves, epi, st);
+        return launch_rows_t<BITS, XMODE, 2, 1>(w, x, M, y, ydt, nwaves, epi, st);
     }
-    if (ns == 4) return launch_rows_t<BITS, XMODE, 4, 4>(w, x, M, y, ydt, nwaves, st);
-    if (ns == 2) return launch_rows_t<BITS, XMODE, 4, 2>(w, x, M, y, ydt, nwaves, st);
+    if (ns == 4) return launch_rows_t<BITS, XMODE, 4, 4>(w, x, M, y, ydt, nwaves, epi, st);
+    if (ns == 2) return launch_rows_t<BITS, XMODE, 4, 2>(w, x, M, y, ydt, nwaves, epi, st);
     // one strip per workgroup and a long K: eight tiles per wave and slab, fewer round trips
-    if (w.KT > nwaves * 4) return launch_rows_t<BITS, XMODE, 8, 1>(w, x, M, y, ydt, nwaves, st);
-    return launch_rows_t<BITS, XMODE, 4, 1>(w, x, M, y, ydt, nwaves, st);
+    if (w.KT > nwaves * 4) return launch_rows_t<BITS, XMODE, 8, 1>(w, x, M, y, ydt, nwaves, epi, st);
+    return launch_rows_t<BITS, XMODE, 4, 1>(w, x, M, y, ydt, nwaves, epi, st);
 }
 
 int g_tune_waves = 0, g_tune_unroll = 0, g_tune_rows = 0;
 
 constexpr int kLdsBudget = 64 * 1024;
 
-template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT>
-hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves,
+template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT, int PAIR>
+hipError_t launch_p(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
                     hipStream_t st)
 {
     const int planes = XMODE == XF32 ? 2 : 1;
@@ -512,8 +556,8 @@ hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt,
     }
     int ldx = slab_tiles * kTileK + 8;
     const size_t xbytes = ((size_t)M * ldx * 2 * planes + 255) & ~(size_t)255;
-    const size_t lds = xbytes + (size_t)nwaves * RMAX * 64 * sizeof(float);     // x, then the waves' partial sums
-    auto kern = gemv_kernel<BITS, XMODE, RMAX, U, ONESHOT>;
+    const size_t lds = xbytes + (size_t)PAIR * nwaves * RMAX * 64 * sizeof(float);     // x, then the waves' partial sums
+    auto kern = gemv_kernel<BITS, XMODE, RMAX, U, ONESHOT, PAIR>;
     static bool attr_set = false;
     if (!attr_set) {
         // M = 16 fp32 activations with 8 waves need 66 KB, just over the default cap
@@ -522,34 +566,43 @@ hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt,
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    hipLaunchKernelGGL(kern, dim3(w.NT), dim3(nwaves * 64), lds, st, w, x, M, y, ydt, slab_tiles, ldx, (int)xbytes);
+    hipLaunchKernelGGL(kern, dim3(w.NT / PAIR), dim3(nwaves * PAIR * 64), lds, st, w, x, M, y, ydt, slab_tiles, ldx, (int)xbytes,
+                       epi);
     return hipGetLastError();
 }
 
-template <int BITS, int XMODE, int U, bool ONESHOT>
-hipError_t launch_r(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves,
+template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT>
+hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
                     hipStream_t st)
 {
-    if (M == 1) return launch_t<BITS, XMODE, 1, U, ONESHOT>(w, x, M, y, ydt, nwaves, st);
-    if (M == 2) return launch_t<BITS, XMODE, 2, U, ONESHOT>(w, x, M, y, ydt, nwaves, st);
-    return launch_t<BITS, XMODE, 4, U, ONESHOT>(w, x, M, y, ydt, nwaves, st);
+    if (epi.kind == kEpiSwiglu) return launch_p<BITS, XMODE, RMAX, U, ONESHOT, 2>(w, x, M, y, ydt, nwaves, epi, st);
+    return launch_p<BITS, XMODE, RMAX, U, ONESHOT, 1>(w, x, M, y, ydt, nwaves, epi, st);
+}
+
+template <int BITS, int XMODE, int U, bool ONESHOT>
+hipError_t launch_r(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
+                    hipStream_t st)
+{
+    if (M == 1) return launch_t<BITS, XMODE, 1, U, ONESHOT>(w, x, M, y, ydt, nwaves, epi, st);
+    if (M == 2) return launch_t<BITS, XMODE, 2, U, ONESHOT>(w, x, M, y, ydt, nwaves, epi, st);
+    return launch_t<BITS, XMODE, 4, U, ONESHOT>(w, x, M, y, ydt, nwaves, epi, st);
 }
 
 template <int BITS, int XMODE>
 hipError_t launch_u(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, int unroll,
-                    hipStream_t st)
+                    const Epilogue& epi, hipStream_t st)
 {
     const int planes = XMODE == XF32 ? 2 : 1;
     const bool one_slab = (int64_t)M * (w.KT * kTileK + 8) * 2 * planes <= kLdsBudget;
     const int per_wave = (w.KT + nwaves - 1) / nwaves;
     if (one_slab && unroll == 0) {
-        if (per_wave <= 2) return launch_r<BITS, XMODE, 2, true>(w, x, M, y, ydt, nwaves, st);
-        if (per_wave <= 4) return launch_r<BITS, XMODE, 4, true>(w, x, M, y, ydt, nwaves, st);
+        if (per_wave <= 2) return launch_r<BITS, XMODE, 2, true>(w, x, M, y, ydt, nwaves, epi, st);
+        if (per_wave <= 4) return launch_r<BITS, XMODE, 4, true>(w, x, M, y, ydt, nwaves, epi, st);
         // (fp32 activations carry two operand planes: 8 tiles in flight would spill)
-        if (per_wave <= 8 && XMODE != XF32) return launch_r<BITS, XMODE, 8, true>(w, x, M, y, ydt, nwaves, st);
+        if (per_wave <= 8 && XMODE != XF32) return launch_r<BITS, XMODE, 8, true>(w, x, M, y, ydt, nwaves, epi, st);
     }
-    if (unroll == 4 && XMODE != XF32) return launch_r<BITS, XMODE, 4, false>(w, x, M, y, ydt, nwaves, st);
-    return launch_r<BITS, XMODE, 2, false>(w, x, M, y, ydt, nwaves, st);
+    if (unroll == 4 && XMODE != XF32) return launch_r<BITS, XMODE, 4, false>(w, x, M, y, ydt, nwaves, epi, st);
+    return launch_r<BITS, XMODE, 2, false>(w, x, M, y, ydt, nwaves, epi, st);
 }
 
 }  // namespace
@@ -562,7 +615,7 @@ void set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll)
 }
 
 hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
-                       int num_cus, hipStream_t st)
+                       int num_cus, const Epilogue& epi, hipStream_t st)
 {
     // Waves per workgroup (= split of a strip's K tiles).  Depends on the weight
     // shape only, never on M, so that the summation order is the same for every
@@ -575,6 +628,7 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
         while (nwaves < 16 && w.KT > 8 * nwaves) nwaves *= 2;
     }
     if (nwaves > 16) nwaves = 16;
+    if (epi.kind == kEpiSwiglu && nwaves > 8) nwaves = 8;      // two strips per workgroup: 2 x 8 waves at most
     while (nwaves > 1 && nwaves > w.KT) nwaves >>= 1;
     // 0: request a wave's whole share up front when it fits, else stream in batches of 2
     int unroll = g_tune_unroll;
@@ -583,21 +637,21 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
     const bool rows_kernel = g_tune_rows == 1 || (g_tune_rows == 0 && M >= 4);
     if (rows_kernel && xdt != kF32) {
         if (w.bits == 4) {
-            if (xdt == kF16) return launch_rows<4, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, st);
-            return launch_rows<4, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, st);
+            if (xdt == kF16) return launch_rows<4, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
+            return launch_rows<4, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
         }
-        if (xdt == kF16) return launch_rows<8, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, st);
-        return launch_rows<8, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, st);
+        if (xdt == kF16) return launch_rows<8, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
+        return launch_rows<8, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
     }
 
     if (w.bits == 4) {
-        if (xdt == kF16) return launch_u<4, XF16>(w, x, M, y, ydt, nwaves, unroll, st);
-        if (xdt == kBF16) return launch_u<4, XBF16>(w, x, M, y, ydt, nwaves, unroll, st);
-        return launch_u<4, XF32>(w, x, M, y, ydt, nwaves, unroll, st);
+        if (xdt == kF16) return launch_u<4, XF16>(w, x, M, y, ydt, nwaves, unroll, epi, st);
+        if (xdt == kBF16) return launch_u<4, XBF16>(w, x, M, y, ydt, nwaves, unroll, epi, st);
+        return launch_u<4, XF32>(w, x, M, y, ydt, nwaves, unroll, epi, st);
     }
-    if (xdt == kF16) return launch_u<8, XF16>(w, x, M, y, ydt, nwaves, unroll, st);
-    if (xdt == kBF16) return launch_u<8, XBF16>(w, x, M, y, ydt, nwaves, unroll, st);
-    return launch_u<8, XF32>(w, x, M, y, ydt, nwaves, unroll, st);
+    if (xdt == kF16) return launch_u<8, XF16>(w, x, M, y, ydt, nwaves, unroll, epi, st);
+    if (xdt == kBF16) return launch_u<8, XBF16>(w, x, M, y, ydt, nwaves, unroll, epi, st);
+    return launch_u<8, XF32>(w, x, M, y, ydt, nwaves, unroll, epi, st);
 }
 
 }  // namespace cybq

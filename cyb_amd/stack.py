@@ -37,6 +37,7 @@ class LinearStack:
     nodes: List[QMatMul] = field(default_factory=list)
     weights: List[QWeight] = field(default_factory=list)
     planar: Dict[str, tuple] = field(default_factory=dict)     # name -> (q bytes, scales) kept for checks
+    epilogues: List[str] = field(default_factory=list)         # per node: "none" | "add" | "swiglu" (empty = none anywhere)
 
     @property
     def weight_bytes(self) -> int:
@@ -59,11 +60,13 @@ def fused_shapes(shapes: Dict[str, tuple] = None) -> Dict[str, tuple]:
 
 
 def build(backend: Backend, layers: int = 32, bits: int = formats.Q4, seed: int = 5, keep_planar: int = 0,
-          shapes: Dict[str, tuple] = None, order: List[str] = None) -> LinearStack:
+          shapes: Dict[str, tuple] = None, order: List[str] = None, epilogues: bool = False) -> LinearStack:
     """Random-init stack with N(0, 0.02) weights quantised on the device.
 
     keep_planar: for the first that many layers, the PLANAR device buffers are kept in
-    `stack.planar` so that a checker can pull them back and recompute outputs."""
+    `stack.planar` so that a checker can pull them back and recompute outputs.
+    epilogues: with the fused shapes, `gate_up_proj` becomes a strip-interleaved pair run with the
+    SwiGLU epilogue (its output has half the columns) and `o_proj` / `down_proj` add a residual."""
     import torch
     shapes = shapes or synth.LLAMA3_8B_LINEARS
     st = LinearStack(backend, layers, bits)
@@ -78,10 +81,27 @@ def build(backend: Backend, layers: int = 32, bits: int = formats.Q4, seed: int 
             sd = torch.empty(N * (K // 32), dtype=torch.int16, device="cuda")
             backend.quantize(bits, w, N, K, qd, sd)
             name = tensor_name(layer, lin)
-            qw = backend.weight_from_device(bits, N, K, qd, sd, name=name)
+            epi = "none"
+            if epilogues and lin == "gate_up_proj":
+                # rows [0, N/2) are the gate projection, [N/2, N) the up projection
+                h = N // 2
+                hq, hs = h * K * bits // 8, h * (K // 32)
+                g = backend.weight_from_device(bits, h, K, qd[:hq], sd[:hs])
+                u = backend.weight_from_device(bits, h, K, qd[hq:], sd[hs:])
+                torch.cuda.synchronize()
+                qw = backend.fuse_pairs(g, u, name=name)
+                g.free()
+                u.free()
+                epi = "swiglu"
+            else:
+                qw = backend.weight_from_device(bits, N, K, qd, sd, name=name)
+                if epilogues and lin in ("o_proj", "down_proj"):
+                    epi = "add"
             torch.cuda.synchronize()              # qd / sd / w are released below
             st.weights.append(qw)
             st.nodes.append(QMatMul(w=name, x=f"in.{K}", y=f"out.{lin}", quant=bits, M=1, N=N, K=K))
+            if epilogues:
+                st.epilogues.append(epi)
             if layer < keep_planar:
                 st.planar[name] = (qd, sd)
             del w
@@ -98,9 +118,18 @@ def edges_for(stack: LinearStack, M: int, seed: int = 5, shapes: Dict[str, tuple
         x = torch.from_numpy(synth.activations(seed, M, K, stream=i)).cuda().to(xdtype or torch.float16)
         edges[f"in.{K}"] = x
     for lin in shapes:
-        edges[f"out.{lin}"] = torch.empty((M, shapes[lin][1]), dtype=torch.float32, device="cuda")
+        cols = shapes[lin][1] // 2 if (stack.epilogues and lin == "gate_up_proj") else shapes[lin][1]
+        edges[f"out.{lin}"] = torch.empty((M, cols), dtype=torch.float32, device="cuda")
+    if stack.epilogues:
+        widths = sorted({shapes[lin][1] for lin in ("o_proj", "down_proj") if lin in shapes})
+        for i, N in enumerate(widths):          # the residual stream entering o_proj / down_proj
+            edges[f"res.{N}"] = torch.from_numpy(synth.activations(seed, M, N, stream=100 + i)).cuda()
     return edges
 
 
 def plan(stack: LinearStack, edges):
-    return stack.backend.plan_many(stack.weights, [edges[n.x] for n in stack.nodes], [edges[n.y] for n in stack.nodes])
+    xs, ys = [edges[n.x] for n in stack.nodes], [edges[n.y] for n in stack.nodes]
+    if not stack.epilogues:
+        return stack.backend.plan_many(stack.weights, xs, ys)
+    res = [edges[f"res.{n.N}"] if e == "add" else None for n, e in zip(stack.nodes, stack.epilogues)]
+    return stack.backend.plan_many(stack.weights, xs, ys, stack.epilogues, res)

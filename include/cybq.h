@@ -144,6 +144,42 @@ int cybq_matmul_many(cybq_ctx* ctx, int64_t count, const cybq_weight* const* w,
                      const void* const* x, void* const* y, cybq_dtype xdt, int64_t M,
                      cybq_dtype ydt, void* stream);
 
+/* What the kernel does with an output element on its way to memory: the ops on
+ * either side of a linear in the decode loop ("norm -> QKV -> ... -> O proj ->
+ * residual -> norm -> FFN -> residual", decide/pipeline.md:51), fused so that
+ * they cost no launch and no round trip through HBM.  The reference's own
+ * definitions of these ops are not visible in its tree; the formulas below are
+ * the LlamaStyle ones and are this library's choice. */
+typedef enum cybq_epilogue {
+    CYBQ_EPI_NONE = 0,
+    CYBQ_EPI_ADD = 1,      /* y = residual + x W^T; residual: [M,N] of ydt; added in fp32, rounded once */
+    CYBQ_EPI_SWIGLU = 2    /* w from cybq_weight_fuse_pairs(gate, up): y[M,N/2] = silu(x Wg^T) * (x Wu^T),
+                              silu(t) = t / (1 + exp(-t)), all in fp32, rounded once */
+} cybq_epilogue;
+
+/* Replaces: the FFN's gate and up projections as one weight (both read the same
+ * activations - decide/pipeline.md:51).  `gate` and `up`: same quant, same
+ * [N,K], N a multiple of 16.  The result has 2N rows, gate and up interleaved in
+ * strips of 16 rows (device to device, no requantisation); as a plain matmul
+ * weight it yields those interleaved columns, with CYBQ_EPI_SWIGLU it yields
+ * the N activated columns.  The inputs stay valid and independent. */
+int cybq_weight_fuse_pairs(cybq_ctx* ctx, const cybq_weight* gate, const cybq_weight* up, cybq_weight** out);
+
+/* cybq_matmul with an epilogue.  `residual` is read only for CYBQ_EPI_ADD (device
+ * pointer, may alias y).  CYBQ_EPI_SWIGLU needs a weight made by
+ * cybq_weight_fuse_pairs and writes y[M, N/2].  fp32 activations support
+ * CYBQ_EPI_NONE / CYBQ_EPI_ADD only for M <= 16. */
+int cybq_matmul_ex(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M,
+                   void* y, cybq_dtype ydt, cybq_epilogue epilogue, const void* residual, void* stream);
+
+/* cybq_matmul_many with an epilogue per node: epilogue[i] is a cybq_epilogue,
+ * residual[i] its residual (NULL unless CYBQ_EPI_ADD); either array may be NULL
+ * (= no epilogues). */
+int cybq_matmul_many_ex(cybq_ctx* ctx, int64_t count, const cybq_weight* const* w,
+                        const void* const* x, void* const* y, const int* epilogue,
+                        const void* const* residual, cybq_dtype xdt, int64_t M, cybq_dtype ydt,
+                        void* stream);
+
 /* Replaces: nothing the runtime calls per token; it is the verification hook
  * ("dequantised weights match bit-exactly"): out[N,K] f32 = f32(scale) * q. */
 int cybq_dequant(cybq_ctx* ctx, const cybq_weight* w, float* out, void* stream);

@@ -41,6 +41,8 @@ struct QMatMulNode {
     cybq_quant quant = CYBQ_Q4;
     int group = CYBQ_GROUP;
     int64_t M = 1, N = 0, K = 0;
+    cybq_epilogue epilogue = CYBQ_EPI_NONE;   // fused op behind the linear
+    std::string residual;                      // edge added to the output (CYBQ_EPI_ADD)
 };
 
 // A device buffer bound to an edge name: pointer, element type, rows.
@@ -101,6 +103,17 @@ public:
         if (s) weights_[name] = std::move(w);
         return s;
     }
+    // gate and up projections of one FFN as a single weight for CYBQ_EPI_SWIGLU
+    Status fuse_pairs(const std::string& name, const std::string& gate, const std::string& up)
+    {
+        const Weight *g = find(gate), *u = find(up);
+        if (!g || !u) return fail(CYBQ_ERR_INVALID, "gate / up not loaded");
+        Weight w;
+        w.ctx_ = ctx_;
+        Status s = wrap(cybq_weight_fuse_pairs(ctx_, g->get(), u->get(), &w.h_));
+        if (s) weights_[name] = std::move(w);
+        return s;
+    }
     void unload(const std::string& name) { weights_.erase(name); }
     const Weight* find(const std::string& name) const
     {
@@ -114,6 +127,11 @@ public:
                   void* stream = nullptr)
     {
         return wrap(cybq_matmul(ctx_, w.get(), x, xdt, M, y, ydt, stream));
+    }
+    Status matmul_ex(const Weight& w, const void* x, cybq_dtype xdt, int64_t M, void* y, cybq_dtype ydt,
+                     cybq_epilogue epilogue, const void* residual, void* stream = nullptr)
+    {
+        return wrap(cybq_matmul_ex(ctx_, w.get(), x, xdt, M, y, ydt, epilogue, residual, stream));
     }
     Status dequant(const Weight& w, float* out, void* stream = nullptr)
     {
@@ -131,7 +149,15 @@ public:
         auto xi = edges.find(node.x), yi = edges.find(node.y);
         if (xi == edges.end() || yi == edges.end()) return fail(CYBQ_ERR_INVALID, "edge not bound");
         if (xi->second.rows < node.M || yi->second.rows < node.M) return fail(CYBQ_ERR_SHAPE, "edge has too few rows");
-        return matmul(*w, xi->second.ptr, xi->second.dtype, node.M, yi->second.ptr, yi->second.dtype, stream);
+        const void* res = nullptr;
+        if (node.epilogue == CYBQ_EPI_ADD) {
+            auto ri = edges.find(node.residual);
+            if (ri == edges.end() || ri->second.dtype != yi->second.dtype || ri->second.rows < node.M)
+                return fail(CYBQ_ERR_INVALID, "residual edge not bound or of another type");
+            res = ri->second.ptr;
+        }
+        return matmul_ex(*w, xi->second.ptr, xi->second.dtype, node.M, yi->second.ptr, yi->second.dtype, node.epilogue,
+                         res, stream);
     }
 
     // a whole step: the nodes are resolved once, then launched back to back from native code
@@ -140,8 +166,9 @@ public:
     {
         if (nodes.empty()) return Status{};
         std::vector<const cybq_weight*> ws;
-        std::vector<const void*> xs;
+        std::vector<const void*> xs, rs;
         std::vector<void*> ys;
+        std::vector<int> es;
         const Edge& x0 = edges.at(nodes[0].x);
         const Edge& y0 = edges.at(nodes[0].y);
         for (const auto& n : nodes) {
@@ -150,12 +177,20 @@ public:
             if (!w || xi == edges.end() || yi == edges.end()) return fail(CYBQ_ERR_INVALID, "unresolved node '" + n.w + "'");
             if (xi->second.dtype != x0.dtype || yi->second.dtype != y0.dtype || n.M != nodes[0].M)
                 return fail(CYBQ_ERR_INVALID, "run_all needs one M and one dtype pair");
+            const void* res = nullptr;
+            if (n.epilogue == CYBQ_EPI_ADD) {
+                auto ri = edges.find(n.residual);
+                if (ri == edges.end() || ri->second.dtype != y0.dtype) return fail(CYBQ_ERR_INVALID, "residual of '" + n.w + "' not bound");
+                res = ri->second.ptr;
+            }
             ws.push_back(w->get());
             xs.push_back(xi->second.ptr);
             ys.push_back(yi->second.ptr);
+            es.push_back((int)n.epilogue);
+            rs.push_back(res);
         }
-        return wrap(cybq_matmul_many(ctx_, (int64_t)nodes.size(), ws.data(), xs.data(), ys.data(), x0.dtype,
-                                     nodes[0].M, y0.dtype, stream));
+        return wrap(cybq_matmul_many_ex(ctx_, (int64_t)nodes.size(), ws.data(), xs.data(), ys.data(), es.data(), rs.data(),
+                                        x0.dtype, nodes[0].M, y0.dtype, stream));
     }
 
 private:

@@ -79,6 +79,28 @@ int main(int argc, char** argv)
     bad.N += 16;
     if (be.run(bad, edges).code != CYBQ_ERR_SHAPE) { std::printf("ERROR shape mismatch not reported\n"); return 1; }
 
+    // fused residual add: with the node's own output as residual the result is exactly twice it
+    {
+        const int64_t cnt = M * nodes[0].N;
+        float* y2 = nullptr;
+        if (hipMalloc((void**)&y2, (size_t)cnt * 4) != hipSuccess) { std::printf("ERROR hip y2\n"); return 1; }
+        edges["y0_twice"] = cybq::Edge{y2, CYBQ_F32, M, nodes[0].N};
+        cybq::QMatMulNode add = nodes[0];
+        add.y = "y0_twice";
+        add.epilogue = CYBQ_EPI_ADD;
+        add.residual = nodes[0].y;
+        s = be.run(add, edges);
+        if (!s) { std::printf("ERROR %d %s\n", s.code, s.text.c_str()); return 1; }
+        std::vector<float> a((size_t)cnt), b((size_t)cnt);
+        if (hipMemcpy(a.data(), outs[0], (size_t)cnt * 4, hipMemcpyDeviceToHost) != hipSuccess ||
+            hipMemcpy(b.data(), y2, (size_t)cnt * 4, hipMemcpyDeviceToHost) != hipSuccess) { std::printf("ERROR copy\n"); return 1; }
+        for (int64_t j = 0; j < cnt; j++)
+            if (b[j] != 2.0f * a[j]) { std::printf("ERROR residual add differs at %lld\n", (long long)j); return 1; }
+        add.residual = "no.such.edge";
+        if (be.run(add, edges).code != CYBQ_ERR_INVALID) { std::printf("ERROR missing residual not reported\n"); return 1; }
+        (void)hipFree(y2);
+    }
+
     const double* want = reinterpret_cast<const double*>(yb.data());
     for (size_t i = 0; i < nodes.size(); i++) {
         const int64_t cnt = M * nodes[i].N;

@@ -357,6 +357,113 @@ def test_config4_full_size(backend, oracle, prefill_mode, M, shape):
         assert torch.equal(y2, y * 2)
 
 
+# ------------------------------------------------------- fused epilogues
+# The reference's definitions of the ops around a linear are not in its tree (parity
+# unpinned); the checks below pin the library's stated formulas: y = r + x W^T, and
+# y = silu(x Wg^T) * (x Wu^T) with silu(t) = t / (1 + exp(-t)), against float64.
+
+def _silu_mul(g, u):
+    return g / (1.0 + np.exp(-g)) * u
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M,xdt", [(1, "f16"), (2, "bf16"), (3, "f32"), (4, "f16"), (16, "bf16"), (40, "bf16"), (300, "f16")])
+def test_epilogue_residual_add(backend, oracle, prefill_mode, bits, M, xdt):
+    N, K = 272, 1024
+    q, s = _quant(oracle, bits, N, K)
+    qw = backend.upload_quantized(q, s, bits)
+    x = _x(M, K, xdt)
+    r = torch.from_numpy(synth.activations(33, M, N)).cuda()
+    ref = oracle.matmul_f64(q, s, x.float().cpu().numpy()) + r.double().cpu().numpy()
+    y = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    backend.matmul_ex(qw, x, y, "add", r)
+    torch.cuda.synchronize()
+    bar = TIGHT if (M <= 16 or xdt == "f32") else _bar(prefill_mode)
+    assert oracle.rel_l2(y.cpu().numpy(), ref) < bar
+    # in place (residual aliases y) and with a 16-bit residual stream: added in fp32, rounded once
+    y2 = r.clone()
+    backend.matmul_ex(qw, x, y2, "add", y2)
+    torch.cuda.synchronize()
+    assert torch.equal(y2, y)
+    rb = r.to(torch.bfloat16)
+    yb = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    backend.matmul_ex(qw, x, yb, "add", rb)
+    y32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    backend.matmul(qw, x, y32)
+    torch.cuda.synchronize()
+    assert torch.equal(yb, (y32 + rb.float()).to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M,xdt", [(1, "f16"), (2, "bf16"), (3, "f32"), (4, "f16"), (9, "f16"), (16, "bf16"), (40, "bf16"), (300, "f16")])
+def test_epilogue_swiglu(backend, oracle, prefill_mode, bits, M, xdt):
+    N, K = 336, 1024                      # 21 strips per projection
+    qg, sg = _quant(oracle, bits, N, K, cfg=41)
+    qu, su = _quant(oracle, bits, N, K, cfg=42)
+    wg = backend.upload_quantized(qg, sg, bits)
+    wu = backend.upload_quantized(qu, su, bits)
+    wf = backend.fuse_pairs(wg, wu)
+    assert (wf.N, wf.K) == (2 * N, K)
+    x = _x(M, K, xdt)
+    xf = x.float().cpu().numpy()
+    g, u = oracle.matmul_f64(qg, sg, xf), oracle.matmul_f64(qu, su, xf)
+    y = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    backend.matmul_ex(wf, x, y, "swiglu")
+    torch.cuda.synchronize()
+    assert not torch.isnan(y).any()
+    bar = TIGHT if (M <= 16 or xdt == "f32") else 2 * _bar(prefill_mode)
+    assert oracle.rel_l2(y.cpu().numpy(), _silu_mul(g, u)) < bar
+    # the fused weight as a plain matmul: gate and up columns interleaved in blocks of 16
+    if xdt != "f32" or M <= 16:
+        yi = _run(backend, wf, x)
+        yg, yu = _run(backend, wg, x), _run(backend, wu, x)
+        inter = torch.stack([yg.view(M, N // 16, 16), yu.view(M, N // 16, 16)], dim=2).reshape(M, 2 * N)
+        if M <= 16:
+            assert torch.equal(yi, inter)
+            # and the epilogue is exactly silu * mul of those sums, in fp32
+            want = (yg / (1.0 + torch.exp(-yg)) * yu)
+            assert (y - want).abs().max().item() <= 2e-6 * want.abs().max().item()
+        else:
+            assert ((yi - inter).double().norm() / inter.double().norm()).item() < 1e-6
+
+
+def test_epilogue_swiglu_full_size_and_split_k(backend, oracle):
+    # Llama-3-8B FFN width at decode (M = 1, 8) and prefill (M = 128: 14 column tiles per row block,
+    # so K is split over workgroups and the activation runs in the slab-adding kernel)
+    K, N = 4096, 14336
+    qg, sg = _quant(oracle, 4, N, K, cfg=43)
+    qu, su = _quant(oracle, 4, N, K, cfg=44)
+    wg, wu = backend.upload_quantized(qg, sg, 4), backend.upload_quantized(qu, su, 4)
+    wf = backend.fuse_pairs(wg, wu)
+    dg = torch.from_numpy(oracle.dequant(qg, sg)).cuda().double()
+    du = torch.from_numpy(oracle.dequant(qu, su)).cuda().double()
+    for M, xdt, bar in ((1, "f16", TIGHT), (8, "f16", TIGHT), (128, "bf16", 2 * FAST), (512, "bf16", 2 * FAST)):
+        x = _x(M, K, xdt)
+        g, u = x.double() @ dg.T, x.double() @ du.T
+        ref = g / (1.0 + torch.exp(-g)) * u
+        y = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        backend.matmul_ex(wf, x, y, "swiglu")
+        torch.cuda.synchronize()
+        err = ((y.double() - ref).norm() / ref.norm()).item()
+        assert err < bar, (M, err)
+
+
+def test_epilogue_errors(backend, oracle):
+    q, s = _quant(oracle, 4, 64, 256)
+    qw = backend.upload_quantized(q, s, 4)
+    x = _x(2, 256, "f16")
+    y = torch.empty((2, 64), dtype=torch.float32, device="cuda")
+    with pytest.raises(CybqError):
+        backend.matmul_ex(qw, x, y, "swiglu")                 # not a fused pair
+    with pytest.raises(CybqError):
+        backend.matmul_ex(qw, x, y, "add", None)              # no residual
+    q2, s2 = _quant(oracle, 4, 40, 256)
+    with pytest.raises(CybqError):
+        backend.fuse_pairs(backend.upload_quantized(q2, s2, 4), backend.upload_quantized(q2, s2, 4))   # N % 16
+    with pytest.raises(CybqError):
+        backend.fuse_pairs(qw, backend.upload_quantized(q2, s2, 4))                                    # shapes differ
+
+
 # ------------------------------------------------------------------ quantise
 
 @pytest.mark.parametrize("bits", [4, 8])
@@ -460,6 +567,38 @@ def test_decode_stack_small(backend, oracle):
         ref = oracle.matmul_f64(q, s, edges[last.x].float().cpu().numpy())
         assert oracle.rel_l2(edges[last.y].cpu().numpy(), ref) < TIGHT
     assert st.step_bytes(1) == sum(formats.matmul_bytes(4, n.N, n.K, 1, 2, 4) for n in st.nodes)
+    for w in st.weights:
+        w.free()
+
+
+def test_decode_stack_with_epilogues(backend, oracle):
+    """The fused node list (qkv, o + residual, gate/up with SwiGLU, down + residual) through
+    cybq_matmul_many_ex; every node's output recomputed from the weights the stack kept."""
+    from cyb_amd import stack
+    base = {"q_proj": (512, 512), "k_proj": (512, 128), "v_proj": (512, 128), "o_proj": (512, 512),
+            "gate_proj": (512, 1792), "up_proj": (512, 1792), "down_proj": (1792, 512)}
+    shapes = stack.fused_shapes(base)
+    st = stack.build(backend, layers=2, seed=6, keep_planar=2, shapes=shapes, order=list(shapes), epilogues=True)
+    assert st.epilogues == ["none", "add", "swiglu", "add"] * 2
+    for M in (1, 8, 40):
+        edges = stack.edges_for(st, M, shapes=shapes, xdtype=torch.bfloat16 if M > 16 else None)
+        pl = stack.plan(st, edges)
+        backend.matmul_many(pl, M)
+        torch.cuda.synchronize()
+        bar = TIGHT if M <= 16 else 2 * FAST
+        for node, epi in list(zip(st.nodes, st.epilogues))[-4:]:          # the last layer's outputs are still in place
+            qd, sd = st.planar[node.w]
+            q = formats.unpack_planar(qd.cpu().numpy(), 4, node.N, node.K)
+            s = sd.cpu().numpy().view(np.uint16).reshape(node.N, node.K // 32)
+            ref = oracle.matmul_f64(q, s, edges[node.x].float().cpu().numpy())
+            if epi == "add":
+                ref = ref + edges[f"res.{node.N}"].double().cpu().numpy()
+            elif epi == "swiglu":
+                h = node.N // 2
+                ref = _silu_mul(ref[:, :h], ref[:, h:])
+            got = edges[node.y].cpu().numpy()
+            assert got.shape == ref.shape
+            assert oracle.rel_l2(got, ref) < bar, (M, node.w, epi)
     for w in st.weights:
         w.free()
 
