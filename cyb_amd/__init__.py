@@ -9,7 +9,7 @@ node, `Backend.run` executes it.  All arithmetic happens in libcybq.so
 op on the host and raises if the library is missing.
 """
 from .backend import Backend, CybqError, QMatMul, QWeight, library_path
-from . import container, formats, stack, synth
+from . import container, driver, formats, stack, synth
 
-__all__ = ["Backend", "CybqError", "QMatMul", "QWeight", "library_path", "formats", "synth", "container", "stack"]
+__all__ = ["Backend", "CybqError", "QMatMul", "QWeight", "library_path", "formats", "synth", "container", "stack", "driver"]
 __version__ = "0.1.0"

@@ -603,6 +603,27 @@ def test_decode_stack_with_epilogues(backend, oracle):
         w.free()
 
 
+def test_driver_events_and_rates(backend):
+    """The caller loop in the reference's units: event order, token counts, positive rates."""
+    from cyb_amd import driver, stack
+    shapes = stack.fused_shapes({"q_proj": (512, 512), "k_proj": (512, 128), "v_proj": (512, 128), "o_proj": (512, 512),
+                                 "gate_proj": (512, 1792), "up_proj": (512, 1792), "down_proj": (1792, 512)})
+    st = stack.build(backend, layers=2, seed=7, shapes=shapes, order=list(shapes))
+    evs = list(driver.ask(backend, st, prompt_tokens=300, new_tokens=5, chunk=128, shapes=shapes))
+    pre = [e["Prefill"] for e in evs if "Prefill" in e]
+    assert [p["done"] for p in pre] == [0, 128, 256, 300] and all(p["total"] == 300 for p in pre)
+    assert [e["Delta"] for e in evs if "Delta" in e] == [0, 1, 2, 3, 4]
+    ans = evs[-1]["Answer"]
+    assert ans.tokens == 5 and ans.tok_in_s > 0 and ans.tok_out_s > 0 and ans.tok_per_s > 0
+    # decode only, batch of 4
+    evs = list(driver.ask(backend, st, prompt_tokens=0, new_tokens=3, batch=4, shapes=shapes))
+    assert evs[-1]["Answer"].tokens == 12 and evs[-1]["Answer"].tok_in_s == 0.0
+    with pytest.raises(ValueError):
+        list(driver.ask(backend, st, 1, 1, batch=17, shapes=shapes))
+    for w in st.weights:
+        w.free()
+
+
 def test_container_to_backend(backend, oracle, tmp_path):
     from cyb_amd import container
     q, s = _quant(oracle, 4, 64, 256)
