@@ -67,10 +67,26 @@ def cpu_baseline(q, s, x32, alg_bytes, budget_s=12.0):
         el = time.perf_counter() - t0
         if el >= budget_s or reps >= 4000:
             break
+    # the same restatement on one thread (fixed summation order), a few passes
+    r1, t1 = 0, time.perf_counter()
+    while r1 < 40 and time.perf_counter() - t1 < 3.0:
+        qq, ss = copies[r1 % len(copies)]
+        ora.matmul_f32(qq, ss, x32)
+        r1 += 1
+    el1 = time.perf_counter() - t1
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next((l.split(":", 1)[1].strip() for l in f if l.startswith("model name")), "")
+    except OSError:
+        pass
     return {"value": round(alg_bytes * reps / el / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": f"{reps} passes of the same 4096->14336 Q4 batch-1 matmul over {len(copies)} weight copies, "
                       f"{el:.1f} s, C restatement (fp32, per-group scale, rows split over {threads} threads)",
-            "us_per_pass": round(el / reps * 1e6, 1)}
+            "us_per_pass": round(el / reps * 1e6, 1),
+            "one_thread": {"value": round(alg_bytes * r1 / el1 / 1e9, 3), "unit": "GB/s", "us_per_pass": round(el1 / r1 * 1e6, 1),
+                           "passes": r1},
+            "host": {"cpus_available": cores, "cpu_model": model}}
 
 
 def main():
