@@ -432,11 +432,15 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
             for (int j = 0; j < 4; j++)
                 a[u][j].u = *reinterpret_cast<const u32x4_t*>(xrow + min(kt[u] * kTileK + j * 32, w.K - 32));
         }
-        // every weight tile of this slab (all strips) is requested before the first
-        // one is used: the whole slab is in flight while the wave works through it
+        // The memory pipeline takes requests at its own pace: a wave that asks for all its
+        // tiles first sits in the issue queue for microseconds and only then starts on
+        // its arithmetic.  So the strips are walked two requests ahead: strip s+2 is
+        // requested, then strip s (whose tiles were requested two steps ago) is
+        // multiplied while the others are on their way.
         TileRegs<BITS> buf[NS][TS];
+        constexpr int AHEAD = NS < 2 ? NS : 2;
 #pragma unroll
-        for (int s = 0; s < NS; s++)
+        for (int s = 0; s < AHEAD; s++)
 #pragma unroll
             for (int u = 0; u < TS; u++) load_tile<BITS>(buf[s][u], w, sbase[s] + kt[u], lane);
 #pragma unroll
@@ -448,6 +452,12 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
                     a[u][j].u[p] = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane, (int)a[u][j].u[p]);
 #pragma unroll
         for (int s = 0; s < NS; s++) {
+            if (NS > 2) __builtin_amdgcn_sched_barrier(0);
+            if (s + AHEAD < NS) {
+#pragma unroll
+                for (int u = 0; u < TS; u++) load_tile<BITS>(buf[s + AHEAD][u], w, sbase[s + AHEAD] + kt[u], lane);
+            }
+            if (NS > 2) __builtin_amdgcn_sched_barrier(0);
             float4_t dprev[4];
             u32x2_t sprev = {0u, 0u};
 #pragma unroll
