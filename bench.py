@@ -101,8 +101,8 @@ def main():
                          "kernels, for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (the op shards by rows of W; "
-              "see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+        print("bench.py measures one GPU: this build has no multi-GPU path (the op would shard by rows of W "
+              "for q/k/v/gate/up and by columns for o/down). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np
