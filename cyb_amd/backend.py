@@ -79,6 +79,7 @@ def load_library() -> ctypes.CDLL:
                                      ctypes.POINTER(i64)]
     lib.cybq_matmul.argtypes = [vp, vp, vp, ci, i64, vp, ci, vp]
     lib.cybq_matmul_ex.argtypes = [vp, vp, vp, ci, i64, vp, ci, ci, vp, vp]
+    lib.cybq_matmul_norm.argtypes = [vp, vp, vp, ci, i64, vp, ci, ctypes.c_float, vp, ci, ci, vp, vp]
     lib.cybq_weight_fuse_pairs.argtypes = [vp, vp, vp, ctypes.POINTER(vp)]
     lib.cybq_matmul_many_ex.argtypes = [vp, i64, vp, vp, vp, vp, vp, ci, i64, ci, vp]
     lib.cybq_set_prefill_mode.argtypes = [vp, ci]
@@ -276,6 +277,17 @@ class Backend:
             M = int(x.shape[0]) if x.dim() == 2 else 1
         self._check(self._lib.cybq_matmul_ex(self._ctx, w.handle, _ptr(x), _dtype_code(x, None), M, _ptr(y),
                                              _dtype_code(y, None), EPILOGUES[epilogue], _ptr(residual), stream))
+
+    def matmul_norm(self, w: QWeight, x, gamma, eps: float, y, epilogue: str = "none", residual=None,
+                    M: Optional[int] = None, stream: int = 0) -> None:
+        """cybq_matmul_norm: RMSNorm (gamma [K], eps) folded into the activation load, then the epilogue."""
+        if epilogue not in EPILOGUES:
+            raise CybqError(-1, "invalid argument", f"unknown epilogue {epilogue!r}")
+        if M is None:
+            M = int(x.shape[0]) if x.dim() == 2 else 1
+        self._check(self._lib.cybq_matmul_norm(self._ctx, w.handle, _ptr(x), _dtype_code(x, None), M, _ptr(gamma),
+                                               _dtype_code(gamma, None), ctypes.c_float(eps), _ptr(y),
+                                               _dtype_code(y, None), EPILOGUES[epilogue], _ptr(residual), stream))
 
     def fuse_pairs(self, gate: QWeight, up: QWeight, name: Optional[str] = None) -> QWeight:
         """One weight holding gate and up projections interleaved by 16-row strip (device to device)."""

@@ -292,8 +292,10 @@ int cybq_weight_info(const cybq_weight* w, int* quant, int64_t* N, int64_t* K, i
     return CYBQ_OK;
 }
 
-int cybq_matmul_ex(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M, void* y,
-                   cybq_dtype ydt, cybq_epilogue epilogue, const void* residual, void* stream)
+namespace {
+int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M, const void* gamma,
+                 cybq_dtype gdt, float eps, void* y, cybq_dtype ydt, cybq_epilogue epilogue, const void* residual,
+                 void* stream)
 {
     if (!ctx) return CYBQ_ERR_INVALID;
     if (!w || !x || !y) return fail(ctx, CYBQ_ERR_INVALID, "w / x / y is NULL");
@@ -302,18 +304,27 @@ int cybq_matmul_ex(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtyp
     if (w->device != ctx->device) return fail(ctx, CYBQ_ERR_INVALID, "weight lives on another device");
     if (!aligned16(x)) return fail(ctx, CYBQ_ERR_ALIGN, "x must be 16-byte aligned");
     if (reinterpret_cast<uintptr_t>(y) % dtype_size(ydt)) return fail(ctx, CYBQ_ERR_ALIGN, "y is not aligned to its element size");
-    cybq::Epilogue epi = {cybq::kEpiNone, nullptr};
+    cybq::Epilogue epi = {cybq::kEpiNone, nullptr, nullptr, 0, 0.f};
+    if (gamma) {
+        if (!dtype_ok(gdt)) return fail(ctx, CYBQ_ERR_INVALID, "unknown gamma dtype");
+        if (reinterpret_cast<uintptr_t>(gamma) % dtype_size(gdt)) return fail(ctx, CYBQ_ERR_ALIGN, "gamma is not aligned to its element size");
+        if (!(eps >= 0.f)) return fail(ctx, CYBQ_ERR_INVALID, "eps must be >= 0");
+    }
     if (epilogue == CYBQ_EPI_ADD) {
         if (!residual) return fail(ctx, CYBQ_ERR_INVALID, "CYBQ_EPI_ADD needs a residual");
         if (reinterpret_cast<uintptr_t>(residual) % dtype_size(ydt)) return fail(ctx, CYBQ_ERR_ALIGN, "residual is not aligned to its element size");
-        epi = {cybq::kEpiAdd, residual};
+        epi.kind = cybq::kEpiAdd;
+        epi.residual = residual;
     } else if (epilogue == CYBQ_EPI_SWIGLU) {
         if (!w->paired) return fail(ctx, CYBQ_ERR_INVALID, "CYBQ_EPI_SWIGLU needs a weight made by cybq_weight_fuse_pairs");
         if (xdt == CYBQ_F32 && M > 16) return fail(ctx, CYBQ_ERR_INVALID, "CYBQ_EPI_SWIGLU with fp32 activations is limited to M <= 16");
-        epi = {cybq::kEpiSwiglu, nullptr};
+        epi.kind = cybq::kEpiSwiglu;
     } else if (epilogue != CYBQ_EPI_NONE) {
         return fail(ctx, CYBQ_ERR_INVALID, "unknown epilogue");
     }
+    epi.gamma = gamma;
+    epi.gamma_dt = (int)gdt;
+    epi.eps = eps;
     DeviceGuard guard(ctx->device);
     if (guard.err != hipSuccess) return fail_hip(ctx, guard.err, "hipSetDevice");
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -339,6 +350,22 @@ int cybq_matmul_ex(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtyp
     }
     if (e != hipSuccess) return fail_hip(ctx, e, "matmul launch");
     return CYBQ_OK;
+}
+}  // namespace
+
+int cybq_matmul_ex(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M, void* y,
+                   cybq_dtype ydt, cybq_epilogue epilogue, const void* residual, void* stream)
+{
+    return matmul_fused(ctx, w, x, xdt, M, nullptr, CYBQ_F32, 0.f, y, ydt, epilogue, residual, stream);
+}
+
+int cybq_matmul_norm(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M, const void* gamma,
+                     cybq_dtype gdt, float eps, void* y, cybq_dtype ydt, cybq_epilogue epilogue, const void* residual,
+                     void* stream)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (!gamma) return fail(ctx, CYBQ_ERR_INVALID, "gamma is NULL");
+    return matmul_fused(ctx, w, x, xdt, M, gamma, gdt, eps, y, ydt, epilogue, residual, stream);
 }
 
 int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M, void* y,

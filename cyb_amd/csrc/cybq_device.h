@@ -134,10 +134,17 @@ __device__ __forceinline__ int q8_slot_value(uint32_t w0, uint32_t w1, int s)
 //   kEpiSwiglu  the weight holds gate and up projections interleaved by 16-row strip
 //               (strip 2i = gate strip i, strip 2i+1 = up strip i); y[:, n] =
 //               silu(gate_n) * up_n has half as many columns as the weight has rows
+//   gamma != nullptr  RMSNorm folded into the activation load: the kernel multiplies
+//               x[m, k] * gamma[k] (rounded once to the operand type) on the way in,
+//               sums x^2 over the row in fp32 in a fixed order, and scales the finished
+//               sums by rstd[m] = 1 / sqrt(mean_k x[m,k]^2 + eps) before the epilogue
 constexpr int kEpiNone = 0, kEpiAdd = 1, kEpiSwiglu = 2;
 struct Epilogue {
     int kind;
     const void* residual;
+    const void* gamma;     // [K] of gamma_dt (kF32 / kF16 / kBF16 codes), or nullptr
+    int gamma_dt;
+    float eps;
 };
 
 __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }

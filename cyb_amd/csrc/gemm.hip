@@ -77,6 +77,20 @@ __device__ __forceinline__ float load_out_g(const void* p, int dt, int64_t idx)
     return __builtin_bit_cast(float, (uint32_t)reinterpret_cast<const uint16_t*>(p)[idx] << 16);
 }
 
+// Folded RMSNorm on the prefill path: the staging pass leaves, per row of the chunk, `nblk`
+// partial sums of squares; rstd of a row adds them in index order.
+struct NormStats {
+    const float* part;
+    int nblk;
+};
+
+__device__ __forceinline__ float rstd_of(const NormStats& ns, int row, int K, float eps)
+{
+    float t = 0.f;
+    for (int j = 0; j < ns.nblk; j++) t += ns.part[(int64_t)row * ns.nblk + j];
+    return 1.0f / sqrtf(t / (float)K + eps);
+}
+
 template <int BITS>
 struct WRegs {               // one native weight tile as loaded by one lane, and its 4 group scales
     u32x4_t q[BITS == 4 ? 1 : 2];
@@ -170,7 +184,7 @@ __device__ __forceinline__ Frag16 bf16_to_f16_frag(const Frag16& a)
 template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kernel(WeightView w, const u32x4_t* __restrict__ x, int x_row_blocks, int M,
                                                    void* __restrict__ y, int ydt, int n_tiles, int m_tiles, float out_scale,
-                                                   float* __restrict__ part, int splits, int kt_per_split, Epilogue epi)
+                                                   float* __restrict__ part, int splits, int kt_per_split, Epilogue epi, NormStats ns)
 {
     // Workgroups are handed to the 8 XCDs round-robin (id % 8) and every XCD has
     // its own L2.  Give each XCD a contiguous run of tiles in row-block-major
@@ -341,6 +355,16 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
             }
         return;
     }
+    if (epi.gamma) {                   // folded RMSNorm: scale every row by its rstd before the epilogue
+#pragma unroll
+        for (int i = 0; i < MF; i++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float rs = rstd_of(ns, min(m0 + i * 16 + oct * 4 + r, M - 1), K, epi.eps);
+#pragma unroll
+                for (int f = 0; f < NF; f++) acc[i][f][r] *= rs;
+            }
+    }
     if (epi.kind == kEpiSwiglu) {      // column blocks 2p / 2p+1 are gate / up of output block (nt0 >> 1) + p
         const int n_out = w.N >> 1;
 #pragma unroll
@@ -378,7 +402,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
 // y = epilogue(out_scale * (part[0] + part[1] + ... + part[splits-1])), slabs added in that order.
 // One thread per output element; N = columns of a slab (for SwiGLU y has N / 2).
 __global__ void splitk_reduce_kernel(const float* __restrict__ part, int splits, int M, int N, void* __restrict__ y, int ydt,
-                                     float out_scale, Epilogue epi)
+                                     float out_scale, Epilogue epi, NormStats ns, int K)
 {
     const int64_t slab = (int64_t)M * N;
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -392,20 +416,22 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ part, int splits,
             g += part[s * slab + ig];
             u += part[s * slab + ig + 16];
         }
-        store_out_g(y, ydt, i, silu_mul(g * out_scale, u * out_scale));
+        const float sc = epi.gamma ? out_scale * rstd_of(ns, m, K, epi.eps) : out_scale;
+        store_out_g(y, ydt, i, silu_mul(g * sc, u * sc));
         return;
     }
     if (i >= slab) return;
     float v = part[i];
     for (int s = 1; s < splits; s++) v += part[s * slab + i];
     v *= out_scale;
+    if (epi.gamma) v *= rstd_of(ns, (int)(i / N), K, epi.eps);
     if (epi.kind == kEpiAdd) v += load_out_g(epi.residual, ydt, i);
     store_out_g(y, ydt, i, v);
 }
 
 template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES>
 hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, float* part,
-                    size_t part_bytes, int num_cus, const Epilogue& epi, hipStream_t st)
+                    size_t part_bytes, int num_cus, const Epilogue& epi, const NormStats& ns, hipStream_t st)
 {
     constexpr int BM = WAVES * MF * 16;
     const size_t lds = (size_t)2 * NF * (4 * (EXACT ? 2 : 1) * 64) * 16;     // operand buffers, 56 .. 128 KB
@@ -430,12 +456,12 @@ hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt,
     splits = (w.KT + kt_per_split - 1) / kt_per_split;          // no empty split
     const unsigned groups = (unsigned)((tiles * splits + 7) / 8 * 8);
     hipLaunchKernelGGL(kern, dim3(groups), dim3(WAVES * 64), lds, st, w, reinterpret_cast<const u32x4_t*>(x), (M + 15) / 16, M,
-                       y, ydt, n_tiles, m_tiles, out_scale, part, splits, kt_per_split, epi);
+                       y, ydt, n_tiles, m_tiles, out_scale, part, splits, kt_per_split, epi, ns);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || splits == 1) return e;
     const int64_t total = (int64_t)M * w.N;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, part, splits, M, w.N, y, ydt,
-                       out_scale, epi);
+                       out_scale, epi, ns, w.K);
     return hipGetLastError();
 }
 
@@ -446,27 +472,27 @@ hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt,
 //       leave CUs idle.
 template <int BITS, int XBF, int NF, bool EXACT>
 hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, float* part,
-                    size_t part_bytes, int num_cus, const Epilogue& epi, hipStream_t st)
+                    size_t part_bytes, int num_cus, const Epilogue& epi, const NormStats& ns, hipStream_t st)
 {
     const int64_t tiles256 = (int64_t)((w.NT + NF - 1) / NF) * ((M + 255) / 256);
-    if (tiles256 < num_cus) return launch_m<BITS, XBF, NF, EXACT, 2, 4>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, st);
-    return launch_m<BITS, XBF, NF, EXACT, 2, 8>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, st);
+    if (tiles256 < num_cus) return launch_m<BITS, XBF, NF, EXACT, 2, 4>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
+    return launch_m<BITS, XBF, NF, EXACT, 2, 8>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
 }
 
 template <int BITS, int XBF>
 hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt, bool exact, float out_scale,
-                     float* part, size_t part_bytes, int num_cus, const Epilogue& epi, hipStream_t st)
+                     float* part, size_t part_bytes, int num_cus, const Epilogue& epi, const NormStats& ns, hipStream_t st)
 {
     // 7 column blocks (BN = 112) tile N = 14336 = 128 * 112 exactly: with M = 512
     // that is 256 workgroups, one per CU; 8 column blocks otherwise
     const bool nf7 = w.NT % 7 == 0 && epi.kind != kEpiSwiglu;      // gate / up pairs need an even number of column blocks
     if (exact) {
-        if (nf7) return launch_t<BITS, XBF, 7, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, st);
-        return launch_t<BITS, XBF, 8, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, st);
+        if (nf7) return launch_t<BITS, XBF, 7, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
+        return launch_t<BITS, XBF, 8, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
     }
     if constexpr (XBF == 0) {       // FAST multiplies in f16: bf16 activations were widened by the staging pass
-        if (nf7) return launch_t<BITS, 0, 7, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, st);
-        return launch_t<BITS, 0, 8, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, st);
+        if (nf7) return launch_t<BITS, 0, 7, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
+        return launch_t<BITS, 0, 8, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
     }
     return hipErrorInvalidValue;
 }
@@ -479,8 +505,12 @@ hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt
 constexpr int kStageGroups = 16;                       // scale groups per workgroup
 constexpr int kStagePitch = kStageGroups * 4 + 1;      // 16 B slots per LDS row (odd: no bank conflicts)
 
-template <bool WIDEN>
-__global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict__ src, u32x4_t* __restrict__ dst, int M, int K8)
+// NORM: RMSNorm folded in.  x * gamma is formed in fp32 and rounded once to the operand type
+// (XBF: the input is bf16; WIDEN: bf16 in, f16 * 2^-4 out); the squares of the unscaled row are
+// summed per (row, workgroup) in a fixed butterfly order into ssq_part[row * gridDim.y + blockIdx.y].
+template <bool WIDEN, bool XBF, bool NORM>
+__global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict__ src, u32x4_t* __restrict__ dst, int M, int K8,
+                                                      Epilogue epi, float* __restrict__ ssq_part)
 {
     __shared__ u32x4_t tile[16 * kStagePitch];
     const int rb = blockIdx.x;
@@ -493,7 +523,38 @@ __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict_
         Frag16 a;
         a.u = (u32x4_t){0u, 0u, 0u, 0u};
         if (row < M && c < K8) a.u = src[(int64_t)row * K8 + c];
-        if (WIDEN) a = bf16_to_f16_frag(a);
+        if (NORM) {
+            float sq = 0.f;
+            if (c < K8) {
+#pragma unroll
+                for (int p = 0; p < 4; p++) {
+                    float v0, v1;
+                    if (XBF) {
+                        v0 = __builtin_bit_cast(float, a.u[p] << 16);
+                        v1 = __builtin_bit_cast(float, a.u[p] & 0xffff0000u);
+                    } else {
+                        const half2_t h = as_h2(a.u[p]);
+                        v0 = (float)h.x;
+                        v1 = (float)h.y;
+                    }
+                    sq = fmaf(v1, v1, fmaf(v0, v0, sq));
+                    const float sc = WIDEN ? 0.0625f : 1.0f;
+                    v0 *= load_out_g(epi.gamma, epi.gamma_dt, c * 8 + 2 * p) * sc;
+                    v1 *= load_out_g(epi.gamma, epi.gamma_dt, c * 8 + 2 * p + 1) * sc;
+                    if (XBF && !WIDEN) {
+                        a.u[p] = (uint32_t)f32_to_bf16_rne_g(v0) | ((uint32_t)f32_to_bf16_rne_g(v1) << 16);
+                    } else {
+                        const half2_t h = {(_Float16)v0, (_Float16)v1};
+                        a.u[p] = as_u32(h);
+                    }
+                }
+            }
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) sq += __shfl_xor(sq, off, 64);
+            if ((t & 63) == 0) ssq_part[(int64_t)row * gridDim.y + blockIdx.y] = sq;      // (rows past M: zeros, never read)
+        } else if (WIDEN) {
+            a = bf16_to_f16_frag(a);
+        }
         tile[r * kStagePitch + (t & 63)] = a.u;
     }
     __syncthreads();
@@ -522,9 +583,14 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
     // First half of the workspace: staged X; second half: partial sums of a K split.
     const size_t half = workspace_bytes / 2;
     float* part = reinterpret_cast<float*>(static_cast<char*>(workspace) + half);
+    // The last MiB of the first half: per-row partial sums of squares of a folded RMSNorm
+    // (rows of a chunk x K / 512 floats: at most half / 256 bytes).
+    const size_t stats_bytes = (size_t)1 << 20;
+    if (!workspace || half <= stats_bytes) return hipErrorOutOfMemory;
+    float* ssq_part = reinterpret_cast<float*>(static_cast<char*>(workspace) + half - stats_bytes);
     const int64_t row_bytes = (int64_t)w.K * 2;
-    const int64_t max_rows = (int64_t)(half / (size_t)row_bytes) / 256 * 256;
-    if (!workspace || max_rows < 256) return hipErrorOutOfMemory;
+    const int64_t max_rows = (int64_t)((half - stats_bytes) / (size_t)row_bytes) / 256 * 256;
+    if (max_rows < 256) return hipErrorOutOfMemory;
     const size_t ysize = ydt == kF32 ? 4 : 2;
     for (int64_t m_lo = 0; m_lo < M; m_lo += max_rows) {
         const int mc = (int)((M - m_lo) < max_rows ? (M - m_lo) : max_rows);
@@ -535,16 +601,25 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
         if (epi.kind == kEpiAdd) ec.residual = static_cast<const char*>(epi.residual) + (size_t)m_lo * n_out * ysize;
         const int K8 = w.K / 8;
         const dim3 grid((unsigned)((mc + 15) / 16), (unsigned)((K8 / 4 + kStageGroups - 1) / kStageGroups));
-        if (widen) hipLaunchKernelGGL(stage_x_kernel<true>, grid, dim3(256), 0, st, xs, reinterpret_cast<u32x4_t*>(workspace), mc, K8);
-        else hipLaunchKernelGGL(stage_x_kernel<false>, grid, dim3(256), 0, st, xs, reinterpret_cast<u32x4_t*>(workspace), mc, K8);
+        u32x4_t* xst = reinterpret_cast<u32x4_t*>(workspace);
+        const NormStats ns = {ssq_part, (int)grid.y};
+        if (epi.gamma) {
+            if (widen) hipLaunchKernelGGL((stage_x_kernel<true, true, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+            else if (xdt == kBF16) hipLaunchKernelGGL((stage_x_kernel<false, true, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+            else hipLaunchKernelGGL((stage_x_kernel<false, false, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+        } else if (widen) {
+            hipLaunchKernelGGL((stage_x_kernel<true, true, false>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+        } else {
+            hipLaunchKernelGGL((stage_x_kernel<false, false, false>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+        }
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         if (w.bits == 4) {
-            e = kdt == kBF16 ? launch_nf<4, 1>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, ec, st)
-                             : launch_nf<4, 0>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, ec, st);
+            e = kdt == kBF16 ? launch_nf<4, 1>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, ec, ns, st)
+                             : launch_nf<4, 0>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, ec, ns, st);
         } else {
-            e = kdt == kBF16 ? launch_nf<8, 1>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, ec, st)
-                             : launch_nf<8, 0>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, ec, st);
+            e = kdt == kBF16 ? launch_nf<8, 1>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, ec, ns, st)
+                             : launch_nf<8, 0>(w, workspace, mc, yc, ydt, exact, out_scale, part, half, num_cus, ec, ns, st);
         }
         if (e != hipSuccess) return e;
     }

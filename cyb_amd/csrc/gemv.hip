@@ -260,10 +260,71 @@ __device__ __forceinline__ float sum_partials(const float* red, int nwaves, int 
     return v;
 }
 
+// ---- RMSNorm folded into the staged x (LDS kernel) ------------------------------
+__device__ __forceinline__ float load_gamma(const void* g, int gdt, int k)
+{
+    if (gdt == kF32) return reinterpret_cast<const float*>(g)[k];
+    if (gdt == kF16) return (float)reinterpret_cast<const _Float16*>(g)[k];
+    return __builtin_bit_cast(float, (uint32_t)reinterpret_cast<const uint16_t*>(g)[k] << 16);
+}
+
+// value k of a staged row as fp32 (XF32: hi + lo planes)
+template <int XMODE>
+__device__ __forceinline__ float staged_x(const uint16_t* row, int plane_elems, int k)
+{
+    if (XMODE == XBF16) return __builtin_bit_cast(float, (uint32_t)row[k] << 16);
+    float v = (float)reinterpret_cast<const _Float16*>(row)[k];
+    if (XMODE == XF32) v += (float)reinterpret_cast<const _Float16*>(row + plane_elems)[k];
+    return v;
+}
+
+template <int XMODE>
+__device__ __forceinline__ void store_staged_x(uint16_t* row, int plane_elems, int k, float v)
+{
+    if (XMODE == XBF16) {
+        row[k] = f32_to_bf16_rne(v);
+    } else {
+        const _Float16 h = (_Float16)v;
+        reinterpret_cast<_Float16*>(row)[k] = h;
+        if (XMODE == XF32) reinterpret_cast<_Float16*>(row + plane_elems)[k] = (_Float16)(v - (float)h);
+    }
+}
+
+// One staged K slab: adds this slab's sum of squares of every row to ssq[row] (row m
+// belongs to wave m % waves; lanes stride over k, then a fixed butterfly: the order of
+// the additions never changes), then replaces x by x * gamma.  Two barriers inside.
+template <int XMODE>
+__device__ __forceinline__ void norm_staged_slab(uint16_t* xs, int M, int slab_k, int k_begin, int K, int ldx,
+                                                 int plane_elems, const Epilogue& epi, float* ssq, int tid,
+                                                 int nthreads)
+{
+    const int lane = tid & 63, wv = tid >> 6, nw = nthreads >> 6;
+    const int kk = min(slab_k, K - k_begin);
+    for (int m = wv; m < M; m += nw) {
+        const uint16_t* row = xs + m * ldx;
+        float a = 0.f;
+        for (int k = lane; k < kk; k += 64) {
+            const float v = staged_x<XMODE>(row, plane_elems, k);
+            a = fmaf(v, v, a);
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) a += __shfl_xor(a, off, 64);
+        if (lane == 0) ssq[m] += a;
+    }
+    __syncthreads();
+    for (int i = tid; i < M * kk; i += nthreads) {
+        const int m = i / kk, k = i - m * kk;
+        uint16_t* row = xs + m * ldx;
+        store_staged_x<XMODE>(row, plane_elems, k, staged_x<XMODE>(row, plane_elems, k) * load_gamma(epi.gamma, epi.gamma_dt, k_begin + k));
+    }
+    __syncthreads();
+}
+
 // U = tiles a wave keeps in flight per batch.  ONESHOT: the wave's whole share
 // of the strip is at most U tiles, all requested before anything else happens
 // (one register set); otherwise two batches are live and ping-pong.
-template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT, int PAIR>
+// NORM: RMSNorm folded into the staged x (only instantiated for the streaming variant U = 2).
+template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT, int PAIR, bool NORM>
 __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __restrict__ x, int M, void* __restrict__ y,
                             int ydt, int slab_tiles, int ldx, int red_offset, Epilogue epi)
 {
@@ -292,6 +353,10 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
 #pragma unroll
     for (int r = 0; r < RMAX; r++) acc[r] = 0.f;
 
+    // folded RMSNorm: per-row sums of squares live behind the partial sums
+    float* ssq = reinterpret_cast<float*>(smem + red_offset) + PAIR * nwaves * RMAX * 64;
+    if (NORM && tid < 16) ssq[tid] = 0.f;            // (ordered before its first use by the staging barrier)
+
     if (ONESHOT) {
         TileRegs<BITS> buf[U];
         XRegs<XMODE> xr;
@@ -300,6 +365,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
         load_batch<BITS, U>(buf, w, strip, wv, nwaves, w.KT, lane);
         stage_x_store<XMODE, RMAX == 1>(xr, xs, M, w.KT * kTileK, ldx, plane_elems, 0, tid, nthreads);
         __syncthreads();
+        if (NORM) norm_staged_slab<XMODE>(xs, M, w.KT * kTileK, 0, w.K, ldx, plane_elems, epi, ssq, tid, nthreads);
         const uint16_t* xbase = xs + mrow * ldx + oct * 8;
         compute_batch<BITS, XMODE, RMAX, U>(buf, wv, nwaves, w.KT, xbase, plane_elems, magic, acc);
     } else {
@@ -316,6 +382,8 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
             load_batch<BITS, U>(bufA, w, base, wv, nwaves, st, lane);
             stage_x_store<XMODE, RMAX == 1>(xr, xs, M, st * kTileK, ldx, plane_elems, 0, tid, nthreads);
             __syncthreads();
+            if (NORM)
+                norm_staged_slab<XMODE>(xs, M, st * kTileK, slab0 * kTileK, w.K, ldx, plane_elems, epi, ssq, tid, nthreads);
 
             const uint16_t* xbase = xs + mrow * ldx + oct * 8;
             for (int i0 = wv; i0 < st; i0 += 2 * stride) {
@@ -338,17 +406,23 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
         const int n_out = w.N >> 1;
         const int n = blockIdx.x * 16 + (lane & 15);
         for (int r = wv_all; r < RMAX; r += 2 * nwaves) {
-            const float g = sum_partials(red + r * 64 + lane, nwaves, RMAX * 64);
-            const float u = sum_partials(red + (nwaves * RMAX + r) * 64 + lane, nwaves, RMAX * 64);
+            float g = sum_partials(red + r * 64 + lane, nwaves, RMAX * 64);
+            float u = sum_partials(red + (nwaves * RMAX + r) * 64 + lane, nwaves, RMAX * 64);
             const int m = 4 * oct + r;
+            if (NORM) {
+                const float rstd = 1.0f / sqrtf(ssq[min(m, M - 1)] / (float)w.K + epi.eps);
+                g *= rstd;
+                u *= rstd;
+            }
             if (m < M && n < n_out) store_out(y, ydt, (int64_t)m * n_out + n, silu_mul(g, u));
         }
         return;
     }
     const int n = nt * 16 + (lane & 15);
     for (int r = wv; r < RMAX; r += nwaves) {
-        const float v = sum_partials(red + r * 64 + lane, nwaves, RMAX * 64);
+        float v = sum_partials(red + r * 64 + lane, nwaves, RMAX * 64);
         const int m = 4 * oct + r;
+        if (NORM) v *= 1.0f / sqrtf(ssq[min(m, M - 1)] / (float)w.K + epi.eps);
         if (m < M && n < w.N) emit(y, ydt, epi, (int64_t)m * w.N + n, v);
     }
 }
@@ -387,7 +461,36 @@ __device__ __forceinline__ void tile_issue_regs(const TileRegs<BITS>& t, const F
     }
 }
 
-template <int BITS, int XMODE, int TS, int NS>
+// NORM: RMSNorm folded into the activation load (epi.gamma / epi.eps): an operand fragment
+// is multiplied by gamma in registers right after it reaches operand order, the lane adds
+// the squares of what it holds; rows meet across lanes and waves in the final exchange.
+template <int XMODE>
+__device__ __forceinline__ void norm_frag(Frag16& a, const Epilogue& epi, int k0, bool counts, float& ssq)
+{
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        float v0, v1;
+        if (XMODE == XBF16) {
+            v0 = __builtin_bit_cast(float, a.u[p] << 16);
+            v1 = __builtin_bit_cast(float, a.u[p] & 0xffff0000u);
+        } else {
+            const half2_t h = as_h2(a.u[p]);
+            v0 = (float)h.x;
+            v1 = (float)h.y;
+        }
+        if (counts) ssq = fmaf(v1, v1, fmaf(v0, v0, ssq));
+        v0 *= load_gamma(epi.gamma, epi.gamma_dt, k0 + 2 * p);
+        v1 *= load_gamma(epi.gamma, epi.gamma_dt, k0 + 2 * p + 1);
+        if (XMODE == XBF16) {
+            a.u[p] = (uint32_t)f32_to_bf16_rne(v0) | ((uint32_t)f32_to_bf16_rne(v1) << 16);
+        } else {
+            const half2_t h = {(_Float16)v0, (_Float16)v1};
+            a.u[p] = as_u32(h);
+        }
+    }
+}
+
+template <int BITS, int XMODE, int TS, int NS, bool NORM>
 // (waves_per_eu: the scheduler would otherwise trade the up-front loads for occupancy)
 __global__ __launch_bounds__(TS <= 2 ? 1024 : 512) __attribute__((amdgpu_waves_per_eu(2, TS <= 2 ? 4 : 2)))
 void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void* __restrict__ y, int ydt, Epilogue epi)
@@ -413,6 +516,7 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
     for (int s = 0; s < NS; s++)
 #pragma unroll
         for (int r = 0; r < 4; r++) acc[s][r] = 0.f;
+    float ssq = 0.f;          // NORM: squares of the x values this lane holds (row lane % 16)
 
     int64_t sbase[NS];
 #pragma unroll
@@ -450,6 +554,15 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
 #pragma unroll
                 for (int p = 0; p < 4; p++)
                     a[u][j].u[p] = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane, (int)a[u][j].u[p]);
+        if (NORM) {
+#pragma unroll
+            for (int u = 0; u < TS; u++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int kg = kt[u] * kTileK + j * 32;            // (a group past K repeats the last one: not counted)
+                    norm_frag<XMODE>(a[u][j], epi, min(kg, w.K - 32) + oct * 8, valid[u] && kg < w.K, ssq);
+                }
+        }
 #pragma unroll
         for (int s = 0; s < NS; s++) {
             if (NS > 2) __builtin_amdgcn_sched_barrier(0);
@@ -484,7 +597,22 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
     for (int s = 0; s < NS; s++)
 #pragma unroll
         for (int r = 0; r < 4; r++) red[((s * nwaves + wv) * 4 + r) * 64 + lane] = acc[s][r];
+    float* ssq_part = red + NS * nwaves * 4 * 64;      // [wave][row]
+    if (NORM) {
+        ssq += __shfl_xor(ssq, 16, 64);
+        ssq += __shfl_xor(ssq, 32, 64);
+        if (lane < 16) ssq_part[wv * 16 + lane] = ssq;
+    }
     __syncthreads();
+    float rstd[4] = {1.f, 1.f, 1.f, 1.f};             // of the rows this lane's outputs belong to
+    if (NORM) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            float t = 0.f;
+            for (int k = 0; k < nwaves; k++) t += ssq_part[k * 16 + 4 * oct + r];
+            rstd[r] = 1.0f / sqrtf(t / (float)w.K + epi.eps);
+        }
+    }
     // wave v finishes (strip, output register) pairs v, v + waves, ...
     if (NS >= 2 && epi.kind == kEpiSwiglu) {       // strips 2j / 2j+1 of the group are gate / up of output strip (strip0 >> 1) + j
         const int n_out = w.N >> 1;
@@ -492,8 +620,8 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
             const int j = p >> 2, r = p & 3;
             const int nt = (strip0 >> 1) + j;
             const int n = nt * 16 + (lane & 15);
-            const float g = sum_partials(red + ((2 * j) * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64);
-            const float u = sum_partials(red + ((2 * j + 1) * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64);
+            const float g = sum_partials(red + ((2 * j) * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64) * rstd[r];
+            const float u = sum_partials(red + ((2 * j + 1) * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64) * rstd[r];
             const int m = 4 * oct + r;
             if (m < M && n < n_out) store_out(y, ydt, (int64_t)m * n_out + n, silu_mul(g, u));
         }
@@ -503,7 +631,7 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
         const int s = p >> 2, r = p & 3;
         const int nt = strip0 + s;
         const int n = nt * 16 + (lane & 15);
-        const float v = sum_partials(red + (s * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64);
+        const float v = sum_partials(red + (s * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64) * rstd[r];
         const int m = 4 * oct + r;
         if (nt < w.NT && m < M && n < w.N) emit(y, ydt, epi, (int64_t)m * w.N + n, v);
     }
@@ -513,10 +641,14 @@ template <int BITS, int XMODE, int TS, int NS>
 hipError_t launch_rows_t(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
                          hipStream_t st)
 {
-    const size_t lds = (size_t)NS * nwaves * 4 * 64 * sizeof(float);
+    const size_t lds = (size_t)NS * nwaves * 4 * 64 * sizeof(float) + (size_t)nwaves * 16 * sizeof(float);
     const unsigned groups = (unsigned)((w.NT + NS - 1) / NS);
-    hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS>), dim3(groups), dim3(nwaves * 64), lds, st, w,
-                       reinterpret_cast<const uint16_t*>(x), M, y, ydt, epi);
+    if (epi.gamma)
+        hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS, true>), dim3(groups), dim3(nwaves * 64), lds, st, w,
+                           reinterpret_cast<const uint16_t*>(x), M, y, ydt, epi);
+    else
+        hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS, false>), dim3(groups), dim3(nwaves * 64), lds, st, w,
+                           reinterpret_cast<const uint16_t*>(x), M, y, ydt, epi);
     return hipGetLastError();
 }
 
@@ -547,7 +679,7 @@ int g_tune_waves = 0, g_tune_unroll = 0, g_tune_rows = 0;
 
 constexpr int kLdsBudget = 64 * 1024;
 
-template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT, int PAIR>
+template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT, int PAIR, bool NORM>
 hipError_t launch_p(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
                     hipStream_t st)
 {
@@ -566,8 +698,9 @@ hipError_t launch_p(const WeightView& w, const void* x, int M, void* y, int ydt,
     }
     int ldx = slab_tiles * kTileK + 8;
     const size_t xbytes = ((size_t)M * ldx * 2 * planes + 255) & ~(size_t)255;
-    const size_t lds = xbytes + (size_t)PAIR * nwaves * RMAX * 64 * sizeof(float);     // x, then the waves' partial sums
-    auto kern = gemv_kernel<BITS, XMODE, RMAX, U, ONESHOT, PAIR>;
+    // x, then the waves' partial sums, then 16 row sums of squares (folded RMSNorm)
+    const size_t lds = xbytes + (size_t)PAIR * nwaves * RMAX * 64 * sizeof(float) + 16 * sizeof(float);
+    auto kern = gemv_kernel<BITS, XMODE, RMAX, U, ONESHOT, PAIR, NORM>;
     static bool attr_set = false;
     if (!attr_set) {
         // M = 16 fp32 activations with 8 waves need 66 KB, just over the default cap
@@ -581,21 +714,21 @@ hipError_t launch_p(const WeightView& w, const void* x, int M, void* y, int ydt,
     return hipGetLastError();
 }
 
-template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT>
+template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT, bool NORM>
 hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
                     hipStream_t st)
 {
-    if (epi.kind == kEpiSwiglu) return launch_p<BITS, XMODE, RMAX, U, ONESHOT, 2>(w, x, M, y, ydt, nwaves, epi, st);
-    return launch_p<BITS, XMODE, RMAX, U, ONESHOT, 1>(w, x, M, y, ydt, nwaves, epi, st);
+    if (epi.kind == kEpiSwiglu) return launch_p<BITS, XMODE, RMAX, U, ONESHOT, 2, NORM>(w, x, M, y, ydt, nwaves, epi, st);
+    return launch_p<BITS, XMODE, RMAX, U, ONESHOT, 1, NORM>(w, x, M, y, ydt, nwaves, epi, st);
 }
 
-template <int BITS, int XMODE, int U, bool ONESHOT>
+template <int BITS, int XMODE, int U, bool ONESHOT, bool NORM = false>
 hipError_t launch_r(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
                     hipStream_t st)
 {
-    if (M == 1) return launch_t<BITS, XMODE, 1, U, ONESHOT>(w, x, M, y, ydt, nwaves, epi, st);
-    if (M == 2) return launch_t<BITS, XMODE, 2, U, ONESHOT>(w, x, M, y, ydt, nwaves, epi, st);
-    return launch_t<BITS, XMODE, 4, U, ONESHOT>(w, x, M, y, ydt, nwaves, epi, st);
+    if (M == 1) return launch_t<BITS, XMODE, 1, U, ONESHOT, NORM>(w, x, M, y, ydt, nwaves, epi, st);
+    if (M == 2) return launch_t<BITS, XMODE, 2, U, ONESHOT, NORM>(w, x, M, y, ydt, nwaves, epi, st);
+    return launch_t<BITS, XMODE, 4, U, ONESHOT, NORM>(w, x, M, y, ydt, nwaves, epi, st);
 }
 
 template <int BITS, int XMODE>
@@ -605,6 +738,7 @@ hipError_t launch_u(const WeightView& w, const void* x, int M, void* y, int ydt,
     const int planes = XMODE == XF32 ? 2 : 1;
     const bool one_slab = (int64_t)M * (w.KT * kTileK + 8) * 2 * planes <= kLdsBudget;
     const int per_wave = (w.KT + nwaves - 1) / nwaves;
+    if (epi.gamma) return launch_r<BITS, XMODE, 2, false, true>(w, x, M, y, ydt, nwaves, epi, st);    // folded RMSNorm
     if (one_slab && unroll == 0) {
         if (per_wave <= 2) return launch_r<BITS, XMODE, 2, true>(w, x, M, y, ydt, nwaves, epi, st);
         if (per_wave <= 4) return launch_r<BITS, XMODE, 4, true>(w, x, M, y, ydt, nwaves, epi, st);

@@ -172,6 +172,19 @@ int cybq_weight_fuse_pairs(cybq_ctx* ctx, const cybq_weight* gate, const cybq_we
 int cybq_matmul_ex(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M,
                    void* y, cybq_dtype ydt, cybq_epilogue epilogue, const void* residual, void* stream);
 
+/* cybq_matmul_ex with RMSNorm folded into the activation load (the norm in front of
+ * QKV and of the FFN - decide/pipeline.md:51):
+ *     rstd[m] = 1 / sqrt(mean_k x[m,k]^2 + eps)            (fp32, fixed summation order)
+ *     y       = epilogue( rstd[m] * sum_k round(x[m,k] * gamma[k]) * W[n,k] )
+ * x * gamma is formed in fp32 and rounded once to the kernel's operand type (the type
+ * of x; f16 for bf16 x in the FAST prefill mode; two f16 halves for fp32 x) - what an
+ * unfused norm writing 16-bit activations would round too, minus its rounding of rstd.
+ * gamma: [K] device pointer of type gdt.  The definition is the LlamaStyle one and this
+ * library's choice (the reference's is not visible in its tree). */
+int cybq_matmul_norm(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M,
+                     const void* gamma, cybq_dtype gdt, float eps, void* y, cybq_dtype ydt,
+                     cybq_epilogue epilogue, const void* residual, void* stream);
+
 /* cybq_matmul_many with an epilogue per node: epilogue[i] is a cybq_epilogue,
  * residual[i] its residual (NULL unless CYBQ_EPI_ADD); either array may be NULL
  * (= no epilogues). */

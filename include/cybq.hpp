@@ -43,6 +43,8 @@ struct QMatMulNode {
     int64_t M = 1, N = 0, K = 0;
     cybq_epilogue epilogue = CYBQ_EPI_NONE;   // fused op behind the linear
     std::string residual;                      // edge added to the output (CYBQ_EPI_ADD)
+    std::string norm_gamma;                    // edge holding gamma [K]: RMSNorm folded into the x load ("" = none)
+    float norm_eps = 1e-5f;
 };
 
 // A device buffer bound to an edge name: pointer, element type, rows.
@@ -133,6 +135,12 @@ public:
     {
         return wrap(cybq_matmul_ex(ctx_, w.get(), x, xdt, M, y, ydt, epilogue, residual, stream));
     }
+    Status matmul_norm(const Weight& w, const void* x, cybq_dtype xdt, int64_t M, const void* gamma, cybq_dtype gdt,
+                       float eps, void* y, cybq_dtype ydt, cybq_epilogue epilogue = CYBQ_EPI_NONE,
+                       const void* residual = nullptr, void* stream = nullptr)
+    {
+        return wrap(cybq_matmul_norm(ctx_, w.get(), x, xdt, M, gamma, gdt, eps, y, ydt, epilogue, residual, stream));
+    }
     Status dequant(const Weight& w, float* out, void* stream = nullptr)
     {
         return wrap(cybq_dequant(ctx_, w.get(), out, stream));
@@ -156,6 +164,12 @@ public:
                 return fail(CYBQ_ERR_INVALID, "residual edge not bound or of another type");
             res = ri->second.ptr;
         }
+        if (!node.norm_gamma.empty()) {
+            auto gi = edges.find(node.norm_gamma);
+            if (gi == edges.end()) return fail(CYBQ_ERR_INVALID, "gamma edge not bound");
+            return matmul_norm(*w, xi->second.ptr, xi->second.dtype, node.M, gi->second.ptr, gi->second.dtype, node.norm_eps,
+                               yi->second.ptr, yi->second.dtype, node.epilogue, res, stream);
+        }
         return matmul_ex(*w, xi->second.ptr, xi->second.dtype, node.M, yi->second.ptr, yi->second.dtype, node.epilogue,
                          res, stream);
     }
@@ -177,6 +191,7 @@ public:
             if (!w || xi == edges.end() || yi == edges.end()) return fail(CYBQ_ERR_INVALID, "unresolved node '" + n.w + "'");
             if (xi->second.dtype != x0.dtype || yi->second.dtype != y0.dtype || n.M != nodes[0].M)
                 return fail(CYBQ_ERR_INVALID, "run_all needs one M and one dtype pair");
+            if (!n.norm_gamma.empty()) return fail(CYBQ_ERR_INVALID, "run_all does not take folded norms: use run()");
             const void* res = nullptr;
             if (n.epilogue == CYBQ_EPI_ADD) {
                 auto ri = edges.find(n.residual);

@@ -448,6 +448,69 @@ def test_epilogue_swiglu_full_size_and_split_k(backend, oracle):
         assert err < bar, (M, err)
 
 
+def _norm_ref(oracle, q, s, x, gamma, eps, op_dt):
+    """float64 restatement of the stated formula: x * gamma rounded once to the operand type,
+    exact matmul, rows scaled by rstd of the unrounded input."""
+    xf = x.float()
+    xg = xf * gamma.float()[None, :]
+    if op_dt == "f32":                                # two f16 halves keep ~22 bits: compare against unrounded
+        xr = xg.double().cpu().numpy()
+    else:
+        xr = xg.to(TDT[op_dt]).double().cpu().numpy()
+    rstd = 1.0 / np.sqrt((xf.double().cpu().numpy() ** 2).mean(axis=1) + eps)
+    return oracle.matmul_f64(q, s, xr) * rstd[:, None]
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M,xdt,gdt", [(1, "f16", "f16"), (2, "bf16", "f32"), (3, "f32", "f32"), (4, "f16", "bf16"), (9, "bf16", "bf16"),
+                                       (16, "f16", "f32"), (16, "f32", "f16"), (40, "bf16", "f32"), (300, "f16", "f16")])
+def test_folded_rmsnorm(backend, oracle, prefill_mode, bits, M, xdt, gdt):
+    N, K = 272, 1184                                   # K = 9 tiles + 1 group: a padded last tile
+    eps = 1e-5
+    q, s = _quant(oracle, bits, N, K)
+    qw = backend.upload_quantized(q, s, bits)
+    x = _x(M, K, xdt)
+    x[0] *= 7.0                                        # rows of different scale: rstd must be per row
+    gamma = (1.0 + 0.25 * torch.from_numpy(synth.activations(51, 1, K)[0])).cuda().to(TDT[gdt])
+    y = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    backend.matmul_norm(qw, x, gamma, eps, y)
+    torch.cuda.synchronize()
+    assert not torch.isnan(y).any()
+    fast_prefill = M > 16 and xdt != "f32" and prefill_mode == "fast"
+    op_dt = "f16" if (fast_prefill and xdt == "bf16") else xdt      # FAST multiplies in f16
+    ref = _norm_ref(oracle, q, s, x, gamma, eps, op_dt)
+    bar = FAST if fast_prefill else TIGHT
+    assert oracle.rel_l2(y.cpu().numpy(), ref) < bar
+    # reproducible, and composes with the epilogues
+    y2 = torch.empty_like(y)
+    backend.matmul_norm(qw, x, gamma, eps, y2)
+    r = torch.from_numpy(synth.activations(52, M, N)).cuda()
+    y3 = torch.empty_like(y)
+    backend.matmul_norm(qw, x, gamma, eps, y3, "add", r)
+    torch.cuda.synchronize()
+    assert torch.equal(y2, y)
+    assert torch.equal(y3, y + r)
+
+
+@pytest.mark.parametrize("M,xdt", [(1, "f16"), (8, "f16"), (64, "bf16")])
+def test_folded_rmsnorm_with_swiglu_and_long_k(backend, oracle, M, xdt):
+    # FFN entry as the decode loop has it: norm -> gate/up -> SwiGLU; K long enough for several x slabs
+    N, K = 192, 14336
+    eps = 1e-6
+    qg, sg = _quant(oracle, 4, N, K, cfg=45)
+    qu, su = _quant(oracle, 4, N, K, cfg=46)
+    wf = backend.fuse_pairs(backend.upload_quantized(qg, sg, 4), backend.upload_quantized(qu, su, 4))
+    x = _x(M, K, xdt)
+    gamma = (1.0 + 0.25 * torch.from_numpy(synth.activations(53, 1, K)[0])).cuda().to(torch.float32)
+    y = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    backend.matmul_norm(wf, x, gamma, eps, y, "swiglu")
+    torch.cuda.synchronize()
+    op_dt = "f16" if M > 16 else xdt
+    g = _norm_ref(oracle, qg, sg, x, gamma, eps, op_dt)
+    u = _norm_ref(oracle, qu, su, x, gamma, eps, op_dt)
+    assert oracle.rel_l2(y.cpu().numpy(), _silu_mul(g, u)) < (2 * FAST if M > 16 else TIGHT)
+
+
 def test_epilogue_errors(backend, oracle):
     q, s = _quant(oracle, 4, 64, 256)
     qw = backend.upload_quantized(q, s, 4)
