@@ -317,7 +317,6 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
         epi.residual = residual;
     } else if (epilogue == CYBQ_EPI_SWIGLU) {
         if (!w->paired) return fail(ctx, CYBQ_ERR_INVALID, "CYBQ_EPI_SWIGLU needs a weight made by cybq_weight_fuse_pairs");
-        if (xdt == CYBQ_F32 && M > 16) return fail(ctx, CYBQ_ERR_INVALID, "CYBQ_EPI_SWIGLU with fp32 activations is limited to M <= 16");
         epi.kind = cybq::kEpiSwiglu;
     } else if (epilogue != CYBQ_EPI_NONE) {
         return fail(ctx, CYBQ_ERR_INVALID, "unknown epilogue");
@@ -332,17 +331,20 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
     hipError_t e;
     if (M <= 16) {
         e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, epi, st);
-    } else if (xdt != CYBQ_F32) {
+    } else if (xdt != CYBQ_F32 && M > 32) {
         e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, ctx->workspace, ctx->workspace_bytes,
                               epi, st);
     } else {
         // fp32 activations keep full precision through the decode kernel's
-        // hi/lo split; prefill in fp32 is walked 16 rows at a time.
+        // hi/lo split; prefill in fp32 is walked 16 rows at a time.  So are 17..32
+        // rows of 16-bit activations: two passes of the batched-rows kernel stream the
+        // weights twice and are still quicker than a 128-row MFMA tile mostly empty.
         e = hipSuccess;
+        const int64_t n_out = epi.kind == cybq::kEpiSwiglu ? w->N / 2 : w->N;
         for (int64_t m0 = 0; m0 < M && e == hipSuccess; m0 += 16) {
             int mm = (int)((M - m0) < 16 ? (M - m0) : 16);
-            const char* xp = static_cast<const char*>(x) + (size_t)m0 * w->K * 4;
-            const size_t yoff = (size_t)m0 * w->N * dtype_size(ydt);
+            const char* xp = static_cast<const char*>(x) + (size_t)m0 * w->K * dtype_size(xdt);
+            const size_t yoff = (size_t)m0 * n_out * dtype_size(ydt);
             cybq::Epilogue ec = epi;
             if (epi.kind == cybq::kEpiAdd) ec.residual = static_cast<const char*>(residual) + yoff;
             e = cybq::launch_gemv(v, xp, xdt, mm, static_cast<char*>(y) + yoff, ydt, ctx->num_cus, ec, st);

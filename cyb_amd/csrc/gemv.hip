@@ -668,10 +668,12 @@ hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int y
         if (ns == 2) return launch_rows_t<BITS, XMODE, 2, 2>(w, x, M, y, ydt, nwaves, epi, st);
         return launch_rows_t<BITS, XMODE, 2, 1>(w, x, M, y, ydt, nwaves, epi, st);
     }
+    // (bf16 operands and Q8 tiles need more registers: four strips x four tiles would spill)
+    if (ns == 4 && (XMODE == XBF16 || BITS == 8)) return launch_rows_t<BITS, XMODE, 2, 4>(w, x, M, y, ydt, nwaves, epi, st);
     if (ns == 4) return launch_rows_t<BITS, XMODE, 4, 4>(w, x, M, y, ydt, nwaves, epi, st);
     if (ns == 2) return launch_rows_t<BITS, XMODE, 4, 2>(w, x, M, y, ydt, nwaves, epi, st);
     // one strip per workgroup and a long K: eight tiles per wave and slab, fewer round trips
-    if (w.KT > nwaves * 4) return launch_rows_t<BITS, XMODE, 8, 1>(w, x, M, y, ydt, nwaves, epi, st);
+    if (w.KT > nwaves * 4 && BITS == 4) return launch_rows_t<BITS, XMODE, 8, 1>(w, x, M, y, ydt, nwaves, epi, st);
     return launch_rows_t<BITS, XMODE, 4, 1>(w, x, M, y, ydt, nwaves, epi, st);
 }
 

@@ -74,8 +74,8 @@ typedef enum cybq_layout { CYBQ_LAYOUT_PLANAR = 0, CYBQ_LAYOUT_BLOCK_AOS = 1 } c
 
 typedef enum cybq_dtype { CYBQ_F32 = 0, CYBQ_F16 = 1, CYBQ_BF16 = 2 } cybq_dtype;
 
-/* How the prefill kernel (M > 16) feeds the matrix cores.  Both stay inside the
- * operator's 1e-3 relative-L2 tolerance; the decode kernel (M <= 16) is always exact.
+/* How the prefill kernel (M > 32) feeds the matrix cores.  Both stay inside the
+ * operator's 1e-3 relative-L2 tolerance; the decode kernels (M <= 32) are always exact.
  *   FAST   (default) one f16 MFMA per 32-group; the weight operand is
  *          round_f16(scale * q), relative error <= 2^-11 per weight (about 2e-4
  *          relative L2 on y).  bf16 activations are widened to f16 after a 2^-4
@@ -124,8 +124,10 @@ int cybq_weight_info(const cybq_weight* w, int* quant, int64_t* N, int64_t* K,
  * with fp32 accumulation.
  *   x  [M,K] row-major, xdt in {F16,BF16,F32}, 16-byte aligned
  *   y  [M,N] row-major, ydt in {F32,F16,BF16} (fp32 accumulator rounded once)
- *   M >= 1.  M <= 16 runs the HBM-streaming decode kernel, larger M the
- *   LDS-tiled MFMA prefill kernel; there is no other path. */
+ *   M >= 1.  M <= 16 runs the HBM-streaming decode kernels (17..32 rows: two
+ *   passes of them), larger M the LDS-tiled MFMA prefill kernel (fp32
+ *   activations: always the decode kernel, 16 rows at a time); there is no
+ *   other path. */
 int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt,
                 int64_t M, void* y, cybq_dtype ydt, void* stream);
 
@@ -167,8 +169,7 @@ int cybq_weight_fuse_pairs(cybq_ctx* ctx, const cybq_weight* gate, const cybq_we
 
 /* cybq_matmul with an epilogue.  `residual` is read only for CYBQ_EPI_ADD (device
  * pointer, may alias y).  CYBQ_EPI_SWIGLU needs a weight made by
- * cybq_weight_fuse_pairs and writes y[M, N/2].  fp32 activations support
- * CYBQ_EPI_NONE / CYBQ_EPI_ADD only for M <= 16. */
+ * cybq_weight_fuse_pairs and writes y[M, N/2]. */
 int cybq_matmul_ex(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M,
                    void* y, cybq_dtype ydt, cybq_epilogue epilogue, const void* residual, void* stream);
 

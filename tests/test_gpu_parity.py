@@ -249,8 +249,8 @@ def test_prefill_matches_oracle(backend, oracle, prefill_mode, bits, xdt, M):
     assert not np.isnan(y).any()
     err = oracle.rel_l2(y, oracle.matmul_f64(q, s, x.float().cpu().numpy()))
     assert err < (TIGHT if xdt == "f32" else _bar(prefill_mode)), err
-    if prefill_mode == "fast" and xdt != "f32":
-        assert err > 1e-6        # the rounded-weight kernel really ran
+    if prefill_mode == "fast" and xdt != "f32" and M > 32:
+        assert err > 1e-6        # the rounded-weight kernel really ran (up to 32 rows take the exact decode kernel)
 
 
 @pytest.mark.parametrize("shape", [(17, 32), (112, 160), (113, 96), (130, 2080)])
@@ -414,7 +414,7 @@ def test_epilogue_swiglu(backend, oracle, prefill_mode, bits, M, xdt):
     bar = TIGHT if (M <= 16 or xdt == "f32") else 2 * _bar(prefill_mode)
     assert oracle.rel_l2(y.cpu().numpy(), _silu_mul(g, u)) < bar
     # the fused weight as a plain matmul: gate and up columns interleaved in blocks of 16
-    if xdt != "f32" or M <= 16:
+    if True:
         yi = _run(backend, wf, x)
         yg, yu = _run(backend, wg, x), _run(backend, wu, x)
         inter = torch.stack([yg.view(M, N // 16, 16), yu.view(M, N // 16, 16)], dim=2).reshape(M, 2 * N)
@@ -476,7 +476,7 @@ def test_folded_rmsnorm(backend, oracle, prefill_mode, bits, M, xdt, gdt):
     backend.matmul_norm(qw, x, gamma, eps, y)
     torch.cuda.synchronize()
     assert not torch.isnan(y).any()
-    fast_prefill = M > 16 and xdt != "f32" and prefill_mode == "fast"
+    fast_prefill = M > 32 and xdt != "f32" and prefill_mode == "fast"
     op_dt = "f16" if (fast_prefill and xdt == "bf16") else xdt      # FAST multiplies in f16
     ref = _norm_ref(oracle, q, s, x, gamma, eps, op_dt)
     bar = FAST if fast_prefill else TIGHT
