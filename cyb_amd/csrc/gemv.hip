@@ -661,12 +661,18 @@ hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int y
     int ns = (w.NT + num_cus / 2) / num_cus;
     ns = ns >= 3 ? 4 : (ns >= 2 ? 2 : 1);
     if (epi.kind == kEpiSwiglu && ns < 2) ns = 2;          // a gate strip and its up strip share a workgroup
+    // seven strips per workgroup when that is exactly one workgroup per CU (N = 28672 on 256 CUs:
+    // with four strips the 448 workgroups need a second, mostly empty round); SwiGLU pairs need an even count
+    const bool seven = w.NT == 7 * num_cus && epi.kind != kEpiSwiglu && !epi.gamma;
     int nwaves = tuned_waves > 0 ? tuned_waves : 8;
     while (nwaves > 1 && nwaves * 2 > w.KT) nwaves >>= 1;
     if (nwaves > 8) {          // 16 waves: 128 registers per lane, two tiles of x in flight
         if (ns == 4) return launch_rows_t<BITS, XMODE, 2, 4>(w, x, M, y, ydt, nwaves, epi, st);
         if (ns == 2) return launch_rows_t<BITS, XMODE, 2, 2>(w, x, M, y, ydt, nwaves, epi, st);
         return launch_rows_t<BITS, XMODE, 2, 1>(w, x, M, y, ydt, nwaves, epi, st);
+    }
+    if constexpr (XMODE == XF16 && BITS == 4) {
+        if (seven && nwaves <= 8) return launch_rows_t<BITS, XMODE, 4, 7>(w, x, M, y, ydt, nwaves, epi, st);
     }
     // (bf16 operands and Q8 tiles need more registers: four strips x four tiles would spill)
     if (ns == 4 && (XMODE == XBF16 || BITS == 8)) return launch_rows_t<BITS, XMODE, 2, 4>(w, x, M, y, ydt, nwaves, epi, st);

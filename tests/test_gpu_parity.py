@@ -114,6 +114,22 @@ def test_decode_ragged_shapes(backend, oracle, shape):
         assert oracle.rel_l2(y, oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT
 
 
+def test_decode_seven_strips_per_workgroup(backend, oracle):
+    # N = 7 * 16 * 256: on a 256-CU part the batched-rows kernel gives every workgroup seven strips
+    N, K = 28672, 256
+    q, s = _quant(oracle, 4, N, K)
+    qw = backend.upload_quantized(q, s, 4)
+    for M in (4, 16):
+        x = _x(M, K, "f16")
+        y = _run(backend, qw, x).cpu().numpy()
+        assert oracle.rel_l2(y, oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT
+    r = torch.from_numpy(synth.activations(34, 16, N)).cuda()
+    y2 = torch.empty((16, N), dtype=torch.float32, device="cuda")
+    backend.matmul_ex(qw, x, y2, "add", r)
+    torch.cuda.synchronize()
+    assert torch.equal(y2, torch.from_numpy(y).cuda() + r)
+
+
 def test_decode_long_k_uses_several_slabs(backend, oracle):
     # M * K * 2 B exceeds the kernel's LDS budget: x is staged slab by slab
     N, K = 64, 14336
