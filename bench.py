@@ -28,8 +28,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 MALL_BYTES = 256 << 20
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain
 # 256 MiB copy: FETCH x 1.9997, WRITE x 1.0000); profiles/decode_gemv_q4_4096x14336_m1.md
-TRAFFIC_DECODE_BYTES = 33_280_700
-TRAFFIC_PREFILL_M512_BYTES = 121_787_300     # multiply 113.4 MB + activation staging pass 8.4 MB
+TRAFFIC_DECODE_BYTES = 33_270_500
+TRAFFIC_PREFILL_M512_BYTES = 121_950_000     # multiply 113.5 MB + activation staging pass 8.4 MB
 
 
 def log(*a):
