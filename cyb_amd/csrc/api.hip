@@ -307,7 +307,7 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
     cybq::Epilogue epi = {cybq::kEpiNone, nullptr, nullptr, 0, 0.f};
     if (gamma) {
         if (!dtype_ok(gdt)) return fail(ctx, CYBQ_ERR_INVALID, "unknown gamma dtype");
-        if (reinterpret_cast<uintptr_t>(gamma) % dtype_size(gdt)) return fail(ctx, CYBQ_ERR_ALIGN, "gamma is not aligned to its element size");
+        if (!aligned16(gamma)) return fail(ctx, CYBQ_ERR_ALIGN, "gamma must be 16-byte aligned");
         if (!(eps >= 0.f)) return fail(ctx, CYBQ_ERR_INVALID, "eps must be >= 0");
     }
     if (epilogue == CYBQ_EPI_ADD) {

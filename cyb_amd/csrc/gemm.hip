@@ -91,6 +91,33 @@ __device__ __forceinline__ float rstd_of(const NormStats& ns, int row, int K, fl
     return 1.0f / sqrtf(t / (float)K + eps);
 }
 
+// gamma[k0 .. k0+8) as fp32 (k0 a multiple of 8, gamma 16-byte aligned)
+__device__ __forceinline__ void load_gamma8_g(const void* g, int gdt, int k0, float out[8])
+{
+    if (gdt == kF32) {
+        const float4_t* p = reinterpret_cast<const float4_t*>(reinterpret_cast<const float*>(g) + k0);
+        const float4_t a = p[0], b = p[1];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            out[i] = a[i];
+            out[4 + i] = b[i];
+        }
+    } else {
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const uint16_t*>(g) + k0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if (gdt == kF16) {
+                const half2_t h = as_h2(v[i]);
+                out[2 * i] = (float)h.x;
+                out[2 * i + 1] = (float)h.y;
+            } else {
+                out[2 * i] = __builtin_bit_cast(float, v[i] << 16);
+                out[2 * i + 1] = __builtin_bit_cast(float, v[i] & 0xffff0000u);
+            }
+        }
+    }
+}
+
 template <int BITS>
 struct WRegs {               // one native weight tile as loaded by one lane, and its 4 group scales
     u32x4_t q[BITS == 4 ? 1 : 2];
@@ -526,6 +553,8 @@ __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict_
         if (NORM) {
             float sq = 0.f;
             if (c < K8) {
+                float g[8];
+                load_gamma8_g(epi.gamma, epi.gamma_dt, c * 8, g);
 #pragma unroll
                 for (int p = 0; p < 4; p++) {
                     float v0, v1;
@@ -539,8 +568,8 @@ __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict_
                     }
                     sq = fmaf(v1, v1, fmaf(v0, v0, sq));
                     const float sc = WIDEN ? 0.0625f : 1.0f;
-                    v0 *= load_out_g(epi.gamma, epi.gamma_dt, c * 8 + 2 * p) * sc;
-                    v1 *= load_out_g(epi.gamma, epi.gamma_dt, c * 8 + 2 * p + 1) * sc;
+                    v0 *= g[2 * p] * sc;
+                    v1 *= g[2 * p + 1] * sc;
                     if (XBF && !WIDEN) {
                         a.u[p] = (uint32_t)f32_to_bf16_rne_g(v0) | ((uint32_t)f32_to_bf16_rne_g(v1) << 16);
                     } else {

@@ -261,61 +261,138 @@ __device__ __forceinline__ float sum_partials(const float* red, int nwaves, int 
 }
 
 // ---- RMSNorm folded into the staged x (LDS kernel) ------------------------------
-__device__ __forceinline__ float load_gamma(const void* g, int gdt, int k)
+// gamma[k0 .. k0+8) as fp32 (k0 a multiple of 8; gamma is 16-byte aligned at such k for f32 and 16-bit types)
+__device__ __forceinline__ void load_gamma8(const void* g, int gdt, int k0, float out[8])
 {
-    if (gdt == kF32) return reinterpret_cast<const float*>(g)[k];
-    if (gdt == kF16) return (float)reinterpret_cast<const _Float16*>(g)[k];
-    return __builtin_bit_cast(float, (uint32_t)reinterpret_cast<const uint16_t*>(g)[k] << 16);
-}
-
-// value k of a staged row as fp32 (XF32: hi + lo planes)
-template <int XMODE>
-__device__ __forceinline__ float staged_x(const uint16_t* row, int plane_elems, int k)
-{
-    if (XMODE == XBF16) return __builtin_bit_cast(float, (uint32_t)row[k] << 16);
-    float v = (float)reinterpret_cast<const _Float16*>(row)[k];
-    if (XMODE == XF32) v += (float)reinterpret_cast<const _Float16*>(row + plane_elems)[k];
-    return v;
-}
-
-template <int XMODE>
-__device__ __forceinline__ void store_staged_x(uint16_t* row, int plane_elems, int k, float v)
-{
-    if (XMODE == XBF16) {
-        row[k] = f32_to_bf16_rne(v);
+    if (gdt == kF32) {
+        const float4_t* p = reinterpret_cast<const float4_t*>(reinterpret_cast<const float*>(g) + k0);
+        const float4_t a = p[0], b = p[1];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            out[i] = a[i];
+            out[4 + i] = b[i];
+        }
     } else {
-        const _Float16 h = (_Float16)v;
-        reinterpret_cast<_Float16*>(row)[k] = h;
-        if (XMODE == XF32) reinterpret_cast<_Float16*>(row + plane_elems)[k] = (_Float16)(v - (float)h);
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const uint16_t*>(g) + k0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if (gdt == kF16) {
+                const half2_t h = as_h2(v[i]);
+                out[2 * i] = (float)h.x;
+                out[2 * i + 1] = (float)h.y;
+            } else {
+                out[2 * i] = __builtin_bit_cast(float, v[i] << 16);
+                out[2 * i + 1] = __builtin_bit_cast(float, v[i] & 0xffff0000u);
+            }
+        }
     }
 }
 
-// One staged K slab: adds this slab's sum of squares of every row to ssq[row] (row m
-// belongs to wave m % waves; lanes stride over k, then a fixed butterfly: the order of
-// the additions never changes), then replaces x by x * gamma.  Two barriers inside.
+// eight staged values (one 16 B piece of a row) as fp32, and back
+template <int XMODE>
+__device__ __forceinline__ void staged_piece(const uint16_t* row, int plane_elems, int c, float out[8])
+{
+    const u32x4_t v = reinterpret_cast<const u32x4_t*>(row)[c];
+    u32x4_t lo = {0u, 0u, 0u, 0u};
+    if (XMODE == XF32) lo = reinterpret_cast<const u32x4_t*>(row + plane_elems)[c];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        if (XMODE == XBF16) {
+            out[2 * i] = __builtin_bit_cast(float, v[i] << 16);
+            out[2 * i + 1] = __builtin_bit_cast(float, v[i] & 0xffff0000u);
+        } else {
+            const half2_t h = as_h2(v[i]);
+            out[2 * i] = (float)h.x;
+            out[2 * i + 1] = (float)h.y;
+            if (XMODE == XF32) {
+                const half2_t l = as_h2(lo[i]);
+                out[2 * i] += (float)l.x;
+                out[2 * i + 1] += (float)l.y;
+            }
+        }
+    }
+}
+
+template <int XMODE>
+__device__ __forceinline__ void store_staged_piece(uint16_t* row, int plane_elems, int c, const float in[8])
+{
+    u32x4_t v, lo;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        if (XMODE == XBF16) {
+            v[i] = (uint32_t)f32_to_bf16_rne(in[2 * i]) | ((uint32_t)f32_to_bf16_rne(in[2 * i + 1]) << 16);
+        } else {
+            const half2_t h = {(_Float16)in[2 * i], (_Float16)in[2 * i + 1]};
+            v[i] = as_u32(h);
+            if (XMODE == XF32) {
+                const half2_t l = {(_Float16)(in[2 * i] - (float)h.x), (_Float16)(in[2 * i + 1] - (float)h.y)};
+                lo[i] = as_u32(l);
+            }
+        }
+    }
+    reinterpret_cast<u32x4_t*>(row)[c] = v;
+    if (XMODE == XF32) reinterpret_cast<u32x4_t*>(row + plane_elems)[c] = lo;
+}
+
+// One staged K slab: adds this slab's sum of squares of every row to ssq[row] and replaces
+// x by x * gamma, in 16 B pieces (ldx, slab_k and K are multiples of 8).  Every thread
+// takes pieces tid, tid + threads, ... of each row; lanes meet in a fixed butterfly, waves
+// through `part` in wave order: the order of the additions never changes.  Two barriers inside.
+// gamma of the first two pieces a thread will scale (pieces tid and tid + threads of every row),
+// requested together with x so that it is there when the slab is staged
+struct GammaPre {
+    float g[2][8];
+};
+__device__ __forceinline__ void prefetch_gamma(GammaPre& gp, const Epilogue& epi, int slab_k, int k_begin, int K, int tid,
+                                               int nthreads)
+{
+    const int pieces = max(min(slab_k, K - k_begin) >> 3, 1);
+    load_gamma8(epi.gamma, epi.gamma_dt, k_begin + min(tid, pieces - 1) * 8, gp.g[0]);
+    load_gamma8(epi.gamma, epi.gamma_dt, k_begin + min(tid + nthreads, pieces - 1) * 8, gp.g[1]);
+}
+
 template <int XMODE>
 __device__ __forceinline__ void norm_staged_slab(uint16_t* xs, int M, int slab_k, int k_begin, int K, int ldx,
-                                                 int plane_elems, const Epilogue& epi, float* ssq, int tid,
-                                                 int nthreads)
+                                                 int plane_elems, const Epilogue& epi, const GammaPre& gp, float* ssq,
+                                                 float* part, int tid, int nthreads)
 {
     const int lane = tid & 63, wv = tid >> 6, nw = nthreads >> 6;
-    const int kk = min(slab_k, K - k_begin);
-    for (int m = wv; m < M; m += nw) {
+    const int pieces = min(slab_k, K - k_begin) >> 3;
+    for (int m = 0; m < M; m++) {
         const uint16_t* row = xs + m * ldx;
         float a = 0.f;
-        for (int k = lane; k < kk; k += 64) {
-            const float v = staged_x<XMODE>(row, plane_elems, k);
-            a = fmaf(v, v, a);
+        for (int c = tid; c < pieces; c += nthreads) {
+            float v[8];
+            staged_piece<XMODE>(row, plane_elems, c, v);
+#pragma unroll
+            for (int i = 0; i < 8; i++) a = fmaf(v[i], v[i], a);
         }
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) a += __shfl_xor(a, off, 64);
-        if (lane == 0) ssq[m] += a;
+        if (lane == 0) part[m * 16 + wv] = a;
     }
     __syncthreads();
-    for (int i = tid; i < M * kk; i += nthreads) {
-        const int m = i / kk, k = i - m * kk;
+    if (tid < M) {
+        float t = ssq[tid];
+        for (int k = 0; k < nw; k++) t += part[tid * 16 + k];
+        ssq[tid] = t;
+    }
+    for (int m = 0; m < M; m++) {
         uint16_t* row = xs + m * ldx;
-        store_staged_x<XMODE>(row, plane_elems, k, staged_x<XMODE>(row, plane_elems, k) * load_gamma(epi.gamma, epi.gamma_dt, k_begin + k));
+        int it = 0;
+        for (int c = tid; c < pieces; c += nthreads, it++) {
+            float v[8], g[8];
+            staged_piece<XMODE>(row, plane_elems, c, v);
+            if (it < 2) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) g[i] = it == 0 ? gp.g[0][i] : gp.g[1][i];
+            } else {
+                load_gamma8(epi.gamma, epi.gamma_dt, k_begin + c * 8, g);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] *= g[i];
+            store_staged_piece<XMODE>(row, plane_elems, c, v);
+        }
     }
     __syncthreads();
 }
@@ -355,6 +432,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
 
     // folded RMSNorm: per-row sums of squares live behind the partial sums
     float* ssq = reinterpret_cast<float*>(smem + red_offset) + PAIR * nwaves * RMAX * 64;
+    float* ssq_part = ssq + 16;                      // [row][wave] partial sums of squares
     if (NORM && tid < 16) ssq[tid] = 0.f;            // (ordered before its first use by the staging barrier)
 
     if (ONESHOT) {
@@ -362,10 +440,12 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
         XRegs<XMODE> xr;
         stage_x_rest<XMODE, RMAX == 1>(xs, x, M, w.K, 0, w.KT * kTileK, ldx, plane_elems, tid, nthreads);
         stage_x_load<XMODE, RMAX == 1>(xr, x, M, w.K, 0, w.KT * kTileK, 0, tid, nthreads);
+        GammaPre gp;
+        if (NORM) prefetch_gamma(gp, epi, w.KT * kTileK, 0, w.K, tid, nthreads);
         load_batch<BITS, U>(buf, w, strip, wv, nwaves, w.KT, lane);
         stage_x_store<XMODE, RMAX == 1>(xr, xs, M, w.KT * kTileK, ldx, plane_elems, 0, tid, nthreads);
         __syncthreads();
-        if (NORM) norm_staged_slab<XMODE>(xs, M, w.KT * kTileK, 0, w.K, ldx, plane_elems, epi, ssq, tid, nthreads);
+        if (NORM) norm_staged_slab<XMODE>(xs, M, w.KT * kTileK, 0, w.K, ldx, plane_elems, epi, gp, ssq, ssq_part, tid, nthreads);
         const uint16_t* xbase = xs + mrow * ldx + oct * 8;
         compute_batch<BITS, XMODE, RMAX, U>(buf, wv, nwaves, w.KT, xbase, plane_elems, magic, acc);
     } else {
@@ -379,11 +459,13 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
             XRegs<XMODE> xr;
             stage_x_rest<XMODE, RMAX == 1>(xs, x, M, w.K, slab0 * kTileK, st * kTileK, ldx, plane_elems, tid, nthreads);
             stage_x_load<XMODE, RMAX == 1>(xr, x, M, w.K, slab0 * kTileK, st * kTileK, 0, tid, nthreads);
+            GammaPre gp;
+            if (NORM) prefetch_gamma(gp, epi, st * kTileK, slab0 * kTileK, w.K, tid, nthreads);
             load_batch<BITS, U>(bufA, w, base, wv, nwaves, st, lane);
             stage_x_store<XMODE, RMAX == 1>(xr, xs, M, st * kTileK, ldx, plane_elems, 0, tid, nthreads);
             __syncthreads();
             if (NORM)
-                norm_staged_slab<XMODE>(xs, M, st * kTileK, slab0 * kTileK, w.K, ldx, plane_elems, epi, ssq, tid, nthreads);
+                norm_staged_slab<XMODE>(xs, M, st * kTileK, slab0 * kTileK, w.K, ldx, plane_elems, epi, gp, ssq, ssq_part, tid, nthreads);
 
             const uint16_t* xbase = xs + mrow * ldx + oct * 8;
             for (int i0 = wv; i0 < st; i0 += 2 * stride) {
@@ -465,8 +547,18 @@ __device__ __forceinline__ void tile_issue_regs(const TileRegs<BITS>& t, const F
 // is multiplied by gamma in registers right after it reaches operand order, the lane adds
 // the squares of what it holds; rows meet across lanes and waves in the final exchange.
 template <int XMODE>
-__device__ __forceinline__ void norm_frag(Frag16& a, const Epilogue& epi, int k0, bool counts, float& ssq)
+__device__ __forceinline__ void norm_frag(Frag16& a, const float* gamma_lds, int k0, bool counts, float& ssq)
 {
+    float g[8];
+    {
+        const float4_t g0 = reinterpret_cast<const float4_t*>(gamma_lds + k0)[0];
+        const float4_t g1 = reinterpret_cast<const float4_t*>(gamma_lds + k0)[1];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            g[i] = g0[i];
+            g[4 + i] = g1[i];
+        }
+    }
 #pragma unroll
     for (int p = 0; p < 4; p++) {
         float v0, v1;
@@ -479,8 +571,8 @@ __device__ __forceinline__ void norm_frag(Frag16& a, const Epilogue& epi, int k0
             v1 = (float)h.y;
         }
         if (counts) ssq = fmaf(v1, v1, fmaf(v0, v0, ssq));
-        v0 *= load_gamma(epi.gamma, epi.gamma_dt, k0 + 2 * p);
-        v1 *= load_gamma(epi.gamma, epi.gamma_dt, k0 + 2 * p + 1);
+        v0 *= g[2 * p];
+        v1 *= g[2 * p + 1];
         if (XMODE == XBF16) {
             a.u[p] = (uint32_t)f32_to_bf16_rne(v0) | ((uint32_t)f32_to_bf16_rne(v1) << 16);
         } else {
@@ -510,6 +602,18 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
     // order directly costs 64 separate accesses per load instead of 16.
     const uint16_t* xrow = x + (int64_t)min(lane >> 2, M - 1) * w.K + (lane & 3) * 8;
     const int from_lane = (((lane & 15) << 2) | oct) << 2;       // byte address for ds_bpermute
+    // NORM: gamma as fp32 in LDS behind the exchange areas (read per fragment with LDS loads, which
+    // do not queue behind the weight requests the way global loads would)
+    float* gamma_lds = reinterpret_cast<float*>(smem) + NS * nwaves * 4 * 64 + nwaves * 16;
+    if (NORM) {
+        for (int c = tid; c < (w.K >> 3); c += (int)blockDim.x) {
+            float g[8];
+            load_gamma8(epi.gamma, epi.gamma_dt, c * 8, g);
+            reinterpret_cast<float4_t*>(gamma_lds + c * 8)[0] = (float4_t){g[0], g[1], g[2], g[3]};
+            reinterpret_cast<float4_t*>(gamma_lds + c * 8)[1] = (float4_t){g[4], g[5], g[6], g[7]};
+        }
+        __syncthreads();
+    }
 
     float acc[NS][4];
 #pragma unroll
@@ -560,7 +664,7 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     const int kg = kt[u] * kTileK + j * 32;            // (a group past K repeats the last one: not counted)
-                    norm_frag<XMODE>(a[u][j], epi, min(kg, w.K - 32) + oct * 8, valid[u] && kg < w.K, ssq);
+                    norm_frag<XMODE>(a[u][j], gamma_lds, min(kg, w.K - 32) + oct * 8, valid[u] && kg < w.K, ssq);
                 }
         }
 #pragma unroll
@@ -641,12 +745,22 @@ template <int BITS, int XMODE, int TS, int NS>
 hipError_t launch_rows_t(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
                          hipStream_t st)
 {
-    const size_t lds = (size_t)NS * nwaves * 4 * 64 * sizeof(float) + (size_t)nwaves * 16 * sizeof(float);
+    size_t lds = (size_t)NS * nwaves * 4 * 64 * sizeof(float) + (size_t)nwaves * 16 * sizeof(float);
     const unsigned groups = (unsigned)((w.NT + NS - 1) / NS);
-    if (epi.gamma)
-        hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS, true>), dim3(groups), dim3(nwaves * 64), lds, st, w,
-                           reinterpret_cast<const uint16_t*>(x), M, y, ydt, epi);
-    else
+    if (epi.gamma) {
+        lds += (size_t)w.K * sizeof(float);            // gamma as fp32
+        auto kern = gemv_rows_kernel<BITS, XMODE, TS, NS, true>;
+        static bool attr_set = false;
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               150 * 1024);
+            if (e != hipSuccess) return e;
+            attr_set = true;
+        }
+        if (lds > 150 * 1024) return hipErrorInvalidValue;      // K beyond ~30 k with a folded norm
+        hipLaunchKernelGGL(kern, dim3(groups), dim3(nwaves * 64), lds, st, w, reinterpret_cast<const uint16_t*>(x), M, y, ydt,
+                           epi);
+    } else
         hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS, false>), dim3(groups), dim3(nwaves * 64), lds, st, w,
                            reinterpret_cast<const uint16_t*>(x), M, y, ydt, epi);
     return hipGetLastError();
@@ -663,7 +777,7 @@ hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int y
     if (epi.kind == kEpiSwiglu && ns < 2) ns = 2;          // a gate strip and its up strip share a workgroup
     // seven strips per workgroup when that is exactly one workgroup per CU (N = 28672 on 256 CUs:
     // with four strips the 448 workgroups need a second, mostly empty round); SwiGLU pairs need an even count
-    const bool seven = w.NT == 7 * num_cus && epi.kind != kEpiSwiglu && !epi.gamma;
+    const bool seven = w.NT == 7 * num_cus && epi.kind != kEpiSwiglu;
     int nwaves = tuned_waves > 0 ? tuned_waves : 8;
     while (nwaves > 1 && nwaves * 2 > w.KT) nwaves >>= 1;
     if (nwaves > 8) {          // 16 waves: 128 registers per lane, two tiles of x in flight
@@ -706,8 +820,8 @@ hipError_t launch_p(const WeightView& w, const void* x, int M, void* y, int ydt,
     }
     int ldx = slab_tiles * kTileK + 8;
     const size_t xbytes = ((size_t)M * ldx * 2 * planes + 255) & ~(size_t)255;
-    // x, then the waves' partial sums, then 16 row sums of squares (folded RMSNorm)
-    const size_t lds = xbytes + (size_t)PAIR * nwaves * RMAX * 64 * sizeof(float) + 16 * sizeof(float);
+    // x, then the waves' partial sums, then 16 row sums of squares and their 16 x 16 per-wave parts (folded RMSNorm)
+    const size_t lds = xbytes + (size_t)PAIR * nwaves * RMAX * 64 * sizeof(float) + (16 + 256) * sizeof(float);
     auto kern = gemv_kernel<BITS, XMODE, RMAX, U, ONESHOT, PAIR, NORM>;
     static bool attr_set = false;
     if (!attr_set) {

@@ -180,7 +180,7 @@ int cybq_matmul_ex(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtyp
  * x * gamma is formed in fp32 and rounded once to the kernel's operand type (the type
  * of x; f16 for bf16 x in the FAST prefill mode; two f16 halves for fp32 x) - what an
  * unfused norm writing 16-bit activations would round too, minus its rounding of rstd.
- * gamma: [K] device pointer of type gdt.  The definition is the LlamaStyle one and this
+ * gamma: [K] device pointer of type gdt, 16-byte aligned.  The definition is the LlamaStyle one and this
  * library's choice (the reference's is not visible in its tree). */
 int cybq_matmul_norm(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M,
                      const void* gamma, cybq_dtype gdt, float eps, void* y, cybq_dtype ydt,
