@@ -510,18 +510,18 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
 }
 
 // ---------------------------------------------------------------------------
-// Batch rows 5..16: x operands live in REGISTERS and are reused across strips.
+// Batch rows 4..16: x operands live in REGISTERS and are reused across strips.
 //
 // With more than a few batch rows the LDS kernel above spends its time moving
 // x: every 16-row strip's workgroup stages all M rows of x (128 KB at M = 16,
 // K = 4096, against 37 KB of weights).  Here a workgroup owns NS consecutive
-// strips; each wave loads the A operands of ITS K tiles once (lane = batch row
-// l%16, 8 k per lane: a 16 B global load per lane per scale group, no LDS, no
-// barrier), requests the weight tiles of all NS strips at once and walks over
-// the strips with the same operands.  Tile kt belongs
-// to wave kt % waves and partials are summed in wave order: deterministic, and a
-// row's bits do not depend on the batch it is part of (within this kernel; the
-// LDS kernel may split K over a different number of waves).
+// strips; each wave loads the x of ITS K tiles once (coalesced, then moved across
+// lanes into A-operand order: lane = batch row l%16, k octet l/16; no LDS
+// staging, no barrier), requests the weight tiles two strips ahead and walks over
+// the strips with the same operands.  Tile kt belongs to wave kt % waves and
+// partials are summed in wave order: deterministic, and a row's bits do not depend
+// on the batch it is part of (within this kernel; the LDS kernel may split K over
+// a different number of waves).
 template <int BITS, int XMODE>
 __device__ __forceinline__ void tile_issue_regs(const TileRegs<BITS>& t, const Frag16 (&a)[4], uint32_t magic,
                                                 float4_t d[4])
