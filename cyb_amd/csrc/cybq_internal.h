@@ -17,13 +17,14 @@ hipError_t launch_repack(int bits, int layout, const void* q, const void* scales
                          uint16_t* sdst, int N, int K, int NT, int KT, hipStream_t st);
 hipError_t launch_dequant(const WeightView& w, float* out, hipStream_t st);
 
-// decode path, 1 <= M <= 16
+// decode path, 1 <= M <= 16 per call (api.hip walks 17..32 rows as two calls)
 hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
                        int num_cus, const Epilogue& epi, hipStream_t st);
-// prefill path, M > 16
+// prefill path (api.hip sends 16-bit activations with M > 32 here)
 // exact: two MFMAs per group with losslessly split weights; otherwise one f16 MFMA
 // per group with weights rounded once to f16
-// workspace: device scratch owned by the context (FAST mode widens bf16 X into it)
+// workspace: device scratch owned by the context (activations restaged in MFMA operand
+// order, fp32 slabs of a K split, per-row statistics of a folded norm)
 hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
                        int num_cus, bool exact, void* workspace, size_t workspace_bytes, const Epilogue& epi,
                        hipStream_t st);
