@@ -527,6 +527,79 @@ def test_folded_rmsnorm_with_swiglu_and_long_k(backend, oracle, M, xdt):
     assert oracle.rel_l2(y.cpu().numpy(), _silu_mul(g, u)) < (2 * FAST if M > 16 else TIGHT)
 
 
+def _random_cases(seed, count):
+    """Seeded draws over everything a call can vary in: block type, interchange layout, ragged N / K,
+    batch rows on both sides of every kernel boundary, the three activation types, output type,
+    epilogue, folded norm, prefill mode.  CYBQ_FUZZ_SEED / CYBQ_FUZZ_COUNT widen the sweep by hand."""
+    rng = np.random.default_rng(seed)
+    rows = [1, 2, 3, 4, 5, 8, 13, 16, 17, 24, 31, 32, 33, 48, 100, 129, 257, 300]
+    cases = []
+    for i in range(count):
+        epi = ["none", "add", "swiglu"][int(rng.integers(0, 3))]
+        N = int(rng.integers(1, 30)) * 16 if epi == "swiglu" else int(rng.integers(1, 500))
+        K = 32 * int(rng.integers(1, 150)) if rng.random() < 0.8 else 32 * int(rng.integers(150, 600))
+        cases.append(dict(i=i, bits=int(rng.choice([4, 8])), layout=int(rng.choice([formats.PLANAR, formats.BLOCK_AOS])),
+                          N=N, K=K, M=int(rng.choice(rows)), xdt=str(rng.choice(["f16", "bf16", "f32"])),
+                          ydt=str(rng.choice(["f32", "f32", "f16", "bf16"])), epi=epi, norm=bool(rng.random() < 0.4),
+                          gdt=str(rng.choice(["f32", "f16", "bf16"])), mode=str(rng.choice(["fast", "exact"]))))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_cases(int(__import__("os").environ.get("CYBQ_FUZZ_SEED", "20240607")), int(__import__("os").environ.get("CYBQ_FUZZ_COUNT", "72"))), ids=lambda c: "-".join(str(v) for v in c.values()))
+def test_random_calls_match_float64(backend, oracle, case):
+    c = case
+    bits, N, K, M = c["bits"], c["N"], c["K"], c["M"]
+    backend.set_prefill_mode(c["mode"])
+    try:
+        x = _x(M, K, c["xdt"], cfg=60 + c["i"])
+        if M > 1:
+            x[M // 2] *= 5.0
+        gamma = (1.0 + 0.25 * torch.from_numpy(synth.activations(61, 1, K)[0])).cuda().to(TDT[c["gdt"]])
+        eps = 1e-5
+        prefill = M > 32 and c["xdt"] != "f32"
+        fast = prefill and c["mode"] == "fast"
+        op_dt = "f16" if (fast and c["xdt"] == "bf16") else c["xdt"]
+
+        def product(q, s):
+            if c["norm"]:
+                return _norm_ref(oracle, q, s, x, gamma, eps, op_dt)
+            return oracle.matmul_f64(q, s, x.float().cpu().numpy())
+
+        if c["epi"] == "swiglu":
+            qg, sg = _quant(oracle, bits, N, K, cfg=70 + c["i"])
+            qu, su = _quant(oracle, bits, N, K, cfg=170 + c["i"])
+            w = backend.fuse_pairs(backend.upload_quantized(qg, sg, bits, c["layout"]),
+                                   backend.upload_quantized(qu, su, bits, c["layout"]))
+            ref = _silu_mul(product(qg, sg), product(qu, su))
+        else:
+            q, s = _quant(oracle, bits, N, K, cfg=70 + c["i"])
+            w = backend.upload_quantized(q, s, bits, c["layout"])
+            ref = product(q, s)
+        r = None
+        if c["epi"] == "add":
+            r = torch.from_numpy(synth.activations(62, M, N)).cuda().to(TDT[c["ydt"]])
+            ref = ref + r.double().cpu().numpy()
+        y = torch.full((M, N), float("nan"), dtype=TDT[c["ydt"]], device="cuda")
+        if c["norm"]:
+            backend.matmul_norm(w, x, gamma, eps, y, c["epi"], r)
+        else:
+            backend.matmul_ex(w, x, y, c["epi"], r)
+        torch.cuda.synchronize()
+        assert not torch.isnan(y).any(), c
+        bar = FAST if fast else TIGHT
+        if c["epi"] == "swiglu":
+            bar *= 2
+        if c["ydt"] == "f16":
+            bar = max(bar, 6e-4)                          # one rounding to 11 bits
+        if c["ydt"] == "bf16":
+            bar = max(bar, 4e-3)                          # one rounding to 8 bits
+        err = oracle.rel_l2(y.float().cpu().numpy(), ref)
+        assert err < bar, (c, err)
+        w.free()
+    finally:
+        backend.set_prefill_mode("fast")
+
+
 def test_epilogue_errors(backend, oracle):
     q, s = _quant(oracle, 4, 64, 256)
     qw = backend.upload_quantized(q, s, 4)
