@@ -87,6 +87,28 @@ __device__ __forceinline__ void unpack_q4_f16(uint32_t w, uint32_t magic, uint32
     out[3] = as_u32(t3);
 }
 
+// The bf16 counterpart: 0x4300 | u is the bf16 number 128 + u (7 mantissa bits, so
+// only a nibble in the low bits fits: every pair is shifted down first).  There is no
+// packed bf16 add to take the 136 = 128 + 8 off again; callers multiply with the
+// biased operand and add a second MFMA against the constant operand -136
+// (kBf16Neg136x2), which subtracts 136 * sum(x) in the same fp32 accumulator.
+__device__ __forceinline__ uint32_t q4_magic_vgpr_bf16()
+{
+    uint32_t mv;
+    asm volatile("v_mov_b32 %0, 0x43004300" : "=v"(mv));
+    return mv;
+}
+constexpr uint32_t kBf16Neg136x2 = 0xC308C308u;
+
+__device__ __forceinline__ void unpack_q4_bf16_biased(uint32_t w, uint32_t magic, uint32_t out[4])
+{
+    const uint32_t lo = 0x000F000Fu;
+    out[0] = (w & lo) | magic;
+    out[1] = ((w >> 4) & lo) | magic;
+    out[2] = ((w >> 8) & lo) | magic;
+    out[3] = ((w >> 12) & lo) | magic;
+}
+
 // Two native Q8 words (8 bytes, u = q + 128) -> 8 exact f16 integers.
 __device__ __forceinline__ void unpack_q8_f16(uint32_t w0, uint32_t w1, uint32_t out[4])
 {

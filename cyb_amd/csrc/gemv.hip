@@ -175,15 +175,22 @@ __device__ __forceinline__ void tile_issue(const TileRegs<BITS>& t, const uint16
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         uint32_t bw[4];
-        if (BITS == 4) unpack_q4_f16(t.q[0][j], magic, bw);
-        else unpack_q8_f16(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
-        if (XMODE == XBF16) f16frag_to_bf16frag(bw);
+        if (BITS == 4 && XMODE == XBF16) {
+            unpack_q4_bf16_biased(t.q[0][j], magic, bw);
+        } else {
+            if (BITS == 4) unpack_q4_f16(t.q[0][j], magic, bw);
+            else unpack_q8_f16(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
+            if (XMODE == XBF16) f16frag_to_bf16frag(bw);
+        }
         b[j].u = (u32x4_t){bw[0], bw[1], bw[2], bw[3]};
     }
+    Frag16 off;
+    off.u = (u32x4_t){kBf16Neg136x2, kBf16Neg136x2, kBf16Neg136x2, kBf16Neg136x2};
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         if (XMODE == XBF16) {
             d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].b, b[j].b, zero, 0, 0, 0);
+            if (BITS == 4) d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].b, off.b, d[j], 0, 0, 0);
         } else {
             d[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j].h, b[j].h, zero, 0, 0, 0);
             if (XMODE == XF32) d[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al[j].h, b[j].h, d[j], 0, 0, 0);
@@ -407,7 +414,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t* xs = reinterpret_cast<uint16_t*>(smem);
-    const uint32_t magic = q4_magic_vgpr();
+    const uint32_t magic = (BITS == 4 && XMODE == XBF16) ? q4_magic_vgpr_bf16() : q4_magic_vgpr();
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
@@ -531,15 +538,23 @@ __device__ __forceinline__ void tile_issue_regs(const TileRegs<BITS>& t, const F
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         uint32_t bw[4];
-        if (BITS == 4) unpack_q4_f16(t.q[0][j], magic, bw);
-        else unpack_q8_f16(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
-        if (XMODE == XBF16) f16frag_to_bf16frag(bw);
+        if (BITS == 4 && XMODE == XBF16) {
+            unpack_q4_bf16_biased(t.q[0][j], magic, bw);
+        } else {
+            if (BITS == 4) unpack_q4_f16(t.q[0][j], magic, bw);
+            else unpack_q8_f16(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
+            if (XMODE == XBF16) f16frag_to_bf16frag(bw);
+        }
         b[j].u = (u32x4_t){bw[0], bw[1], bw[2], bw[3]};
     }
+    Frag16 off;
+    off.u = (u32x4_t){kBf16Neg136x2, kBf16Neg136x2, kBf16Neg136x2, kBf16Neg136x2};
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        if (XMODE == XBF16) d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].b, b[j].b, zero, 0, 0, 0);
-        else d[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j].h, b[j].h, zero, 0, 0, 0);
+        if (XMODE == XBF16) {
+            d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].b, b[j].b, zero, 0, 0, 0);
+            if (BITS == 4) d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].b, off.b, d[j], 0, 0, 0);
+        } else d[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j].h, b[j].h, zero, 0, 0, 0);
     }
 }
 
@@ -588,7 +603,7 @@ __global__ __launch_bounds__(TS <= 2 ? 1024 : 512) __attribute__((amdgpu_waves_p
 void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void* __restrict__ y, int ydt, Epilogue epi)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    const uint32_t magic = q4_magic_vgpr();
+    const uint32_t magic = (BITS == 4 && XMODE == XBF16) ? q4_magic_vgpr_bf16() : q4_magic_vgpr();
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
