@@ -125,19 +125,26 @@ __device__ __forceinline__ void unpack_q8_f16(uint32_t w0, uint32_t w1, uint32_t
     out[3] = as_u32(as_h2(p3) + sub);
 }
 
-// packed pair of exact small f16 integers -> packed pair of bf16 (exact)
-__device__ __forceinline__ uint32_t h2_to_bf16x2_exact(uint32_t h2)
+// fp32 -> bf16, round to nearest even, in hardware (v_cvt_pk_bf16_f32)
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
 {
-    half2_t v = as_h2(h2);
-    uint32_t a = __builtin_bit_cast(uint32_t, (float)v.x);
-    uint32_t b = __builtin_bit_cast(uint32_t, (float)v.y);
-    return __builtin_amdgcn_perm(b, a, 0x07060302u);   // [a.hi16, b.hi16]
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 
-__device__ __forceinline__ void f16frag_to_bf16frag(uint32_t f[4])
+// Two native Q8 words -> 8 biased bf16 operands u = q + 128 (0 .. 255 is exact in bf16's 8
+// significant bits); as with Q4 the bias comes off through a second MFMA against the
+// constant -128 (kBf16Neg128x2).
+constexpr uint32_t kBf16Neg128x2 = 0xC300C300u;
+__device__ __forceinline__ void unpack_q8_bf16_biased(uint32_t w0, uint32_t w1, uint32_t out[4])
 {
-#pragma unroll
-    for (int i = 0; i < 4; i++) f[i] = h2_to_bf16x2_exact(f[i]);
+    out[0] = pack_bf16x2((float)(w0 & 0xffu), (float)((w0 >> 8) & 0xffu));
+    out[1] = pack_bf16x2((float)((w0 >> 16) & 0xffu), (float)(w0 >> 24));
+    out[2] = pack_bf16x2((float)(w1 & 0xffu), (float)((w1 >> 8) & 0xffu));
+    out[3] = pack_bf16x2((float)((w1 >> 16) & 0xffu), (float)(w1 >> 24));
 }
 
 // signed value of weight slot s of a native Q4 word / Q8 word pair (scalar helpers)

@@ -51,22 +51,13 @@ namespace cybq {
 
 namespace {
 
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float float2_t __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ uint16_t f32_to_bf16_rne_g(float f)
-{
-    uint32_t u = __builtin_bit_cast(uint32_t, f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
-}
 
 __device__ __forceinline__ void store_out_g(void* y, int ydt, int64_t idx, float v)
 {
     if (ydt == kF32) reinterpret_cast<float*>(y)[idx] = v;
     else if (ydt == kF16) reinterpret_cast<_Float16*>(y)[idx] = (_Float16)v;
-    else reinterpret_cast<uint16_t*>(y)[idx] = f32_to_bf16_rne_g(v);
+    else reinterpret_cast<uint16_t*>(y)[idx] = f32_to_bf16_bits(v);
 }
 
 
@@ -571,7 +562,7 @@ __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict_
                     v0 *= g[2 * p] * sc;
                     v1 *= g[2 * p + 1] * sc;
                     if (XBF && !WIDEN) {
-                        a.u[p] = (uint32_t)f32_to_bf16_rne_g(v0) | ((uint32_t)f32_to_bf16_rne_g(v1) << 16);
+                        a.u[p] = pack_bf16x2(v0, v1);
                     } else {
                         const half2_t h = {(_Float16)v0, (_Float16)v1};
                         a.u[p] = as_u32(h);

@@ -42,19 +42,11 @@ __device__ __forceinline__ void load_tile(TileRegs<BITS>& t, const WeightView& w
     t.s = __builtin_nontemporal_load(sp + tile * 16 + (lane & 15));
 }
 
-__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f)
-{
-    uint32_t u = __builtin_bit_cast(uint32_t, f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
-}
-
 __device__ __forceinline__ void store_out(void* y, int ydt, int64_t idx, float v)
 {
     if (ydt == kF32) reinterpret_cast<float*>(y)[idx] = v;
     else if (ydt == kF16) reinterpret_cast<_Float16*>(y)[idx] = (_Float16)v;
-    else reinterpret_cast<uint16_t*>(y)[idx] = f32_to_bf16_rne(v);
+    else reinterpret_cast<uint16_t*>(y)[idx] = f32_to_bf16_bits(v);
 }
 
 __device__ __forceinline__ float load_out(const void* p, int dt, int64_t idx)
@@ -177,20 +169,22 @@ __device__ __forceinline__ void tile_issue(const TileRegs<BITS>& t, const uint16
         uint32_t bw[4];
         if (BITS == 4 && XMODE == XBF16) {
             unpack_q4_bf16_biased(t.q[0][j], magic, bw);
+        } else if (XMODE == XBF16) {
+            unpack_q8_bf16_biased(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
         } else {
             if (BITS == 4) unpack_q4_f16(t.q[0][j], magic, bw);
             else unpack_q8_f16(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
-            if (XMODE == XBF16) f16frag_to_bf16frag(bw);
         }
         b[j].u = (u32x4_t){bw[0], bw[1], bw[2], bw[3]};
     }
     Frag16 off;
-    off.u = (u32x4_t){kBf16Neg136x2, kBf16Neg136x2, kBf16Neg136x2, kBf16Neg136x2};
+    const uint32_t offw = BITS == 4 ? kBf16Neg136x2 : kBf16Neg128x2;
+    off.u = (u32x4_t){offw, offw, offw, offw};
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         if (XMODE == XBF16) {
             d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].b, b[j].b, zero, 0, 0, 0);
-            if (BITS == 4) d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].b, off.b, d[j], 0, 0, 0);
+            d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].b, off.b, d[j], 0, 0, 0);
         } else {
             d[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j].h, b[j].h, zero, 0, 0, 0);
             if (XMODE == XF32) d[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al[j].h, b[j].h, d[j], 0, 0, 0);
@@ -327,7 +321,7 @@ __device__ __forceinline__ void store_staged_piece(uint16_t* row, int plane_elem
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         if (XMODE == XBF16) {
-            v[i] = (uint32_t)f32_to_bf16_rne(in[2 * i]) | ((uint32_t)f32_to_bf16_rne(in[2 * i + 1]) << 16);
+            v[i] = pack_bf16x2(in[2 * i], in[2 * i + 1]);
         } else {
             const half2_t h = {(_Float16)in[2 * i], (_Float16)in[2 * i + 1]};
             v[i] = as_u32(h);
@@ -540,20 +534,22 @@ __device__ __forceinline__ void tile_issue_regs(const TileRegs<BITS>& t, const F
         uint32_t bw[4];
         if (BITS == 4 && XMODE == XBF16) {
             unpack_q4_bf16_biased(t.q[0][j], magic, bw);
+        } else if (XMODE == XBF16) {
+            unpack_q8_bf16_biased(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
         } else {
             if (BITS == 4) unpack_q4_f16(t.q[0][j], magic, bw);
             else unpack_q8_f16(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
-            if (XMODE == XBF16) f16frag_to_bf16frag(bw);
         }
         b[j].u = (u32x4_t){bw[0], bw[1], bw[2], bw[3]};
     }
     Frag16 off;
-    off.u = (u32x4_t){kBf16Neg136x2, kBf16Neg136x2, kBf16Neg136x2, kBf16Neg136x2};
+    const uint32_t offw = BITS == 4 ? kBf16Neg136x2 : kBf16Neg128x2;
+    off.u = (u32x4_t){offw, offw, offw, offw};
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         if (XMODE == XBF16) {
             d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].b, b[j].b, zero, 0, 0, 0);
-            if (BITS == 4) d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].b, off.b, d[j], 0, 0, 0);
+            d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].b, off.b, d[j], 0, 0, 0);
         } else d[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j].h, b[j].h, zero, 0, 0, 0);
     }
 }
@@ -589,7 +585,7 @@ __device__ __forceinline__ void norm_frag(Frag16& a, const float* gamma_lds, int
         v0 *= g[2 * p];
         v1 *= g[2 * p + 1];
         if (XMODE == XBF16) {
-            a.u[p] = (uint32_t)f32_to_bf16_rne(v0) | ((uint32_t)f32_to_bf16_rne(v1) << 16);
+            a.u[p] = pack_bf16x2(v0, v1);
         } else {
             const half2_t h = {(_Float16)v0, (_Float16)v1};
             a.u[p] = as_u32(h);
@@ -800,11 +796,12 @@ hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int y
         if (ns == 2) return launch_rows_t<BITS, XMODE, 2, 2>(w, x, M, y, ydt, nwaves, epi, st);
         return launch_rows_t<BITS, XMODE, 2, 1>(w, x, M, y, ydt, nwaves, epi, st);
     }
-    if constexpr (XMODE == XF16 && BITS == 4) {
+    if constexpr (BITS == 4) {
         if (seven && nwaves <= 8) return launch_rows_t<BITS, XMODE, 4, 7>(w, x, M, y, ydt, nwaves, epi, st);
     }
-    // (bf16 operands and Q8 tiles need more registers: four strips x four tiles would spill)
-    if (ns == 4 && (XMODE == XBF16 || BITS == 8)) return launch_rows_t<BITS, XMODE, 2, 4>(w, x, M, y, ydt, nwaves, epi, st);
+    // Q8 tiles are twice the registers: four strips x four tiles of f16 operands would spill.  Two
+    // strips x two tiles (80 registers, six waves per SIMD) stream best there; bf16 operands fit
+    if (ns == 4 && BITS == 8 && XMODE == XF16) return launch_rows_t<BITS, XMODE, 2, 2>(w, x, M, y, ydt, nwaves, epi, st);
     if (ns == 4) return launch_rows_t<BITS, XMODE, 4, 4>(w, x, M, y, ydt, nwaves, epi, st);
     if (ns == 2) return launch_rows_t<BITS, XMODE, 4, 2>(w, x, M, y, ydt, nwaves, epi, st);
     // one strip per workgroup and a long K: eight tiles per wave and slab, fewer round trips
