@@ -240,11 +240,30 @@ def main():
             sweep[f"M{Mb}"] = {"us": round(e * 1e6, 2),
                                "GB/s": round(formats.matmul_bytes(bits, N, K, Mb, 2, 4) / e / 1e9, 1)}
         extra["decode_batch_sweep_4096x14336"] = sweep
-        # the reference-shaped decode step: 32 layers x (q,k,v,o,gate,up,down), Q4, random init,
-        # one native walk over the 224 linear nodes per step (BASELINE configs[4])
+        # the sweep's second shape, the down projection (BASELINE configs[2]): 256 strips of 112 K tiles
         for t in ws[1:]:
             t.free()
         del ws[1:]
+        qd, sd = formats.quantize(synth.weights(6, K, N), bits)
+        wd = [be.upload_quantized(qd, sd, bits)]
+        wd += [wd[0].clone() for _ in range(copies - 1)]
+        del qd, sd
+        sweep_d = {}
+        for Mb in (1, 4, 8, 16):
+            xb = torch.from_numpy(synth.activations(3, Mb, N, outliers=0.001)).to(dev).to(torch.float16)
+            yb = torch.empty((Mb, K), dtype=torch.float32, device=dev)
+            n = 240
+            pl = be.plan_many([wd[i % copies] for i in range(n)], [xb] * n, [yb] * n)
+            be.matmul_many(pl, Mb, stream)
+            e = timed_many(be, pl, Mb, stream, torch) / n
+            sweep_d[f"M{Mb}"] = {"us": round(e * 1e6, 2),
+                                 "GB/s": round(formats.matmul_bytes(bits, K, N, Mb, 2, 4) / e / 1e9, 1)}
+        extra["decode_batch_sweep_14336x4096"] = sweep_d
+        for t in wd:
+            t.free()
+        del wd
+        # the reference-shaped decode step: 32 layers x (q,k,v,o,gate,up,down), Q4, random init,
+        # one native walk over the 224 linear nodes per step (BASELINE configs[4])
         from cyb_amd import stack as stk
         stack_out = {}
         for label, shapes, epis in (("per_linear_224_launches", None, False),
