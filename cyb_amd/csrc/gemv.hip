@@ -593,7 +593,7 @@ __device__ __forceinline__ void norm_frag(Frag16& a, const float* gamma_lds, int
     }
 }
 
-template <int BITS, int XMODE, int TS, int NS, bool NORM>
+template <int BITS, int XMODE, int TS, int NS, bool NORM, int XR>
 // (waves_per_eu: the scheduler would otherwise trade the up-front loads for occupancy)
 __global__ __launch_bounds__(TS <= 2 ? 1024 : 512) __attribute__((amdgpu_waves_per_eu(2, TS <= 2 ? 4 : 2)))
 void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void* __restrict__ y, int ydt, Epilogue epi)
@@ -607,12 +607,18 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
     const int oct = lane >> 4;
     const int strip0 = blockIdx.x * NS;
     const int KT = w.KT;
-    // x is read the way memory likes it - lane l takes 16 B number l%4 of row l/4, so
-    // four neighbouring lanes cover 64 contiguous bytes - and then moved across lanes
-    // into MFMA A-operand order (lane l: row l%16, k octet l/16).  Reading in operand
-    // order directly costs 64 separate accesses per load instead of 16.
-    const uint16_t* xrow = x + (int64_t)min(lane >> 2, M - 1) * w.K + (lane & 3) * 8;
-    const int from_lane = (((lane & 15) << 2) | oct) << 2;       // byte address for ds_bpermute
+    // x is read the way memory likes it - one load instruction covers XR rows (the batch rounded
+    // up to 4, 8 or 16) x P = 64 / XR neighbouring 16 B pieces, lane l takes piece l % P of row
+    // l / P - and then moved across lanes into MFMA A-operand order (lane l: row l%16, k octet
+    // l/16).  Reading in operand order directly costs 64 separate accesses per load instead of
+    // 16; and the address path takes 16 cycles per load whatever the lanes ask for, so a batch of
+    // four rows gets a whole tile (128 k) with one load where sixteen rows need four.
+    constexpr int P = 64 / XR;                  // 16 B pieces per row and load
+    constexpr int L = 16 / P;                   // loads per tile: 1, 2, 4
+    constexpr int GPL = 4 / L;                  // scale groups per load
+    const uint16_t* xrow = x + (int64_t)min(lane / P, M - 1) * w.K + (lane % P) * 8;
+    const int klast = w.K - 8 - (lane % P) * 8;          // last start at which this lane's piece is inside the row
+    const int from_lane = ((((lane & 15) & (XR - 1)) * P) | oct) << 2;       // byte address for ds_bpermute (+ 16 per group)
     // NORM: gamma as fp32 in LDS behind the exchange areas (read per fragment with LDS loads, which
     // do not queue behind the weight requests the way global loads would)
     float* gamma_lds = reinterpret_cast<float*>(smem) + NS * nwaves * 4 * 64 + nwaves * 16;
@@ -648,8 +654,12 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
             valid[u] = t < KT;
             kt[u] = min(t, KT - 1);
 #pragma unroll
-            for (int j = 0; j < 4; j++)
-                a[u][j].u = *reinterpret_cast<const u32x4_t*>(xrow + min(kt[u] * kTileK + j * 32, w.K - 32));
+            for (int h = 0; h < L; h++) {
+                // (past the end of K: any x inside the row will do, the padded weights are zero)
+                const int k0 = kt[u] * kTileK + h * (GPL * 32);
+                if (XR == 16) a[u][h].u = *reinterpret_cast<const u32x4_t*>(xrow + min(k0, w.K - 32));
+                else a[u][h].u = *reinterpret_cast<const u32x4_t*>(xrow + min(k0, klast));
+            }
         }
         // The memory pipeline takes requests at its own pace: a wave that asks for all its
         // tiles first sits in the issue queue for microseconds and only then starts on
@@ -663,12 +673,17 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
 #pragma unroll
             for (int u = 0; u < TS; u++) load_tile<BITS>(buf[s][u], w, sbase[s] + kt[u], lane);
 #pragma unroll
-        for (int u = 0; u < TS; u++)
+        for (int u = 0; u < TS; u++) {
+            u32x4_t raw[L];
+#pragma unroll
+            for (int h = 0; h < L; h++) raw[h] = a[u][h].u;
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
                 for (int p = 0; p < 4; p++)
-                    a[u][j].u[p] = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane, (int)a[u][j].u[p]);
+                    a[u][j].u[p] =
+                        (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane + (j % GPL) * 16, (int)raw[j / GPL][p]);
+        }
         if (NORM) {
 #pragma unroll
             for (int u = 0; u < TS; u++)
@@ -752,15 +767,15 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
     }
 }
 
-template <int BITS, int XMODE, int TS, int NS>
-hipError_t launch_rows_t(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
+template <int BITS, int XMODE, int TS, int NS, int XR>
+hipError_t launch_rows_x(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
                          hipStream_t st)
 {
     size_t lds = (size_t)NS * nwaves * 4 * 64 * sizeof(float) + (size_t)nwaves * 16 * sizeof(float);
     const unsigned groups = (unsigned)((w.NT + NS - 1) / NS);
     if (epi.gamma) {
         lds += (size_t)w.K * sizeof(float);            // gamma as fp32
-        auto kern = gemv_rows_kernel<BITS, XMODE, TS, NS, true>;
+        auto kern = gemv_rows_kernel<BITS, XMODE, TS, NS, true, XR>;
         static bool attr_set = false;
         if (!attr_set) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -772,9 +787,19 @@ hipError_t launch_rows_t(const WeightView& w, const void* x, int M, void* y, int
         hipLaunchKernelGGL(kern, dim3(groups), dim3(nwaves * 64), lds, st, w, reinterpret_cast<const uint16_t*>(x), M, y, ydt,
                            epi);
     } else
-        hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS, false>), dim3(groups), dim3(nwaves * 64), lds, st, w,
+        hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS, false, XR>), dim3(groups), dim3(nwaves * 64), lds, st, w,
                            reinterpret_cast<const uint16_t*>(x), M, y, ydt, epi);
     return hipGetLastError();
+}
+
+// (the x load pattern follows the batch: up to 4, up to 8, up to 16 rows per load)
+template <int BITS, int XMODE, int TS, int NS>
+hipError_t launch_rows_t(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
+                         hipStream_t st)
+{
+    if (M <= 4) return launch_rows_x<BITS, XMODE, TS, NS, 4>(w, x, M, y, ydt, nwaves, epi, st);
+    if (M <= 8) return launch_rows_x<BITS, XMODE, TS, NS, 8>(w, x, M, y, ydt, nwaves, epi, st);
+    return launch_rows_x<BITS, XMODE, TS, NS, 16>(w, x, M, y, ydt, nwaves, epi, st);
 }
 
 template <int BITS, int XMODE>
@@ -789,23 +814,23 @@ hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int y
     // seven strips per workgroup when that is exactly one workgroup per CU (N = 28672 on 256 CUs:
     // with four strips the 448 workgroups need a second, mostly empty round); SwiGLU pairs need an even count
     const bool seven = w.NT == 7 * num_cus && epi.kind != kEpiSwiglu;
-    int nwaves = tuned_waves > 0 ? tuned_waves : 8;
+    int nwaves = tuned_waves > 0 ? min(tuned_waves, 8) : 8;
     while (nwaves > 1 && nwaves * 2 > w.KT) nwaves >>= 1;
-    if (nwaves > 8) {          // 16 waves: 128 registers per lane, two tiles of x in flight
-        if (ns == 4) return launch_rows_t<BITS, XMODE, 2, 4>(w, x, M, y, ydt, nwaves, epi, st);
-        if (ns == 2) return launch_rows_t<BITS, XMODE, 2, 2>(w, x, M, y, ydt, nwaves, epi, st);
-        return launch_rows_t<BITS, XMODE, 2, 1>(w, x, M, y, ydt, nwaves, epi, st);
-    }
     if constexpr (BITS == 4) {
-        if (seven && nwaves <= 8) return launch_rows_t<BITS, XMODE, 4, 7>(w, x, M, y, ydt, nwaves, epi, st);
+        if (seven) return launch_rows_t<BITS, XMODE, 4, 7>(w, x, M, y, ydt, nwaves, epi, st);
+        if (ns == 4) return launch_rows_t<BITS, XMODE, 4, 4>(w, x, M, y, ydt, nwaves, epi, st);
+    } else if constexpr (XMODE == XF16) {
+        // Q8 tiles are twice the registers: four strips x four tiles of f16 operands would spill.  Two
+        // strips x two tiles (80 registers, six waves per SIMD) stream best there; bf16 operands fit
+        if (ns == 4) return launch_rows_t<BITS, XMODE, 2, 2>(w, x, M, y, ydt, nwaves, epi, st);
+    } else {
+        if (ns == 4) return launch_rows_t<BITS, XMODE, 4, 4>(w, x, M, y, ydt, nwaves, epi, st);
     }
-    // Q8 tiles are twice the registers: four strips x four tiles of f16 operands would spill.  Two
-    // strips x two tiles (80 registers, six waves per SIMD) stream best there; bf16 operands fit
-    if (ns == 4 && BITS == 8 && XMODE == XF16) return launch_rows_t<BITS, XMODE, 2, 2>(w, x, M, y, ydt, nwaves, epi, st);
-    if (ns == 4) return launch_rows_t<BITS, XMODE, 4, 4>(w, x, M, y, ydt, nwaves, epi, st);
     if (ns == 2) return launch_rows_t<BITS, XMODE, 4, 2>(w, x, M, y, ydt, nwaves, epi, st);
-    // one strip per workgroup and a long K: eight tiles per wave and slab, fewer round trips
-    if (w.KT > nwaves * 4 && BITS == 4) return launch_rows_t<BITS, XMODE, 8, 1>(w, x, M, y, ydt, nwaves, epi, st);
+    if constexpr (BITS == 4) {
+        // one strip per workgroup and a long K: eight tiles per wave and slab, fewer round trips
+        if (w.KT > nwaves * 4) return launch_rows_t<BITS, XMODE, 8, 1>(w, x, M, y, ydt, nwaves, epi, st);
+    }
     return launch_rows_t<BITS, XMODE, 4, 1>(w, x, M, y, ydt, nwaves, epi, st);
 }
 
