@@ -346,6 +346,21 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
             // a quarter of the next tile's dequantisation rides along with every group
             stage_units(wreg[(R + 1) % SETS], j, wnxt);
         }
+        // Order inside the K tile (two waves per SIMD): the dequantisation of the next tile is
+        // spread between the MFMAs.  A wave issues in order: arithmetic queued behind a run of
+        // MFMAs waits for all of them and the matrix pipe idles while it runs afterwards; and the
+        // barrier keeps the two waves of a SIMD in the same phase, so they do not cover for each
+        // other.  (With one wave per SIMD, the 128-row shape, the same order measured slower.)
+        if constexpr (WAVES == 8 && !EXACT) {
+            constexpr int PAIRS = 4 * NF * OPS * MF / 2;
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);          // LDS reads run two ahead of their MFMAs
+#pragma unroll
+            for (int i = 0; i < PAIRS; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // one LDS read
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);      // two MFMAs
+                __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);      // two vector ALU instructions
+            }
+        }
         __syncthreads();
     };
     for (int kt = 0; kt < KT; kt += SETS) {
