@@ -828,8 +828,15 @@ hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int y
     }
     if (ns == 2) return launch_rows_t<BITS, XMODE, 4, 2>(w, x, M, y, ydt, nwaves, epi, st);
     if constexpr (BITS == 4) {
-        // one strip per workgroup and a long K: eight tiles per wave and slab, fewer round trips
-        if (w.KT > nwaves * 4) return launch_rows_t<BITS, XMODE, 8, 1>(w, x, M, y, ydt, nwaves, epi, st);
+        // one strip per workgroup and a long K: eight tiles per wave and slab (fewer round trips), unless
+        // that leaves more of the last slab empty than seven or four would - tiles past the end are still loaded
+        // (11008 -> 4096: 86 tiles are 2 slabs of 64 or 3 of 32, 15.6 -> 11.7 us at 16 rows; 14336 -> 4096:
+        // 112 tiles are 2 slabs of 56, seven tiles per wave)
+        auto pad = [&](int ts) { return (w.KT + nwaves * ts - 1) / (nwaves * ts) * (nwaves * ts) - w.KT; };
+        if (w.KT > nwaves * 4) {
+            if (pad(8) <= pad(7) && pad(8) <= pad(4)) return launch_rows_t<BITS, XMODE, 8, 1>(w, x, M, y, ydt, nwaves, epi, st);
+            if (pad(7) <= pad(4)) return launch_rows_t<BITS, XMODE, 7, 1>(w, x, M, y, ydt, nwaves, epi, st);
+        }
     }
     return launch_rows_t<BITS, XMODE, 4, 1>(w, x, M, y, ydt, nwaves, epi, st);
 }
