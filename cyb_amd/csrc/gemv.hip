@@ -469,12 +469,24 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
                 norm_staged_slab<XMODE>(xs, M, st * kTileK, slab0 * kTileK, w.K, ldx, plane_elems, epi, gp, ssq, ssq_part, tid, nthreads);
 
             const uint16_t* xbase = xs + mrow * ldx + oct * 8;
-            for (int i0 = wv; i0 < st; i0 += 2 * stride) {
-                // bufA holds batch i0; fetch batch i0 + stride into bufB, and so on
-                load_batch<BITS, U>(bufB, w, base, i0 + stride, nwaves, st, lane);
-                compute_batch<BITS, XMODE, RMAX, U>(bufA, i0, nwaves, st, xbase, plane_elems, magic, acc);
-                load_batch<BITS, U>(bufA, w, base, i0 + 2 * stride, nwaves, st, lane);
-                compute_batch<BITS, XMODE, RMAX, U>(bufB, i0 + stride, nwaves, st, xbase, plane_elems, magic, acc);
+            for (int r0 = 0; r0 < st; r0 += 2 * stride) {
+                // bufA holds batch r0; fetch batch r0 + stride into bufB, and so on.  A batch that
+                // starts past the end of the slab is not requested at all (its loads would only
+                // be cache hits, but they would still queue in the address path).  Every arm is
+                // straight-line code of its own, so the load counters stay exact.
+                const int i0 = r0 + wv;
+                if (r0 + stride < st) {
+                    load_batch<BITS, U>(bufB, w, base, i0 + stride, nwaves, st, lane);
+                    compute_batch<BITS, XMODE, RMAX, U>(bufA, i0, nwaves, st, xbase, plane_elems, magic, acc);
+                    if (r0 + 2 * stride < st) {
+                        load_batch<BITS, U>(bufA, w, base, i0 + 2 * stride, nwaves, st, lane);
+                        compute_batch<BITS, XMODE, RMAX, U>(bufB, i0 + stride, nwaves, st, xbase, plane_elems, magic, acc);
+                    } else {
+                        compute_batch<BITS, XMODE, RMAX, U>(bufB, i0 + stride, nwaves, st, xbase, plane_elems, magic, acc);
+                    }
+                } else {
+                    compute_batch<BITS, XMODE, RMAX, U>(bufA, i0, nwaves, st, xbase, plane_elems, magic, acc);
+                }
             }
         }
     }
