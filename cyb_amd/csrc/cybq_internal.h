@@ -32,6 +32,21 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
 hipError_t launch_quantize(int bits, const float* src, int N, int K, void* q_out, void* s_out,
                            hipStream_t st);
 
+// Raises a kernel's dynamic LDS limit, once per kernel and device: `done` is the caller's
+// static bit mask of devices already served (the attribute belongs to the kernel as loaded on
+// one device; a process may drive several).
+inline hipError_t raise_lds_limit_once(const void* kernel, int bytes, unsigned long long& done)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const unsigned long long bit = 1ull << (dev & 63);
+    if (done & bit) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) done |= bit;
+    return e;
+}
+
 // test/bench hook: overrides the decode kernel's launch heuristics (0 = automatic)
 void set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll);
 

@@ -469,13 +469,8 @@ hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt,
     constexpr int BM = WAVES * MF * 16;
     const size_t lds = (size_t)2 * NF * (4 * (EXACT ? 2 : 1) * 64) * 16;     // operand buffers, 56 .. 128 KB
     auto kern = gemm_kernel<BITS, XBF, NF, EXACT, MF, WAVES>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static unsigned long long lds_raised = 0;
+    if (hipError_t e = raise_lds_limit_once(reinterpret_cast<const void*>(kern), (int)lds, lds_raised); e != hipSuccess) return e;
     const int n_tiles = (w.NT + NF - 1) / NF, m_tiles = (M + BM - 1) / BM;
     // Too few tiles to fill the chip: split K over workgroups.  Every split adds its
     // K range in fp32 into its own slab of `part`; a second kernel adds the slabs in

@@ -788,13 +788,8 @@ hipError_t launch_rows_x(const WeightView& w, const void* x, int M, void* y, int
     if (epi.gamma) {
         lds += (size_t)w.K * sizeof(float);            // gamma as fp32
         auto kern = gemv_rows_kernel<BITS, XMODE, TS, NS, true, XR>;
-        static bool attr_set = false;
-        if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               150 * 1024);
-            if (e != hipSuccess) return e;
-            attr_set = true;
-        }
+        static unsigned long long lds_raised = 0;
+        if (hipError_t e = raise_lds_limit_once(reinterpret_cast<const void*>(kern), 150 * 1024, lds_raised); e != hipSuccess) return e;
         if (lds > 150 * 1024) return hipErrorInvalidValue;      // K beyond ~30 k with a folded norm
         hipLaunchKernelGGL(kern, dim3(groups), dim3(nwaves * 64), lds, st, w, reinterpret_cast<const uint16_t*>(x), M, y, ydt,
                            epi);
@@ -879,14 +874,9 @@ hipError_t launch_p(const WeightView& w, const void* x, int M, void* y, int ydt,
     // x, then the waves' partial sums, then 16 row sums of squares and their 16 x 16 per-wave parts (folded RMSNorm)
     const size_t lds = xbytes + (size_t)PAIR * nwaves * RMAX * 64 * sizeof(float) + (16 + 256) * sizeof(float);
     auto kern = gemv_kernel<BITS, XMODE, RMAX, U, ONESHOT, PAIR, NORM>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        // M = 16 fp32 activations with 8 waves need 66 KB, just over the default cap
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    // M = 16 fp32 activations with 8 waves need 66 KB, just over the default cap
+    static unsigned long long lds_raised = 0;
+    if (hipError_t e = raise_lds_limit_once(reinterpret_cast<const void*>(kern), 96 * 1024, lds_raised); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(w.NT / PAIR), dim3(nwaves * PAIR * 64), lds, st, w, x, M, y, ydt, slab_tiles, ldx, (int)xbytes,
                        epi);
     return hipGetLastError();
