@@ -101,6 +101,67 @@ int main(int argc, char** argv)
         (void)hipFree(y2);
     }
 
+    // folded RMSNorm with gamma = 1: exactly the plain result scaled by each row's rstd;
+    // SwiGLU over a tensor fused with itself: silu(g) * g of the plain result
+    {
+        const int64_t N0 = nodes[0].N, K0 = nodes[0].K, cnt = M * N0;
+        std::vector<float> ones((size_t)K0, 1.0f), plain((size_t)cnt), got((size_t)cnt);
+        float *gd = nullptr, *y3 = nullptr;
+        if (hipMalloc((void**)&gd, (size_t)K0 * 4) != hipSuccess || hipMalloc((void**)&y3, (size_t)cnt * 4) != hipSuccess ||
+            hipMemcpy(gd, ones.data(), (size_t)K0 * 4, hipMemcpyHostToDevice) != hipSuccess) { std::printf("ERROR hip gamma\n"); return 1; }
+        edges["gamma"] = cybq::Edge{gd, CYBQ_F32, 1, K0};
+        edges["y0_norm"] = cybq::Edge{y3, CYBQ_F32, M, N0};
+        cybq::QMatMulNode nn = nodes[0];
+        nn.y = "y0_norm";
+        nn.norm_gamma = "gamma";
+        nn.norm_eps = 1e-5f;
+        s = be.run(nn, edges);
+        if (!s) { std::printf("ERROR %d %s\n", s.code, s.text.c_str()); return 1; }
+        if (hipMemcpy(plain.data(), outs[0], (size_t)cnt * 4, hipMemcpyDeviceToHost) != hipSuccess ||
+            hipMemcpy(got.data(), y3, (size_t)cnt * 4, hipMemcpyDeviceToHost) != hipSuccess) { std::printf("ERROR copy\n"); return 1; }
+        const uint16_t* xh = reinterpret_cast<const uint16_t*>(xb.data());
+        auto h2f = [](uint16_t h) {
+            const int e = (h >> 10) & 31, m = h & 1023;
+            const double v = e == 0 ? std::ldexp((double)m, -24) : std::ldexp((double)(m + 1024), e - 25);
+            return (h & 0x8000) ? -v : v;
+        };
+        for (int64_t m = 0; m < M; m++) {
+            double ss = 0;
+            for (int64_t k = 0; k < K0; k++) { const double v = h2f(xh[m * K0 + k]); ss += v * v; }
+            const double rstd = 1.0 / std::sqrt(ss / (double)K0 + 1e-5);
+            for (int64_t n = 0; n < N0; n++) {
+                const double want_v = plain[m * N0 + n] * rstd;
+                if (std::fabs(got[m * N0 + n] - want_v) > 2e-6 * std::fabs(want_v) + 1e-9) {
+                    std::printf("ERROR folded norm differs at %lld,%lld: %g vs %g\n", (long long)m, (long long)n, got[m * N0 + n], want_v);
+                    return 1;
+                }
+            }
+        }
+        nn.norm_gamma = "no.such.edge";
+        if (be.run(nn, edges).code != CYBQ_ERR_INVALID) { std::printf("ERROR missing gamma not reported\n"); return 1; }
+
+        s = be.fuse_pairs("fused.gate_up", nodes[0].w, nodes[0].w);
+        if (!s) { std::printf("ERROR %d %s\n", s.code, s.text.c_str()); return 1; }
+        cybq::QMatMulNode sw = nodes[0];
+        sw.w = "fused.gate_up";
+        sw.N = 2 * N0;
+        sw.y = "y0_norm";                          // half the fused rows: same shape as the plain output
+        sw.epilogue = CYBQ_EPI_SWIGLU;
+        s = be.run(sw, edges);
+        if (!s) { std::printf("ERROR %d %s\n", s.code, s.text.c_str()); return 1; }
+        if (hipMemcpy(got.data(), y3, (size_t)cnt * 4, hipMemcpyDeviceToHost) != hipSuccess) { std::printf("ERROR copy\n"); return 1; }
+        // (the fused tensor is summed in another order than the plain one: compare in the L2 norm)
+        double num = 0, den = 0;
+        for (int64_t j = 0; j < cnt; j++) {
+            const double g = plain[j], want_v = g / (1.0 + std::exp(-g)) * g, d = got[j] - want_v;
+            num += d * d;
+            den += want_v * want_v;
+        }
+        if (!(std::sqrt(num / den) < 2e-6)) { std::printf("ERROR swiglu differs: rel_l2 %g\n", std::sqrt(num / den)); return 1; }
+        (void)hipFree(gd);
+        (void)hipFree(y3);
+    }
+
     const double* want = reinterpret_cast<const double*>(yb.data());
     for (size_t i = 0; i < nodes.size(); i++) {
         const int64_t cnt = M * nodes[i].N;
