@@ -262,6 +262,27 @@ def main():
         for t in wd:
             t.free()
         del wd
+        # the same kernel on Q8 blocks (twice the bytes per weight, half the unpack work per byte):
+        # shows how much of the Q4 time is arithmetic rather than memory
+        q8, s8 = formats.quantize(synth.weights(2, N, K), formats.Q8)
+        n8 = max(2, (3 * MALL_BYTES) // formats.weight_bytes(formats.Q8, N, K) + 1)
+        w8 = [be.upload_quantized(q8, s8, formats.Q8)]
+        w8 += [w8[0].clone() for _ in range(n8 - 1)]
+        del q8, s8
+        q8res = {}
+        for Mb in (1, 8):
+            xb = torch.from_numpy(synth.activations(3, Mb, K)).to(dev).to(torch.float16)
+            yb = torch.empty((Mb, N), dtype=torch.float32, device=dev)
+            n = 240
+            pl = be.plan_many([w8[i % n8] for i in range(n)], [xb] * n, [yb] * n)
+            be.matmul_many(pl, Mb, stream)
+            e = timed_many(be, pl, Mb, stream, torch) / n
+            gbs = formats.matmul_bytes(formats.Q8, N, K, Mb, 2, 4) / e / 1e9
+            q8res[f"M{Mb}"] = {"us": round(e * 1e6, 2), "GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        extra["q8_decode_4096x14336"] = q8res
+        for t in w8:
+            t.free()
+        del w8
         # the reference-shaped decode step: 32 layers x (q,k,v,o,gate,up,down), Q4, random init,
         # one native walk over the 224 linear nodes per step (BASELINE configs[4])
         from cyb_amd import stack as stk
