@@ -130,6 +130,30 @@ def test_decode_seven_strips_per_workgroup(backend, oracle):
     assert torch.equal(y2, torch.from_numpy(y).cuda() + r)
 
 
+@pytest.mark.parametrize("bits,xdt", [(4, "f16"), (4, "bf16"), (8, "f16"), (8, "bf16")])
+@pytest.mark.parametrize("N", [14336, 28672, 8192])
+def test_decode_batched_rows_wide_shapes(backend, oracle, bits, xdt, N):
+    """Wide outputs give a workgroup of the batched-rows kernel 4, 7 or 2 strips; which shape runs
+    depends on block type and activation type (register budget), and the x load pattern on the
+    batch (up to 4 / 8 / 16 rows per load).  K = 384 is three K tiles: a partly filled slab."""
+    K = 384
+    q, s = _quant(oracle, bits, N, K, cfg=23)
+    qw = backend.upload_quantized(q, s, bits)
+    wd = torch.from_numpy(oracle.dequant(q, s)).cuda().double()
+    y1 = None
+    for M in (16, 8, 5, 4):
+        x = _x(16, K, xdt, cfg=24)[:M].contiguous()
+        y = _run(backend, qw, x)
+        ref = x.double() @ wd.T
+        err = ((y.double() - ref).norm() / ref.norm()).item()
+        assert err < TIGHT, (M, err)
+        # a row's bits do not depend on the batch it travels in (nor on the x load pattern)
+        if y1 is None:
+            y1 = y
+        else:
+            assert torch.equal(y, y1[:M]), M
+
+
 def test_decode_long_k_uses_several_slabs(backend, oracle):
     # M * K * 2 B exceeds the kernel's LDS budget: x is staged slab by slab
     N, K = 64, 14336
