@@ -800,6 +800,43 @@ def test_driver_events_and_rates(backend):
         w.free()
 
 
+@pytest.mark.parametrize("M,xdt", [(1, "f16"), (8, "f16"), (300, "bf16")])
+def test_calls_can_be_captured_in_a_graph(backend, oracle, M, xdt):
+    """Every call is a short run of plain kernel launches on the caller's stream (no allocation, no
+    memset, no host synchronisation), so a caller may record a step into a HIP graph.  The graph is
+    replayed several times with eager work and synchronisations in between, every replay checked
+    bit for bit against the eager result (decode kernels; staging pass + multiply + slab adding for
+    the prefill shape, whose 4096 columns split K over workgroups)."""
+    K1, N1, K2, N2 = 512, 1024, 2048, 4096
+    q1, s1 = _quant(oracle, 4, N1, K1, cfg=81)
+    q2, s2 = _quant(oracle, 8, N2, K2, cfg=82)
+    w1, w2 = backend.upload_quantized(q1, s1, 4), backend.upload_quantized(q2, s2, 8)
+    x1, x2 = _x(M, K1, xdt, cfg=83), _x(M, K2, xdt, cfg=84)
+    r = torch.from_numpy(synth.activations(85, M, N2)).cuda()
+    h = torch.empty((M, N1), dtype=torch.float32, device="cuda")
+    y = torch.empty((M, N2), dtype=torch.float32, device="cuda")
+
+    def step(stream):
+        backend.matmul(w1, x1, h, stream=stream)
+        backend.matmul_ex(w2, x2, y, "add", r, stream=stream)
+
+    step(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    h0, y0 = h.clone(), y.clone()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        step(torch.cuda.current_stream().cuda_stream)
+    for _ in range(3):
+        h.zero_()
+        y.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(h, h0) and torch.equal(y, y0)
+        assert (x1.float() @ x1.float().T).sum().isfinite()          # eager work between replays
+
+
 def test_container_to_backend(backend, oracle, tmp_path):
     from cyb_amd import container
     q, s = _quant(oracle, 4, 64, 256)
