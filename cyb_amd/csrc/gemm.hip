@@ -462,6 +462,31 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ part, int splits,
     store_out_g(y, ydt, i, v);
 }
 
+// The same sum, four neighbouring elements per thread with 128-bit slab reads (slab a multiple of
+// four elements, no SwiGLU): the pass is pure memory traffic, splits + 1 times the output.
+__global__ void splitk_reduce4_kernel(const float* __restrict__ part, int splits, int M, int N, void* __restrict__ y, int ydt,
+                                      float out_scale, Epilogue epi, NormStats ns, int K)
+{
+    const int64_t slab = (int64_t)M * N;
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i >= slab) return;
+    float4_t v = *reinterpret_cast<const float4_t*>(part + i);
+    for (int s = 1; s < splits; s++) v += *reinterpret_cast<const float4_t*>(part + s * slab + i);
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        float t = v[e] * out_scale;
+        if (epi.gamma) t *= rstd_of(ns, (int)((i + e) / N), K, epi.eps);
+        if (epi.kind == kEpiAdd) t += load_out_g(epi.residual, ydt, i + e);
+        v[e] = t;
+    }
+    if (ydt == kF32) {
+        *reinterpret_cast<float4_t*>(reinterpret_cast<float*>(y) + i) = v;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) store_out_g(y, ydt, i + e, v[e]);
+    }
+}
+
 template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES>
 hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, float* part,
                     size_t part_bytes, int num_cus, const Epilogue& epi, const NormStats& ns, hipStream_t st)
@@ -488,8 +513,12 @@ hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt,
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || splits == 1) return e;
     const int64_t total = (int64_t)M * w.N;
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, part, splits, M, w.N, y, ydt,
-                       out_scale, epi, ns, w.K);
+    if (total % 4 == 0 && epi.kind != kEpiSwiglu && (ydt != kF32 || (reinterpret_cast<uintptr_t>(y) & 15u) == 0))
+        hipLaunchKernelGGL(splitk_reduce4_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, st, part, splits, M, w.N, y,
+                           ydt, out_scale, epi, ns, w.K);
+    else
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, part, splits, M, w.N, y, ydt,
+                           out_scale, epi, ns, w.K);
     return hipGetLastError();
 }
 
