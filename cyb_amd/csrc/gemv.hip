@@ -931,12 +931,14 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
 {
     // Waves per workgroup (= split of a strip's K tiles).  Depends on the weight
     // shape only, never on M, so that the summation order is the same for every
-    // batch size: enough waves for ~8 per CU (at most 8), then 16 if that is what
-    // it takes to bring a wave's share down to 8 tiles, all requested up front.
+    // batch size: up to 4 waves (2 when there are strips enough for 8 waves per CU anyway), then
+    // more if that is what it takes to bring a wave's share down to 8 tiles, all requested
+    // up front.  (K = 4096 is 4 waves x 8 tiles for every N: with few strips 8 waves x 4 tiles
+    // measured 2 - 4 % slower.)
     int nwaves = g_tune_waves;
     if (nwaves <= 0) {
         nwaves = 2;
-        while (nwaves < 8 && (int64_t)w.NT * nwaves < (int64_t)num_cus * 8) nwaves *= 2;
+        while (nwaves < 4 && (int64_t)w.NT * nwaves < (int64_t)num_cus * 8) nwaves *= 2;
         while (nwaves < 16 && w.KT > 8 * nwaves) nwaves *= 2;
     }
     if (nwaves > 16) nwaves = 16;
