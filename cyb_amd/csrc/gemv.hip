@@ -523,7 +523,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
 }
 
 // ---------------------------------------------------------------------------
-// Batch rows 4..16: x operands live in REGISTERS and are reused across strips.
+// Batch rows 3..16: x operands live in REGISTERS and are reused across strips.
 //
 // With more than a few batch rows the LDS kernel above spends its time moving
 // x: every 16-row strip's workgroup stages all M rows of x (128 KB at M = 16,
@@ -955,8 +955,8 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
         unroll = 2;
     }
 
-    // four or more batch rows (16-bit activations): x in registers, shared across strips
-    const bool rows_kernel = g_tune_rows == 1 || (g_tune_rows == 0 && M >= 4);
+    // three or more batch rows (16-bit activations): x in registers, shared across strips
+    const bool rows_kernel = g_tune_rows == 1 || (g_tune_rows == 0 && M >= 3);
     if (rows_kernel && xdt != kF32) {
         if (w.bits == 4) {
             if (xdt == kF16) return launch_rows<4, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);

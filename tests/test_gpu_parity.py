@@ -206,7 +206,7 @@ def test_decode_batched_rows_equal_single_rows_bitwise(backend, oracle):
             assert torch.equal(_run(backend, qw, x[:batch].contiguous()), yb)     # and run to run
     finally:
         backend.set_gemv_tuning(0, 0, 0)
-    # the automatic choice (LDS kernel up to 4 rows, registers beyond) is deterministic too
+    # the automatic choice (LDS kernel for one or two rows, registers beyond) is deterministic too
     y16 = _run(backend, qw, x)
     assert torch.equal(_run(backend, qw, x), y16)
 
