@@ -956,7 +956,9 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
     }
 
     // three or more batch rows (16-bit activations): x in registers, shared across strips
-    const bool rows_kernel = g_tune_rows == 1 || (g_tune_rows == 0 && M >= 3);
+    // (Q8 on wide outputs: at exactly three rows the LDS kernel is still the quicker one)
+    const bool wide_q8 = w.bits == 8 && (w.NT + num_cus / 2) / num_cus >= 3;
+    const bool rows_kernel = g_tune_rows == 1 || (g_tune_rows == 0 && (M >= 4 || (M == 3 && !wide_q8)));
     if (rows_kernel && xdt != kF32) {
         if (w.bits == 4) {
             if (xdt == kF16) return launch_rows<4, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
