@@ -567,10 +567,14 @@ constexpr int kStagePitch = kStageGroups * 4 + 1;      // 16 B slots per LDS row
 // NORM: RMSNorm folded in.  x * gamma is formed in fp32 and rounded once to the operand type
 // (XBF: the input is bf16; WIDEN: bf16 in, f16 * 2^-4 out); the squares of the unscaled row are
 // summed per (row, workgroup) in a fixed butterfly order into ssq_part[row * gridDim.y + blockIdx.y].
-template <bool WIDEN, bool XBF, bool NORM>
+// XT: element type of X (0 f16, 1 bf16, 2 f32).  fp32 rows are rounded once to f16 * 2^-4 (WIDEN),
+// two 16 B chunks in, one out.
+template <bool WIDEN, int XT, bool NORM>
 __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict__ src, u32x4_t* __restrict__ dst, int M, int K8,
                                                       Epilogue epi, float* __restrict__ ssq_part)
 {
+    constexpr bool XBF = XT == 1;
+    static_assert(XT != 2 || WIDEN, "fp32 activations are staged as prescaled f16");
     __shared__ u32x4_t tile[16 * kStagePitch];
     const int rb = blockIdx.x;
     const int c0 = blockIdx.y * (kStageGroups * 4);     // first 16 B chunk of the row handled here
@@ -581,7 +585,26 @@ __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict_
         const int row = rb * 16 + r;
         Frag16 a;
         a.u = (u32x4_t){0u, 0u, 0u, 0u};
-        if (row < M && c < K8) a.u = src[(int64_t)row * K8 + c];
+        float xf[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};       // XT == 2: the chunk as loaded
+        if (row < M && c < K8) {
+            if (XT == 2) {
+                const u32x4_t lo = src[((int64_t)row * K8 + c) * 2], hi = src[((int64_t)row * K8 + c) * 2 + 1];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    xf[e] = __builtin_bit_cast(float, (uint32_t)lo[e]);
+                    xf[4 + e] = __builtin_bit_cast(float, (uint32_t)hi[e]);
+                }
+            } else {
+                a.u = src[(int64_t)row * K8 + c];
+            }
+        }
+        if (XT == 2 && !NORM) {
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                const half2_t h = {(_Float16)(xf[2 * p] * 0.0625f), (_Float16)(xf[2 * p + 1] * 0.0625f)};
+                a.u[p] = as_u32(h);
+            }
+        }
         if (NORM) {
             float sq = 0.f;
             if (c < K8) {
@@ -590,7 +613,10 @@ __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict_
 #pragma unroll
                 for (int p = 0; p < 4; p++) {
                     float v0, v1;
-                    if (XBF) {
+                    if (XT == 2) {
+                        v0 = xf[2 * p];
+                        v1 = xf[2 * p + 1];
+                    } else if (XBF) {
                         v0 = __builtin_bit_cast(float, a.u[p] << 16);
                         v1 = __builtin_bit_cast(float, a.u[p] & 0xffff0000u);
                     } else {
@@ -613,7 +639,7 @@ __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict_
 #pragma unroll
             for (int off = 32; off >= 1; off >>= 1) sq += __shfl_xor(sq, off, 64);
             if ((t & 63) == 0) ssq_part[(int64_t)row * gridDim.y + blockIdx.y] = sq;      // (rows past M: zeros, never read)
-        } else if (WIDEN) {
+        } else if (WIDEN && XT == 1) {
             a = bf16_to_f16_frag(a);
         }
         tile[r * kStagePitch + (t & 63)] = a.u;
@@ -634,9 +660,10 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
                        int num_cus, bool exact, void* workspace, size_t workspace_bytes, const Epilogue& epi,
                        hipStream_t st)
 {
-    if (xdt == kF32) return hipErrorNotSupported;   // api.hip walks fp32 prefill through the decode kernel
-    // FAST multiplies in f16: bf16 activations are widened (2^-4 prescale, undone in the epilogue)
-    const bool widen = !exact && xdt == kBF16;
+    if (xdt == kF32 && exact) return hipErrorNotSupported;   // api.hip walks exact fp32 prefill through the decode kernel
+    // FAST multiplies in f16: bf16 activations are widened, fp32 activations rounded to f16
+    // (both with a 2^-4 prescale that is undone in the epilogue)
+    const bool widen = !exact && xdt != kF16;
     const float out_scale = widen ? 16.0f : 1.0f;
     const int kdt = widen ? kF16 : xdt;
     // Rows are staged through the workspace in chunks that fit it; work on one stream is
@@ -649,8 +676,8 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
     const size_t stats_bytes = (size_t)1 << 20;
     if (!workspace || half <= stats_bytes) return hipErrorOutOfMemory;
     float* ssq_part = reinterpret_cast<float*>(static_cast<char*>(workspace) + half - stats_bytes);
-    const int64_t row_bytes = (int64_t)w.K * 2;
-    const int64_t max_rows = (int64_t)((half - stats_bytes) / (size_t)row_bytes) / 256 * 256;
+    const int64_t row_bytes = (int64_t)w.K * (xdt == kF32 ? 4 : 2);        // a row of the caller's X
+    const int64_t max_rows = (int64_t)((half - stats_bytes) / (size_t)(w.K * 2)) / 256 * 256;    // staged rows are 16-bit
     if (max_rows < 256) return hipErrorOutOfMemory;
     const size_t ysize = ydt == kF32 ? 4 : 2;
     for (int64_t m_lo = 0; m_lo < M; m_lo += max_rows) {
@@ -665,13 +692,16 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
         u32x4_t* xst = reinterpret_cast<u32x4_t*>(workspace);
         const NormStats ns = {ssq_part, (int)grid.y};
         if (epi.gamma) {
-            if (widen) hipLaunchKernelGGL((stage_x_kernel<true, true, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
-            else if (xdt == kBF16) hipLaunchKernelGGL((stage_x_kernel<false, true, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
-            else hipLaunchKernelGGL((stage_x_kernel<false, false, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+            if (xdt == kF32) hipLaunchKernelGGL((stage_x_kernel<true, 2, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+            else if (widen) hipLaunchKernelGGL((stage_x_kernel<true, 1, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+            else if (xdt == kBF16) hipLaunchKernelGGL((stage_x_kernel<false, 1, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+            else hipLaunchKernelGGL((stage_x_kernel<false, 0, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+        } else if (xdt == kF32) {
+            hipLaunchKernelGGL((stage_x_kernel<true, 2, false>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
         } else if (widen) {
-            hipLaunchKernelGGL((stage_x_kernel<true, true, false>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+            hipLaunchKernelGGL((stage_x_kernel<true, 1, false>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
         } else {
-            hipLaunchKernelGGL((stage_x_kernel<false, false, false>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+            hipLaunchKernelGGL((stage_x_kernel<false, 0, false>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
         }
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;

@@ -126,8 +126,9 @@ int cybq_weight_info(const cybq_weight* w, int* quant, int64_t* N, int64_t* K,
  *   y  [M,N] row-major, ydt in {F32,F16,BF16} (fp32 accumulator rounded once)
  *   M >= 1.  M <= 16 runs the HBM-streaming decode kernels (17..32 rows: two
  *   passes of them), larger M the LDS-tiled MFMA prefill kernel (fp32
- *   activations: always the decode kernel, 16 rows at a time); there is no
- *   other path. */
+ *   activations in CYBQ_PREFILL_EXACT mode: the decode kernel, 16 rows at a
+ *   time; in FAST mode they are rounded once to f16 on the way in); there is
+ *   no other path. */
 int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt,
                 int64_t M, void* y, cybq_dtype ydt, void* stream);
 
@@ -178,7 +179,8 @@ int cybq_matmul_ex(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtyp
  *     rstd[m] = 1 / sqrt(mean_k x[m,k]^2 + eps)            (fp32, fixed summation order)
  *     y       = epilogue( rstd[m] * sum_k round(x[m,k] * gamma[k]) * W[n,k] )
  * x * gamma is formed in fp32 and rounded once to the kernel's operand type (the type
- * of x; f16 for bf16 x in the FAST prefill mode; two f16 halves for fp32 x) - what an
+ * of x; f16 for bf16 and fp32 x in the FAST prefill mode; two f16 halves for fp32 x
+ * elsewhere) - what an
  * unfused norm writing 16-bit activations would round too, minus its rounding of rstd.
  * gamma: [K] device pointer of type gdt, 16-byte aligned.  The definition is the LlamaStyle one and this
  * library's choice (the reference's is not visible in its tree). */
