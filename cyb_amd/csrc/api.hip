@@ -331,13 +331,14 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
     hipError_t e;
     if (M <= 16) {
         e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, epi, st);
-    } else if (M > 32 && (xdt != CYBQ_F32 || !ctx->prefill_exact)) {
+    } else if (xdt == CYBQ_F32 ? !ctx->prefill_exact : M > 32) {
         e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, ctx->workspace, ctx->workspace_bytes,
                               epi, st);
     } else {
         // fp32 activations keep full precision through the decode kernel's hi/lo split:
         // exact-mode prefill in fp32 is walked 16 rows at a time (FAST mode rounds them to f16
-        // in the staging pass and takes the MFMA kernel like any other).  So are 17..32
+        // in the staging pass and takes the MFMA kernel from 17 rows on: the LDS decode kernel
+        // needs 52 - 65 us for 24 - 32 fp32 rows, the MFMA kernel 31).  So are 17..32
         // rows of 16-bit activations: two passes of the batched-rows kernel stream the
         // weights twice and are still quicker than a 128-row MFMA tile mostly empty.
         e = hipSuccess;

@@ -127,8 +127,8 @@ int cybq_weight_info(const cybq_weight* w, int* quant, int64_t* N, int64_t* K,
  *   M >= 1.  M <= 16 runs the HBM-streaming decode kernels (17..32 rows: two
  *   passes of them), larger M the LDS-tiled MFMA prefill kernel (fp32
  *   activations in CYBQ_PREFILL_EXACT mode: the decode kernel, 16 rows at a
- *   time; in FAST mode they are rounded once to f16 on the way in); there is
- *   no other path. */
+ *   time; in FAST mode they are rounded once to f16 on the way in and take
+ *   the prefill kernel from 17 rows on); there is no other path. */
 int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt,
                 int64_t M, void* y, cybq_dtype ydt, void* stream);
 

@@ -297,9 +297,9 @@ def test_prefill_matches_oracle(backend, oracle, prefill_mode, bits, xdt, M):
     err = oracle.rel_l2(y, oracle.matmul_f64(q, s, x.float().cpu().numpy()))
     # fp32 activations: exact through the decode kernel's hi/lo split up to 32 rows and in EXACT mode;
     # FAST prefill rounds them to f16 in the staging pass like any other
-    exact_path = M <= 32 or prefill_mode == "exact"
+    exact_path = M <= (16 if xdt == "f32" else 32) or prefill_mode == "exact"
     assert err < (TIGHT if (xdt == "f32" and exact_path) else _bar(prefill_mode)), err
-    if prefill_mode == "fast" and M > 32:
+    if prefill_mode == "fast" and M > (16 if xdt == "f32" else 32):
         assert err > 1e-6        # the rounded-weight kernel really ran (up to 32 rows take the exact decode kernel)
 
 
@@ -527,7 +527,7 @@ def test_folded_rmsnorm(backend, oracle, prefill_mode, bits, M, xdt, gdt):
     backend.matmul_norm(qw, x, gamma, eps, y)
     torch.cuda.synchronize()
     assert not torch.isnan(y).any()
-    fast_prefill = M > 32 and prefill_mode == "fast"
+    fast_prefill = M > (16 if xdt == "f32" else 32) and prefill_mode == "fast"
     op_dt = "f16" if (fast_prefill and xdt != "f16") else xdt       # FAST multiplies in f16
     ref = _norm_ref(oracle, q, s, x, gamma, eps, op_dt)
     bar = FAST if fast_prefill else TIGHT
@@ -591,7 +591,7 @@ def test_random_calls_match_float64(backend, oracle, case):
             x[M // 2] *= 5.0
         gamma = (1.0 + 0.25 * torch.from_numpy(synth.activations(61, 1, K)[0])).cuda().to(TDT[c["gdt"]])
         eps = 1e-5
-        prefill = M > 32 and (c["xdt"] != "f32" or c["mode"] == "fast")
+        prefill = (M > 32 and c["xdt"] != "f32") or (M > 16 and c["xdt"] == "f32" and c["mode"] == "fast")
         fast = prefill and c["mode"] == "fast"
         op_dt = "f16" if (fast and c["xdt"] != "f16") else c["xdt"]
 
