@@ -25,9 +25,8 @@ struct cybq_weight {
     int bits = 0;
     int64_t N = 0, K = 0;
     int NT = 0, KT = 0;
-    uint32_t* q = nullptr;
-    uint16_t* s = nullptr;
-    size_t q_bytes = 0, s_bytes = 0;
+    uint8_t* data = nullptr;            // native tiles (q words + scales per tile), strip-major
+    size_t bytes = 0;
     bool paired = false;                // made by cybq_weight_fuse_pairs: strips alternate gate / up
 };
 
@@ -58,8 +57,7 @@ struct DeviceGuard {
 cybq::WeightView view_of(const cybq_weight* w)
 {
     cybq::WeightView v;
-    v.q = w->q;
-    v.s = w->s;
+    v.base = w->data;
     v.N = (int)w->N;
     v.K = (int)w->K;
     v.NT = w->NT;
@@ -83,12 +81,9 @@ int alloc_weight(cybq_ctx* ctx, int bits, int64_t N, int64_t K, cybq_weight** ou
     w->K = K;
     w->NT = (int)((N + cybq::kTileN - 1) / cybq::kTileN);
     w->KT = (int)((K + cybq::kTileK - 1) / cybq::kTileK);
-    w->q_bytes = (size_t)w->NT * w->KT * (bits == 4 ? 1024 : 2048);
-    w->s_bytes = (size_t)w->NT * w->KT * 128;
-    hipError_t e = hipMalloc(reinterpret_cast<void**>(&w->q), w->q_bytes);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&w->s), w->s_bytes);
+    w->bytes = (size_t)w->NT * w->KT * cybq::tile_bytes(bits);
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&w->data), w->bytes);
     if (e != hipSuccess) {
-        if (w->q) (void)hipFree(w->q);
         delete w;
         return fail_hip(ctx, e, "hipMalloc(weight)");
     }
@@ -203,12 +198,11 @@ int cybq_weight_upload(cybq_ctx* ctx, cybq_quant quant, cybq_layout layout, int6
         e = hipMemcpy(q_tmp, q, q_src_bytes, hipMemcpyHostToDevice);
         if (e == hipSuccess && s_src_bytes) e = hipMemcpy(s_tmp, scales, s_src_bytes, hipMemcpyHostToDevice);
         if (e == hipSuccess)
-            e = cybq::launch_repack(quant, layout, q_tmp, s_tmp, w->q, w->s, (int)N, (int)K, w->NT, w->KT, nullptr);
+            e = cybq::launch_repack(quant, layout, q_tmp, s_tmp, w->data, (int)N, (int)K, w->NT, w->KT, nullptr);
         if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
         if (e != hipSuccess) {
             rc = fail_hip(ctx, e, "weight upload");
-            (void)hipFree(w->q);
-            (void)hipFree(w->s);
+            (void)hipFree(w->data);
             delete w;
             w = nullptr;
         }
@@ -227,6 +221,8 @@ int cybq_weight_from_device(cybq_ctx* ctx, cybq_quant quant, int64_t N, int64_t 
     if (!out) return fail(ctx, CYBQ_ERR_INVALID, "out is NULL");
     *out = nullptr;
     if (!q_dev || !scales_dev) return fail(ctx, CYBQ_ERR_INVALID, "q_dev / scales_dev is NULL");
+    if (reinterpret_cast<uintptr_t>(q_dev) % 4 || reinterpret_cast<uintptr_t>(scales_dev) % 2)
+        return fail(ctx, CYBQ_ERR_ALIGN, "q_dev must be 4-byte and scales_dev 2-byte aligned");
     int rc = check_weight_shape(ctx, quant, N, K);
     if (rc) return rc;
     DeviceGuard guard(ctx->device);
@@ -234,11 +230,10 @@ int cybq_weight_from_device(cybq_ctx* ctx, cybq_quant quant, int64_t N, int64_t 
     cybq_weight* w = nullptr;
     rc = alloc_weight(ctx, quant, N, K, &w);
     if (rc) return rc;
-    hipError_t e = cybq::launch_repack(quant, CYBQ_LAYOUT_PLANAR, q_dev, scales_dev, w->q, w->s, (int)N, (int)K,
+    hipError_t e = cybq::launch_repack(quant, CYBQ_LAYOUT_PLANAR, q_dev, scales_dev, w->data, (int)N, (int)K,
                                        w->NT, w->KT, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) {
-        (void)hipFree(w->q);
-        (void)hipFree(w->s);
+        (void)hipFree(w->data);
         delete w;
         return fail_hip(ctx, e, "repack launch");
     }
@@ -257,11 +252,9 @@ int cybq_weight_clone(cybq_ctx* ctx, const cybq_weight* src, cybq_weight** out)
     cybq_weight* w = nullptr;
     int rc = alloc_weight(ctx, src->bits, src->N, src->K, &w);
     if (rc) return rc;
-    hipError_t e = hipMemcpy(w->q, src->q, src->q_bytes, hipMemcpyDeviceToDevice);
-    if (e == hipSuccess) e = hipMemcpy(w->s, src->s, src->s_bytes, hipMemcpyDeviceToDevice);
+    hipError_t e = hipMemcpy(w->data, src->data, src->bytes, hipMemcpyDeviceToDevice);
     if (e != hipSuccess) {
-        (void)hipFree(w->q);
-        (void)hipFree(w->s);
+        (void)hipFree(w->data);
         delete w;
         return fail_hip(ctx, e, "weight clone");
     }
@@ -274,11 +267,9 @@ int cybq_weight_free(cybq_ctx* ctx, cybq_weight* w)
 {
     if (!w) return CYBQ_OK;
     hipError_t e = hipSetDevice(w->device);
-    if (e == hipSuccess) e = hipFree(w->q);
-    hipError_t e2 = hipFree(w->s);
+    if (e == hipSuccess) e = hipFree(w->data);
     delete w;
     if (e != hipSuccess) return fail_hip(ctx, e, "hipFree(weight)");
-    if (e2 != hipSuccess) return fail_hip(ctx, e2, "hipFree(weight)");
     return CYBQ_OK;
 }
 
@@ -288,7 +279,7 @@ int cybq_weight_info(const cybq_weight* w, int* quant, int64_t* N, int64_t* K, i
     if (quant) *quant = w->bits;
     if (N) *N = w->N;
     if (K) *K = w->K;
-    if (device_bytes) *device_bytes = (int64_t)(w->q_bytes + w->s_bytes);
+    if (device_bytes) *device_bytes = (int64_t)w->bytes;
     return CYBQ_OK;
 }
 
@@ -393,15 +384,12 @@ int cybq_weight_fuse_pairs(cybq_ctx* ctx, const cybq_weight* gate, const cybq_we
     int rc = alloc_weight(ctx, gate->bits, 2 * gate->N, gate->K, &w);
     if (rc) return rc;
     // the native layout is strip-major: output strip 2i is gate strip i, 2i+1 is up strip i
-    const size_t qs = (size_t)gate->KT * (gate->bits == 4 ? 1024 : 2048), ss = (size_t)gate->KT * 128;
-    hipError_t e = hipMemcpy2D(w->q, 2 * qs, gate->q, qs, qs, gate->NT, hipMemcpyDeviceToDevice);
-    if (e == hipSuccess) e = hipMemcpy2D(reinterpret_cast<char*>(w->q) + qs, 2 * qs, up->q, qs, qs, up->NT, hipMemcpyDeviceToDevice);
-    if (e == hipSuccess) e = hipMemcpy2D(w->s, 2 * ss, gate->s, ss, ss, gate->NT, hipMemcpyDeviceToDevice);
-    if (e == hipSuccess) e = hipMemcpy2D(reinterpret_cast<char*>(w->s) + ss, 2 * ss, up->s, ss, ss, up->NT, hipMemcpyDeviceToDevice);
+    const size_t sb = (size_t)gate->KT * cybq::tile_bytes(gate->bits);          // bytes of one strip
+    hipError_t e = hipMemcpy2D(w->data, 2 * sb, gate->data, sb, sb, gate->NT, hipMemcpyDeviceToDevice);
+    if (e == hipSuccess) e = hipMemcpy2D(w->data + sb, 2 * sb, up->data, sb, sb, up->NT, hipMemcpyDeviceToDevice);
     if (e == hipSuccess) e = hipDeviceSynchronize();
     if (e != hipSuccess) {
-        (void)hipFree(w->q);
-        (void)hipFree(w->s);
+        (void)hipFree(w->data);
         delete w;
         return fail_hip(ctx, e, "weight fuse");
     }

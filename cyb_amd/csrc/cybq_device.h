@@ -3,20 +3,24 @@
 //
 // Native layout.  A weight tensor W[N,K] is cut into tiles of 16 rows x 128 k
 // (4 scale groups).  Tiles are stored strip-major: tile (nt, kt) sits at index
-// nt*KT + kt, so a 16-row strip is one contiguous stream along K.
+// nt*KT + kt, so a 16-row strip is one contiguous stream along K.  A tile is its
+// q words followed by its scales, one contiguous record (1152 B for Q4, 2176 B
+// for Q8): a kernel that streams a strip reads one run of memory.
 //
-//   Q4 q plane : tile = 64 lanes x 16 B (1024 B).  Lane l, word j (0..3) holds
-//       row   n = 16*nt + (l & 15)
-//       group g = 4*kt + j
-//       the 8 weights k = 32*g + 8*(l >> 4) + s,  s = 0..7
-//       as nibbles u = q + 8, weight s at nibble position (s >> 1) + 4*(s & 1).
-//     One 128-bit load per lane is therefore four ready-made B operands of
-//     v_mfma_f32_16x16x32 (lane = column n, 8 consecutive k per lane), and the
-//     nibble order lets one and-or peel two weights into one packed-f16 register.
-//   Q8 q plane : tile = 2 halves x 64 lanes x 16 B (2048 B).  Half h, lane l
+//   Q4 q part  : 64 lanes x 16 B (1024 B).  Lane l owns row n = 16*nt + (l & 15)
+//       and the k octet o = l >> 4 of every scale group: for group j (0..3) and slot
+//       s (0..7), weight k = 128*kt + 32*j + 8*o + s is the nibble u = q + 8 of
+//       word  2*(j >> 1) + (s >> 2)  at bit  16*(s & 1) + 8*((s >> 1) & 1) + 4*(j & 1).
+//     Read as four MFMA B operands (lane = column n, 8 consecutive k per lane): a
+//     word pair (2p, 2p+1) holds groups 2p (low nibble of every byte) and 2p+1 (high
+//     nibble), and (w & 0x000F000F), ((w >> 8) & 0x000F000F) are the slots (0,1),
+//     (2,3) of the even group as two 16-bit integers each - which, read as IEEE f16,
+//     are the subnormals u * 2^-24 - while the mask 0x00F000F0 yields the odd
+//     group as 16u * 2^-24.  One shift and four ANDs turn a word into operands.
+//   Q8 q part  : 2 halves x 64 lanes x 16 B (2048 B).  Half h, lane l
 //     holds groups 4*kt + 2*h and 4*kt + 2*h + 1, 8 bytes each, byte s =
 //     q + 128 for k = 32*g + 8*(l >> 4) + s.
-//   scale plane: tile = 16 rows x 4 groups of IEEE f16 (128 B): [row][group].
+//   scale part : 16 rows x 4 groups of IEEE f16 (128 B): [row][group].
 //
 // N is padded to 16 and K to 128 with q = 0 / scale = 0.
 #pragma once
@@ -30,6 +34,11 @@ constexpr int kGroup = 32;
 constexpr int kTileN = 16;
 constexpr int kTileK = 128;
 constexpr int kGroupsPerTile = kTileK / kGroup;
+constexpr int kTileScaleBytes = kTileN * kGroupsPerTile * 2;              // 128
+template <int BITS> constexpr int kTileQBytes = BITS == 4 ? 1024 : 2048;
+template <int BITS> constexpr int kTileBytes = kTileQBytes<BITS> + kTileScaleBytes;
+__host__ __device__ inline int tile_q_bytes(int bits) { return bits == 4 ? 1024 : 2048; }
+__host__ __device__ inline int tile_bytes(int bits) { return tile_q_bytes(bits) + kTileScaleBytes; }
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -52,8 +61,9 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t bits16)
     return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
 }
 
-// nibble position of weight slot s inside a native Q4 word
-__host__ __device__ __forceinline__ int q4_nibble_pos(int s) { return (s >> 1) + 4 * (s & 1); }
+// where weight (group j, slot s) of a lane sits inside the lane's four Q4 words
+__host__ __device__ __forceinline__ int q4_word(int j, int s) { return 2 * (j >> 1) + (s >> 2); }
+__host__ __device__ __forceinline__ int q4_shift(int j, int s) { return 16 * (s & 1) + 8 * ((s >> 1) & 1) + 4 * (j & 1); }
 
 // The f16 magic constant 0x64006400 held in a vector register whose value the
 // compiler cannot see.  With it (w & mask) | magic compiles to one v_and_or_b32
@@ -67,24 +77,37 @@ __device__ __forceinline__ uint32_t q4_magic_vgpr()
     return mv;
 }
 
-// One native Q4 word -> 8 exact f16 integers in MFMA operand order.
-// 0x6400 | u is the f16 number 1024 + u; 0x6400 | (u << 4) is 1024 + 16u.
-// `magic` = q4_magic_vgpr().
-__device__ __forceinline__ void unpack_q4_f16(uint32_t w, uint32_t magic, uint32_t out[4])
+// Group 2p + t of a tile from the word pair (wa, wb) = words 2p, 2p + 1 of a lane
+// -> 8 exact f16 integers in MFMA operand order.  0x6400 | u is the f16 number
+// 1024 + u; 0x6400 | (u << 4) is 1024 + 16u.  `magic` = q4_magic_vgpr().
+__device__ __forceinline__ void unpack_q4_f16(uint32_t wa, uint32_t wb, int t, uint32_t magic, uint32_t out[4])
 {
-    const uint32_t lo = 0x000F000Fu, hi = 0x00F000F0u;
-    const half2_t sub = {(_Float16)-1032.0f, (_Float16)-1032.0f};
-    const half2_t mul = {(_Float16)0.0625f, (_Float16)0.0625f};
-    const half2_t add = {(_Float16)-72.0f, (_Float16)-72.0f};
-    uint32_t w8 = w >> 8;
-    half2_t t0 = as_h2((w & lo) | magic) + sub;
-    half2_t t1 = as_h2((w & hi) | magic) * mul + add;
-    half2_t t2 = as_h2((w8 & lo) | magic) + sub;
-    half2_t t3 = as_h2((w8 & hi) | magic) * mul + add;
-    out[0] = as_u32(t0);
-    out[1] = as_u32(t1);
-    out[2] = as_u32(t2);
-    out[3] = as_u32(t3);
+    const uint32_t src[4] = {wa, wa >> 8, wb, wb >> 8};
+    if (t == 0) {
+        const half2_t sub = {(_Float16)-1032.0f, (_Float16)-1032.0f};
+#pragma unroll
+        for (int i = 0; i < 4; i++) out[i] = as_u32(as_h2((src[i] & 0x000F000Fu) | magic) + sub);
+    } else {
+        const half2_t mul = {(_Float16)0.0625f, (_Float16)0.0625f};
+        const half2_t add = {(_Float16)-72.0f, (_Float16)-72.0f};
+#pragma unroll
+        for (int i = 0; i < 4; i++) out[i] = as_u32(as_h2((src[i] & 0x00F000F0u) | magic) * mul + add);
+    }
+}
+
+// The same group as f16 subnormals: u * 2^-24 (t = 0) or 16u * 2^-24 (t = 1), u = q + 8.
+// The matrix cores of gfx950 take f16 subnormals at face value, so these ARE operands; a
+// caller takes the bias off with one more MFMA of its activations against the constant
+// operand kSubBiasL / kSubBiasH (-8 * 2^-24, -128 * 2^-24) and folds 2^24 (and the 16 of
+// an odd group) into the scale.
+constexpr uint32_t kSubBiasL = 0x80088008u, kSubBiasH = 0x80808080u;
+__device__ __forceinline__ void unpack_q4_sub(uint32_t wa, uint32_t wb, int t, uint32_t out[4])
+{
+    const uint32_t m = t ? 0x00F000F0u : 0x000F000Fu;
+    out[0] = wa & m;
+    out[1] = (wa >> 8) & m;
+    out[2] = wb & m;
+    out[3] = (wb >> 8) & m;
 }
 
 // The bf16 counterpart: 0x4300 | u is the bf16 number 128 + u (7 mantissa bits, so
@@ -100,13 +123,13 @@ __device__ __forceinline__ uint32_t q4_magic_vgpr_bf16()
 }
 constexpr uint32_t kBf16Neg136x2 = 0xC308C308u;
 
-__device__ __forceinline__ void unpack_q4_bf16_biased(uint32_t w, uint32_t magic, uint32_t out[4])
+__device__ __forceinline__ void unpack_q4_bf16_biased(uint32_t wa, uint32_t wb, int t, uint32_t magic, uint32_t out[4])
 {
     const uint32_t lo = 0x000F000Fu;
-    out[0] = (w & lo) | magic;
-    out[1] = ((w >> 4) & lo) | magic;
-    out[2] = ((w >> 8) & lo) | magic;
-    out[3] = ((w >> 12) & lo) | magic;
+    out[0] = ((wa >> (4 * t)) & lo) | magic;
+    out[1] = ((wa >> (4 * t + 8)) & lo) | magic;
+    out[2] = ((wb >> (4 * t)) & lo) | magic;
+    out[3] = ((wb >> (4 * t + 8)) & lo) | magic;
 }
 
 // Two native Q8 words (8 bytes, u = q + 128) -> 8 exact f16 integers.
@@ -148,9 +171,9 @@ __device__ __forceinline__ void unpack_q8_bf16_biased(uint32_t w0, uint32_t w1, 
 }
 
 // signed value of weight slot s of a native Q4 word / Q8 word pair (scalar helpers)
-__device__ __forceinline__ int q4_slot_value(uint32_t w, int s)
+__host__ __device__ __forceinline__ int q4_slot_value(const uint32_t words[4], int j, int s)
 {
-    return (int)((w >> (4 * q4_nibble_pos(s))) & 15u) - 8;
+    return (int)((words[q4_word(j, s)] >> q4_shift(j, s)) & 15u) - 8;
 }
 __device__ __forceinline__ int q8_slot_value(uint32_t w0, uint32_t w1, int s)
 {
@@ -179,11 +202,22 @@ struct Epilogue {
 __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
 
 struct WeightView {       // what kernels need to know about an uploaded tensor
-    const uint32_t* q;    // native q plane
-    const uint16_t* s;    // native scale plane
+    const uint8_t* base;  // native tiles, strip-major
     int N, K;             // logical
     int NT, KT;           // tiles (padded)
     int bits;             // 4 or 8
 };
+
+// q words and scales of tile index `tile` (= nt*KT + kt)
+template <int BITS>
+__device__ __forceinline__ const u32x4_t* tile_q(const WeightView& w, int64_t tile)
+{
+    return reinterpret_cast<const u32x4_t*>(w.base + tile * kTileBytes<BITS>);
+}
+template <int BITS>
+__device__ __forceinline__ const u32x2_t* tile_s(const WeightView& w, int64_t tile)
+{
+    return reinterpret_cast<const u32x2_t*>(w.base + tile * kTileBytes<BITS> + kTileQBytes<BITS>);
+}
 
 }  // namespace cybq

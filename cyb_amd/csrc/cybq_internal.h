@@ -13,8 +13,9 @@ namespace cybq {
 // dtype codes mirror enum cybq_dtype
 constexpr int kF32 = 0, kF16 = 1, kBF16 = 2;
 
-hipError_t launch_repack(int bits, int layout, const void* q, const void* scales, uint32_t* qdst,
-                         uint16_t* sdst, int N, int K, int NT, int KT, hipStream_t st);
+// q: PLANAR q plane (4-byte aligned) with `scales`, or BLOCK_AOS blocks (2-byte aligned, scales unused)
+hipError_t launch_repack(int bits, int layout, const void* q, const void* scales, uint8_t* dst, int N, int K, int NT, int KT,
+                         hipStream_t st);
 hipError_t launch_dequant(const WeightView& w, float* out, hipStream_t st);
 
 // decode path, 1 <= M <= 16 per call (api.hip walks 17..32 rows as two calls)

@@ -116,16 +116,12 @@ struct WRegs {               // one native weight tile as loaded by one lane, an
 };
 
 template <int BITS>
-__device__ __forceinline__ void load_wtile(WRegs<BITS>& r, const u32x4_t* qp, const u32x2_t* sp, int64_t tile,
-                                           int lane)
+__device__ __forceinline__ void load_wtile(WRegs<BITS>& r, const WeightView& w, int64_t tile, int lane)
 {
-    if (BITS == 4) {
-        r.q[0] = qp[tile * 64 + lane];
-    } else {
-        r.q[0] = qp[tile * 128 + lane];
-        r.q[BITS == 4 ? 0 : 1] = qp[tile * 128 + 64 + lane];
-    }
-    r.s = sp[tile * 16 + (lane & 15)];
+    const u32x4_t* qp = tile_q<BITS>(w, tile);
+    r.q[0] = qp[lane];
+    if (BITS == 8) r.q[BITS == 4 ? 0 : 1] = qp[64 + lane];
+    r.s = tile_s<BITS>(w, tile)[lane & 15];
 }
 
 // (w0, w1) fp32 -> packed 16-bit hi pair and lo pair with hi + lo == w
@@ -153,7 +149,7 @@ __device__ __forceinline__ void dequant_group_to_lds(const WRegs<BITS>& r, int j
                                                      int lane)
 {
     uint32_t bw[4];
-    if (BITS == 4) unpack_q4_f16(r.q[0][j], magic, bw);
+    if (BITS == 4) unpack_q4_f16(r.q[0][2 * (j >> 1)], r.q[0][2 * (j >> 1) + 1], j & 1, magic, bw);
     else unpack_q8_f16(r.q[(BITS == 4) ? 0 : (j >> 1)][(j & 1) * 2], r.q[(BITS == 4) ? 0 : (j >> 1)][(j & 1) * 2 + 1], bw);
     const uint32_t sb = (j & 1) ? (r.s[j >> 1] >> 16) : (r.s[j >> 1] & 0xffffu);
     if (!EXACT) {
@@ -247,9 +243,6 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
         return kt_lo + (r >= KT ? r - KT : r);
     };
 
-    const u32x4_t* qp = reinterpret_cast<const u32x4_t*>(w.q);
-    const u32x2_t* sp = reinterpret_cast<const u32x2_t*>(w.s);
-
     // X arrives staged in A-operand order (stage_x_kernel): row block rb, scale group
     // g is one contiguous KB, lane after lane, so a load is one wave-uniform base
     // plus lane * 16 B and adjacent lanes read adjacent memory.  Row blocks past the
@@ -278,7 +271,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
     }
     auto load_units = [&](WRegs<BITS> (&dst)[WT], int kt) {
 #pragma unroll
-        for (int t = 0; t < WT; t++) load_wtile<BITS>(dst[t], qp, sp, wtile[t] + rot(kt), lane);
+        for (int t = 0; t < WT; t++) load_wtile<BITS>(dst[t], w, wtile[t] + rot(kt), lane);
     };
     auto stage_units = [&](WRegs<BITS> (&src)[WT], int j, u32x4_t* buf) {
 #pragma unroll

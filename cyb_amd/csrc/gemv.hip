@@ -31,15 +31,10 @@ struct TileRegs {
 template <int BITS>
 __device__ __forceinline__ void load_tile(TileRegs<BITS>& t, const WeightView& w, int64_t tile, int lane)
 {
-    const u32x4_t* qp = reinterpret_cast<const u32x4_t*>(w.q);
-    if (BITS == 4) {
-        t.q[0] = __builtin_nontemporal_load(qp + tile * 64 + lane);
-    } else {
-        t.q[0] = __builtin_nontemporal_load(qp + tile * 128 + lane);
-        t.q[1] = __builtin_nontemporal_load(qp + tile * 128 + 64 + lane);
-    }
-    const u32x2_t* sp = reinterpret_cast<const u32x2_t*>(w.s);
-    t.s = __builtin_nontemporal_load(sp + tile * 16 + (lane & 15));
+    const u32x4_t* qp = tile_q<BITS>(w, tile);
+    t.q[0] = __builtin_nontemporal_load(qp + lane);
+    if (BITS == 8) t.q[BITS == 8 ? 1 : 0] = __builtin_nontemporal_load(qp + 64 + lane);
+    t.s = __builtin_nontemporal_load(tile_s<BITS>(w, tile) + (lane & 15));
 }
 
 __device__ __forceinline__ void store_out(void* y, int ydt, int64_t idx, float v)
@@ -168,11 +163,11 @@ __device__ __forceinline__ void tile_issue(const TileRegs<BITS>& t, const uint16
     for (int j = 0; j < 4; j++) {
         uint32_t bw[4];
         if (BITS == 4 && XMODE == XBF16) {
-            unpack_q4_bf16_biased(t.q[0][j], magic, bw);
+            unpack_q4_bf16_biased(t.q[0][2 * (j >> 1)], t.q[0][2 * (j >> 1) + 1], j & 1, magic, bw);
         } else if (XMODE == XBF16) {
             unpack_q8_bf16_biased(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
         } else {
-            if (BITS == 4) unpack_q4_f16(t.q[0][j], magic, bw);
+            if (BITS == 4) unpack_q4_f16(t.q[0][2 * (j >> 1)], t.q[0][2 * (j >> 1) + 1], j & 1, magic, bw);
             else unpack_q8_f16(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
         }
         b[j].u = (u32x4_t){bw[0], bw[1], bw[2], bw[3]};
@@ -545,11 +540,11 @@ __device__ __forceinline__ void tile_issue_regs(const TileRegs<BITS>& t, const F
     for (int j = 0; j < 4; j++) {
         uint32_t bw[4];
         if (BITS == 4 && XMODE == XBF16) {
-            unpack_q4_bf16_biased(t.q[0][j], magic, bw);
+            unpack_q4_bf16_biased(t.q[0][2 * (j >> 1)], t.q[0][2 * (j >> 1) + 1], j & 1, magic, bw);
         } else if (XMODE == XBF16) {
             unpack_q8_bf16_biased(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
         } else {
-            if (BITS == 4) unpack_q4_f16(t.q[0][j], magic, bw);
+            if (BITS == 4) unpack_q4_f16(t.q[0][2 * (j >> 1)], t.q[0][2 * (j >> 1) + 1], j & 1, magic, bw);
             else unpack_q8_f16(t.q[j >> 1][(j & 1) * 2], t.q[j >> 1][(j & 1) * 2 + 1], bw);
         }
         b[j].u = (u32x4_t){bw[0], bw[1], bw[2], bw[3]};

@@ -1,0 +1,265 @@
+// gemv1.hip - decode kernel for ONE activation row: y[1,N] = x[1,K] * W^T, f16 activations.
+//
+// HBM-bound: a workgroup owns one 16-row strip of W (one contiguous run of memory) and
+// requests all of it up front; everything else is arranged so that nothing stands between
+// the kernel's start and those requests, and so that little remains to do once the last
+// byte has arrived.
+//
+//  * No LDS staging of x, no barrier before the arithmetic.  A wave works on "sets" of four
+//    consecutive K tiles (512 k, 16 scale groups).  Its MFMA A operand for a set is ONE
+//    16-byte load per lane: lane (i = l & 15, o = l >> 4) reads x[512*set + 32*i + 8*o ..+8],
+//    so row i of the 16x16x32 MFMA holds the activations of scale group i of the set.
+//    Multiplying that operand with the weights of group g gives the wanted dot products in
+//    output row g (rows != g pair the weights with another group's activations and are
+//    ignored).  Output row g = 4*b + r lives in register r of lane block b (lanes 16b..16b+15):
+//    lane block b ends up with tile b of the set, register r with scale group r - exactly
+//    the four scales a lane gets from one 8-byte load of the tile's scale record.
+//  * Weight operands cost one shift and four ANDs per eight weights: the native nibble
+//    order makes (w & 0x000F000F) two f16 subnormals u * 2^-24 (u = q + 8), which the matrix
+//    cores take at face value.  The bias comes off inside the same accumulation: the MFMA's C
+//    operand is x times the constant -8 * 2^-24 (one extra MFMA per set, its row g is exactly
+//    -8 * sum of group g's activations).  Odd groups sit in the high nibbles (16u * 2^-24,
+//    constant -128 * 2^-24); the 16 and the 2^24 are folded into the final scaling.
+//    Q8 bytes u = q + 128 become subnormals with one byte permute per pair.
+//  * Per-group f16 scales are applied in fp32 on the MFMA results; lanes add up what their
+//    block owns, blocks meet through two cross-lane moves, waves through LDS in wave order:
+//    the order of all additions is fixed, results are reproducible.
+#include "cybq_device.h"
+#include "cybq_internal.h"
+
+namespace cybq {
+
+namespace {
+
+__device__ __forceinline__ void store_out1(void* y, int ydt, int64_t idx, float v)
+{
+    if (ydt == kF32) reinterpret_cast<float*>(y)[idx] = v;
+    else if (ydt == kF16) reinterpret_cast<_Float16*>(y)[idx] = (_Float16)v;
+    else reinterpret_cast<uint16_t*>(y)[idx] = f32_to_bf16_bits(v);
+}
+
+__device__ __forceinline__ float load_out1(const void* p, int dt, int64_t idx)
+{
+    if (dt == kF32) return reinterpret_cast<const float*>(p)[idx];
+    if (dt == kF16) return (float)reinterpret_cast<const _Float16*>(p)[idx];
+    return __builtin_bit_cast(float, (uint32_t)reinterpret_cast<const uint16_t*>(p)[idx] << 16);
+}
+
+// B operand of scale group r of one tile as loaded by a lane
+template <int BITS>
+__device__ __forceinline__ Frag16 sub_operand(const u32x4_t (&q)[BITS == 4 ? 1 : 2], int r)
+{
+    Frag16 b;
+    if (BITS == 4) {
+        uint32_t o[4];
+        unpack_q4_sub(q[0][2 * (r >> 1)], q[0][2 * (r >> 1) + 1], r & 1, o);
+        b.u = (u32x4_t){o[0], o[1], o[2], o[3]};
+    } else {
+        // bytes [b0 b1 b2 b3] -> halves [b0, b1], [b2, b3] zero-extended (selector 0x0c = constant 0)
+        const uint32_t w0 = q[BITS == 4 ? 0 : (r >> 1)][(r & 1) * 2], w1 = q[BITS == 4 ? 0 : (r >> 1)][(r & 1) * 2 + 1];
+        b.u = (u32x4_t){__builtin_amdgcn_perm(0u, w0, 0x0c010c00u), __builtin_amdgcn_perm(0u, w0, 0x0c030c02u),
+                        __builtin_amdgcn_perm(0u, w1, 0x0c010c00u), __builtin_amdgcn_perm(0u, w1, 0x0c030c02u)};
+    }
+    return b;
+}
+
+// SETS: sets a wave owns (set index wv + nwaves * h).  NS: strips per workgroup (2 = a gate strip
+// and its up strip, SwiGLU epilogue).  EVEN: K is a multiple of 512 and every wave has SETS
+// whole sets, so nothing needs clamping.
+template <int BITS, int SETS, int NS, bool EVEN>
+__global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float16* __restrict__ x, void* __restrict__ y, int ydt,
+                                                     Epilogue epi)
+{
+    constexpr int QV = BITS == 4 ? 1 : 2;
+    __shared__ float red[NS * 16 * 16];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nwaves = (int)blockDim.x >> 6;
+    const int row = lane & 15, blk = lane >> 4;
+    const int KT = w.KT;
+
+    Frag16 a[SETS];
+    u32x2_t sc[NS][SETS];
+    u32x4_t q[NS][SETS][4][QV];
+    bool tile_ok[SETS];               // this lane block's tile of the set exists (!EVEN)
+#pragma unroll
+    for (int h = 0; h < SETS; h++) {
+        const int set = wv + nwaves * h;
+        const int k = set * 512 + row * 32 + blk * 8;
+        if (EVEN) {
+            a[h].u = *reinterpret_cast<const u32x4_t*>(x + k);
+        } else {
+            a[h].u = *reinterpret_cast<const u32x4_t*>(x + min(k, w.K - 8));
+            tile_ok[h] = 4 * set + blk < KT;
+        }
+    }
+#pragma unroll
+    for (int st = 0; st < NS; st++) {
+        const int64_t strip = (int64_t)(blockIdx.x * NS + st) * KT;
+#pragma unroll
+        for (int h = 0; h < SETS; h++) {
+            const int t0 = 4 * (wv + nwaves * h);
+            sc[st][h] = __builtin_nontemporal_load(tile_s<BITS>(w, strip + (EVEN ? t0 + blk : min(t0 + blk, KT - 1))) + row);
+        }
+#pragma unroll
+        for (int h = 0; h < SETS; h++) {
+            const int t0 = 4 * (wv + nwaves * h);
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const u32x4_t* qp = tile_q<BITS>(w, strip + (EVEN ? t0 + b : min(t0 + b, KT - 1)));
+#pragma unroll
+                for (int v = 0; v < QV; v++) q[st][h][b][v] = __builtin_nontemporal_load(qp + v * 64 + lane);
+            }
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);       // every request is out before any arithmetic
+
+    if (!EVEN) {
+#pragma unroll
+        for (int h = 0; h < SETS; h++) {
+            // activations past K (the padded tail of the last tile) count as zero; a tile past
+            // the end of the strip was clamped to the last one and gets scale zero
+            const bool x_ok = (wv + nwaves * h) * 512 + row * 32 + blk * 8 < w.K;
+#pragma unroll
+            for (int p = 0; p < 4; p++) a[h].u[p] = x_ok ? a[h].u[p] : 0u;
+#pragma unroll
+            for (int st = 0; st < NS; st++) {
+                sc[st][h][0] = tile_ok[h] ? sc[st][h][0] : 0u;
+                sc[st][h][1] = tile_ok[h] ? sc[st][h][1] : 0u;
+            }
+        }
+    }
+
+    Frag16 kL, kH;
+    kL.u = (u32x4_t){kSubBiasL, kSubBiasL, kSubBiasL, kSubBiasL};
+    kH.u = (u32x4_t){kSubBiasH, kSubBiasH, kSubBiasH, kSubBiasH};
+    const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+    float4_t biasL[SETS], biasH[SETS];
+#pragma unroll
+    for (int h = 0; h < SETS; h++) {
+        if (BITS == 4) biasL[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[h].h, kL.h, zero, 0, 0, 0);
+        biasH[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[h].h, kH.h, zero, 0, 0, 0);
+    }
+
+    // Lane block b holds meaningful sums only for tile b of every set.  All four tiles are
+    // accumulated with the lane's own scales (the other three sums are finite and unused) and the
+    // meaningful one is picked once at the end.  Even groups (low nibbles) and odd groups
+    // (high nibbles, 16 times too large) are kept apart until the final scaling.
+    float accL[NS][4], accH[NS][4];
+#pragma unroll
+    for (int st = 0; st < NS; st++)
+#pragma unroll
+        for (int b = 0; b < 4; b++) accL[st][b] = accH[st][b] = 0.f;
+    constexpr int T = NS * SETS * 4;
+    float4_t dprev[4];
+#pragma unroll
+    for (int i = 0; i <= T; i++) {
+        // MFMAs of tile i first, then the scaling of tile i - 1 whose results have landed meanwhile
+        float4_t d[4];
+        if (i < T) {
+            const int st = i / (SETS * 4), h = (i / 4) % SETS, b = i % 4;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const Frag16 B = sub_operand<BITS>(q[st][h][b], r);
+                d[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[h].h, B.h, (BITS == 8 || (r & 1)) ? biasH[h] : biasL[h], 0, 0, 0);
+            }
+        }
+        if (i > 0) {
+            const int st = (i - 1) / (SETS * 4), h = ((i - 1) / 4) % SETS, b = (i - 1) % 4;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const uint32_t sb = (r & 1) ? (sc[st][h][r >> 1] >> 16) : (sc[st][h][r >> 1] & 0xffffu);
+                const float sf = f16_bits_to_f32(sb);
+                if (BITS == 4 && (r & 1)) accH[st][b] = __builtin_fmaf(sf, dprev[r][r], accH[st][b]);
+                else accL[st][b] = __builtin_fmaf(sf, dprev[r][r], accL[st][b]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) dprev[r] = d[r];
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // blocks meet across lanes, waves through LDS (wave order), then the epilogue
+#pragma unroll
+    for (int st = 0; st < NS; st++) {
+        float tb[4];
+#pragma unroll
+        for (int b = 0; b < 4; b++) tb[b] = BITS == 4 ? accL[st][b] + accH[st][b] * 0.0625f : accL[st][b];
+        float t = blk == 0 ? tb[0] : (blk == 1 ? tb[1] : (blk == 2 ? tb[2] : tb[3]));
+        t += __shfl_xor(t, 16, 64);
+        t += __shfl_xor(t, 32, 64);
+        if (lane < 16) red[(st * 16 + wv) * 16 + lane] = t;
+    }
+    __syncthreads();
+    if (NS == 2) {               // SwiGLU: strips 2i / 2i+1 are gate / up of output strip i
+        if (tid < 16) {
+            float g = 0.f, u = 0.f;
+            for (int k = 0; k < nwaves; k++) {
+                g += red[k * 16 + tid];
+                u += red[(16 + k) * 16 + tid];
+            }
+            const int n = blockIdx.x * 16 + tid;
+            if (n < (w.N >> 1)) store_out1(y, ydt, n, silu_mul(g * 16777216.0f, u * 16777216.0f));
+        }
+        return;
+    }
+    if (tid < 16) {
+        float v = 0.f;
+        for (int k = 0; k < nwaves; k++) v += red[k * 16 + tid];
+        v *= 16777216.0f;
+        const int n = blockIdx.x * 16 + tid;
+        if (n < w.N) {
+            if (epi.kind == kEpiAdd) v += load_out1(epi.residual, ydt, n);
+            store_out1(y, ydt, n, v);
+        }
+    }
+}
+
+template <int BITS, int SETS, int NS>
+hipError_t launch1_e(const WeightView& w, const void* x, void* y, int ydt, int nwaves, bool even, const Epilogue& epi,
+                     hipStream_t st)
+{
+    const dim3 grid((unsigned)(w.NT / NS)), block((unsigned)nwaves * 64);
+    if (even)
+        hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, true>), grid, block, 0, st, w, reinterpret_cast<const _Float16*>(x), y, ydt,
+                           epi);
+    else
+        hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, false>), grid, block, 0, st, w, reinterpret_cast<const _Float16*>(x), y, ydt,
+                           epi);
+    return hipGetLastError();
+}
+
+template <int BITS, int NS>
+hipError_t launch1_s(const WeightView& w, const void* x, void* y, int ydt, const Epilogue& epi, hipStream_t st)
+{
+    // sets of four K tiles; a wave takes up to four of them, a workgroup has up to 16 waves
+    const int nsets = (w.KT + 3) / 4;
+    const int per_wave = (nsets + 15) / 16;
+    const int nwaves = (nsets + per_wave - 1) / per_wave;
+    const bool even = w.K % 512 == 0 && nsets % nwaves == 0;
+    switch (per_wave) {
+        case 1: return launch1_e<BITS, 1, NS>(w, x, y, ydt, nwaves, even, epi, st);
+        case 2: return launch1_e<BITS, 2, NS>(w, x, y, ydt, nwaves, even, epi, st);
+        case 3: return launch1_e<BITS, 3, NS>(w, x, y, ydt, nwaves, even, epi, st);
+        default: return launch1_e<BITS, 4, NS>(w, x, y, ydt, nwaves, even, epi, st);
+    }
+}
+
+}  // namespace
+
+bool gemv1_serves(const WeightView& w, int xdt, int M, const Epilogue& epi)
+{
+    return M == 1 && xdt == kF16 && !epi.gamma && w.KT <= 4 * 4 * 16;
+}
+
+hipError_t launch_gemv1(const WeightView& w, const void* x, void* y, int ydt, const Epilogue& epi, hipStream_t st)
+{
+    if (epi.kind == kEpiSwiglu) {
+        if (w.bits == 4) return launch1_s<4, 2>(w, x, y, ydt, epi, st);
+        return launch1_s<8, 2>(w, x, y, ydt, epi, st);
+    }
+    if (w.bits == 4) return launch1_s<4, 1>(w, x, y, ydt, epi, st);
+    return launch1_s<8, 1>(w, x, y, ydt, epi, st);
+}
+
+}  // namespace cybq

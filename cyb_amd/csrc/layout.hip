@@ -5,90 +5,111 @@
 
 namespace cybq {
 
-// signed weight and f16 scale bits from an interchange buffer ------------------
+namespace {
 
+// Bytes one scale group occupies in a row of the interchange buffer.
 template <int BITS, int LAYOUT>
-__device__ __forceinline__ int src_weight(const uint8_t* q, int64_t n, int64_t k, int64_t K)
+constexpr int kSrcGroupBytes = LAYOUT == 0 ? (BITS == 4 ? 16 : 32) : (BITS == 4 ? 18 : 34);
+
+// signed weight i (0..31) of group `gl` of a staged source row ---------------------
+template <int BITS, int LAYOUT>
+__device__ __forceinline__ int staged_weight(const uint8_t* row, int gl, int i)
 {
+    const uint8_t* g = row + gl * kSrcGroupBytes<BITS, LAYOUT>;
     if (LAYOUT == 0) {                               // PLANAR
-        if (BITS == 8) return (int)(int8_t)q[n * K + k];
-        uint8_t b = q[(n * K + k) >> 1];
-        int nib = (k & 1) ? (b >> 4) : (b & 15);
+        if (BITS == 8) return (int)(int8_t)g[i];
+        const uint8_t b = g[i >> 1];
+        const int nib = (i & 1) ? (b >> 4) : (b & 15);
         return (nib & 8) ? nib - 16 : nib;
-    } else {                                         // BLOCK_AOS
-        const int bs = BITS == 4 ? 18 : 34;
-        const uint8_t* blk = q + (n * (K / kGroup) + k / kGroup) * bs + 2;
-        int i = (int)(k % kGroup);
-        if (BITS == 8) return (int)(int8_t)blk[i];
-        uint8_t b = blk[i & 15];
-        return (int)((i < 16) ? (b & 15) : (b >> 4)) - 8;
     }
+    if (BITS == 8) return (int)(int8_t)g[2 + i];     // BLOCK_AOS: f16 d, then the weights
+    const uint8_t b = g[2 + (i & 15)];
+    return (int)((i < 16) ? (b & 15) : (b >> 4)) - 8;
 }
 
-template <int BITS, int LAYOUT>
-__device__ __forceinline__ uint16_t src_scale(const uint8_t* q, const uint16_t* scales,
-                                              int64_t n, int64_t g, int64_t K)
-{
-    if (LAYOUT == 0) return scales[n * (K / kGroup) + g];
-    const int bs = BITS == 4 ? 18 : 34;
-    const uint8_t* blk = q + (n * (K / kGroup) + g) * bs;
-    return (uint16_t)(blk[0] | (blk[1] << 8));
-}
+// One workgroup repacks CT consecutive K tiles of one 16-row strip.  The source rows of
+// that piece are first copied into LDS with coalesced loads (a row's piece is one
+// contiguous run in either interchange layout), then every thread assembles one lane's
+// share of a native tile from LDS and stores it with 128-bit stores: global memory only
+// sees whole runs, the byte-granular gathering stays inside the CU.
+constexpr int kRepackTiles = 4;
 
-// One thread per native 32-bit q word.
 template <int BITS, int LAYOUT>
-__global__ void repack_q_kernel(const uint8_t* __restrict__ q, uint32_t* __restrict__ dst,
-                                int N, int K, int NT, int KT)
+__global__ __launch_bounds__(256) void repack_kernel(const uint8_t* __restrict__ q, const uint16_t* __restrict__ scales,
+                                                      uint8_t* __restrict__ dst, int N, int K, int KT)
 {
-    const int words_per_tile = BITS == 4 ? 256 : 512;
-    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    int64_t total = (int64_t)NT * KT * words_per_tile;
-    if (idx >= total) return;
-    int64_t tile = idx / words_per_tile;
-    int r = (int)(idx % words_per_tile);
-    int nt = (int)(tile / KT), kt = (int)(tile % KT);
-    uint32_t out = 0;
+    constexpr int CT = kRepackTiles;
+    constexpr int GB = kSrcGroupBytes<BITS, LAYOUT>;
+    constexpr int ROWB = CT * kGroupsPerTile * GB;                  // bytes of one row's piece
+    constexpr int UNIT = LAYOUT == 0 ? 4 : 2;                       // load width the source alignment allows
+    constexpr int UPR = ROWB / UNIT;                                // units per row
+    __shared__ __attribute__((aligned(16))) uint8_t rows[kTileN][ROWB];
+
+    const int t = threadIdx.x;
+    const int chunks = (KT + CT - 1) / CT;
+    const int nt = (int)(blockIdx.x / (unsigned)chunks), kt0 = (int)(blockIdx.x % (unsigned)chunks) * CT;
+    const int G = K / kGroup;
+    const int g0 = kt0 * kGroupsPerTile;
+    const int ng = min(CT * kGroupsPerTile, G - g0);                // groups of this piece that exist
+    for (int i = t; i < kTileN * UPR; i += 256) {
+        const int r = i / UPR, u = i - r * UPR;
+        const int64_t n = (int64_t)nt * kTileN + r;
+        if (n < N && u * UNIT < ng * GB) {
+            const uint8_t* src = q + (n * G + g0) * GB + u * UNIT;
+            if (UNIT == 4) *reinterpret_cast<uint32_t*>(&rows[r][u * 4]) = *reinterpret_cast<const uint32_t*>(src);
+            else *reinterpret_cast<uint16_t*>(&rows[r][u * 2]) = *reinterpret_cast<const uint16_t*>(src);
+        }
+    }
+    __syncthreads();
+
+    const int b = t >> 6, lane = t & 63;
+    const int kt = kt0 + b;
+    if (kt >= KT) return;
+    const int row = lane & 15, oct = lane >> 4;
+    const bool row_ok = (int64_t)nt * kTileN + row < N;
+    uint8_t* tile = dst + ((int64_t)nt * KT + kt) * kTileBytes<BITS>;
     if (BITS == 4) {
-        int lane = r >> 2, j = r & 3;
-        int64_t n = (int64_t)nt * 16 + (lane & 15);
-        int64_t k0 = (int64_t)kt * 128 + j * 32 + (lane >> 4) * 8;
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
-            int v = 0;
-            if (n < N && k0 + s < K) v = src_weight<4, LAYOUT>(q, n, k0 + s, K);
-            out |= (uint32_t)((v + 8) & 15) << (4 * q4_nibble_pos(s));
+        for (int j = 0; j < 4; j++) {
+            const int gl = b * 4 + j;
+            const bool ok = row_ok && gl < ng;
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                const int v = ok ? staged_weight<4, LAYOUT>(rows[row], gl, oct * 8 + s) : 0;
+                w[q4_word(j, s)] |= (uint32_t)((v + 8) & 15) << q4_shift(j, s);
+            }
         }
+        reinterpret_cast<u32x4_t*>(tile)[lane] = (u32x4_t){w[0], w[1], w[2], w[3]};
     } else {
-        int h = r >> 8, lane = (r >> 2) & 63, wd = r & 3;     // half, lane, word in lane
-        int64_t n = (int64_t)nt * 16 + (lane & 15);
-        int j = 2 * h + (wd >> 1);
-        int64_t k0 = (int64_t)kt * 128 + j * 32 + (lane >> 4) * 8 + (wd & 1) * 4;
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
-            int v = 0;
-            if (n < N && k0 + s < K) v = src_weight<8, LAYOUT>(q, n, k0 + s, K);
-            out |= (uint32_t)((v + 128) & 255) << (8 * s);
+        for (int h = 0; h < 2; h++) {
+            uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int wd = 0; wd < 4; wd++) {
+                const int gl = b * 4 + 2 * h + (wd >> 1);
+                const bool ok = row_ok && gl < ng;
+#pragma unroll
+                for (int s = 0; s < 4; s++) {
+                    const int v = ok ? staged_weight<8, LAYOUT>(rows[row], gl, oct * 8 + (wd & 1) * 4 + s) : 0;
+                    w[wd] |= (uint32_t)((v + 128) & 255) << (8 * s);
+                }
+            }
+            reinterpret_cast<u32x4_t*>(tile)[h * 64 + lane] = (u32x4_t){w[0], w[1], w[2], w[3]};
         }
     }
-    dst[idx] = out;
-}
-
-// One thread per native scale.
-template <int BITS, int LAYOUT>
-__global__ void repack_s_kernel(const uint8_t* __restrict__ q, const uint16_t* __restrict__ scales,
-                                uint16_t* __restrict__ dst, int N, int K, int NT, int KT)
-{
-    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    int64_t total = (int64_t)NT * KT * 64;
-    if (idx >= total) return;
-    int64_t tile = idx >> 6;
-    int r = (int)(idx & 63);
-    int nt = (int)(tile / KT), kt = (int)(tile % KT);
-    int64_t n = (int64_t)nt * 16 + (r >> 2);
-    int64_t g = (int64_t)kt * 4 + (r & 3);
-    uint16_t v = 0;
-    if (n < N && g * kGroup < K) v = src_scale<BITS, LAYOUT>(q, scales, n, g, K);
-    dst[idx] = v;
+    // the tile's 64 scales: [row][group]
+    {
+        const int r = lane >> 2, j = lane & 3;
+        const int gl = b * 4 + j;
+        const int64_t n = (int64_t)nt * kTileN + r;
+        uint16_t v = 0;
+        if (n < N && gl < ng) {
+            if (LAYOUT == 0) v = scales[n * G + g0 + gl];
+            else v = (uint16_t)(rows[r][gl * GB] | (rows[r][gl * GB + 1] << 8));
+        }
+        reinterpret_cast<uint16_t*>(tile + kTileQBytes<BITS>)[lane] = v;
+    }
 }
 
 // native -> f32 [N,K].  One thread per 8 consecutive k of one row.
@@ -104,15 +125,17 @@ __global__ void dequant_kernel(WeightView w, float* __restrict__ out)
     int kt = (int)(k0 >> 7), j = (int)((k0 >> 5) & 3), oct = (int)((k0 >> 3) & 3);
     int lane = oct * 16 + row;
     int64_t tile = (int64_t)nt * w.KT + kt;
-    float d = f16_bits_to_f32(w.s[tile * 64 + row * 4 + j]);
+    const uint16_t* sp = reinterpret_cast<const uint16_t*>(tile_s<BITS>(w, tile));
+    float d = f16_bits_to_f32(sp[row * 4 + j]);
     float v[8];
     if (BITS == 4) {
-        uint32_t word = w.q[(tile * 64 + lane) * 4 + j];
+        const u32x4_t lw = tile_q<4>(w, tile)[lane];
+        const uint32_t words[4] = {lw[0], lw[1], lw[2], lw[3]};
 #pragma unroll
-        for (int s = 0; s < 8; s++) v[s] = d * (float)q4_slot_value(word, s);
+        for (int s = 0; s < 8; s++) v[s] = d * (float)q4_slot_value(words, j, s);
     } else {
-        const uint32_t* p = w.q + tile * 512 + (j >> 1) * 256 + lane * 4 + (j & 1) * 2;
-        uint32_t w0 = p[0], w1 = p[1];
+        const u32x4_t lw = tile_q<8>(w, tile)[(j >> 1) * 64 + lane];
+        uint32_t w0 = lw[(j & 1) * 2], w1 = lw[(j & 1) * 2 + 1];
 #pragma unroll
         for (int s = 0; s < 8; s++) v[s] = d * (float)q8_slot_value(w0, w1, s);
     }
@@ -122,26 +145,24 @@ __global__ void dequant_kernel(WeightView w, float* __restrict__ out)
 }
 
 template <int BITS, int LAYOUT>
-static hipError_t launch_repack_t(const void* q, const void* scales, uint32_t* qdst, uint16_t* sdst,
-                                  int N, int K, int NT, int KT, hipStream_t st)
+hipError_t launch_repack_t(const void* q, const void* scales, uint8_t* dst, int N, int K, int NT, int KT, hipStream_t st)
 {
-    const int threads = 256;
-    int64_t qwords = (int64_t)NT * KT * (BITS == 4 ? 256 : 512);
-    int64_t swords = (int64_t)NT * KT * 64;
-    hipLaunchKernelGGL((repack_q_kernel<BITS, LAYOUT>), dim3((unsigned)((qwords + threads - 1) / threads)),
-                       dim3(threads), 0, st, (const uint8_t*)q, qdst, N, K, NT, KT);
-    hipLaunchKernelGGL((repack_s_kernel<BITS, LAYOUT>), dim3((unsigned)((swords + threads - 1) / threads)),
-                       dim3(threads), 0, st, (const uint8_t*)q, (const uint16_t*)scales, sdst, N, K, NT, KT);
+    const int64_t groups = (int64_t)((KT + kRepackTiles - 1) / kRepackTiles) * NT;
+    if (groups > 0x7fffffff) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((repack_kernel<BITS, LAYOUT>), dim3((unsigned)groups), dim3(256), 0, st, (const uint8_t*)q, (const uint16_t*)scales, dst, N, K,
+                       KT);
     return hipGetLastError();
 }
 
-hipError_t launch_repack(int bits, int layout, const void* q, const void* scales, uint32_t* qdst,
-                         uint16_t* sdst, int N, int K, int NT, int KT, hipStream_t st)
+}  // namespace
+
+hipError_t launch_repack(int bits, int layout, const void* q, const void* scales, uint8_t* dst, int N, int K, int NT, int KT,
+                         hipStream_t st)
 {
-    if (bits == 4 && layout == 0) return launch_repack_t<4, 0>(q, scales, qdst, sdst, N, K, NT, KT, st);
-    if (bits == 4 && layout == 1) return launch_repack_t<4, 1>(q, scales, qdst, sdst, N, K, NT, KT, st);
-    if (bits == 8 && layout == 0) return launch_repack_t<8, 0>(q, scales, qdst, sdst, N, K, NT, KT, st);
-    if (bits == 8 && layout == 1) return launch_repack_t<8, 1>(q, scales, qdst, sdst, N, K, NT, KT, st);
+    if (bits == 4 && layout == 0) return launch_repack_t<4, 0>(q, scales, dst, N, K, NT, KT, st);
+    if (bits == 4 && layout == 1) return launch_repack_t<4, 1>(q, scales, dst, N, K, NT, KT, st);
+    if (bits == 8 && layout == 0) return launch_repack_t<8, 0>(q, scales, dst, N, K, NT, KT, st);
+    if (bits == 8 && layout == 1) return launch_repack_t<8, 1>(q, scales, dst, N, K, NT, KT, st);
     return hipErrorInvalidValue;
 }
 
