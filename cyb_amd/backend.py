@@ -83,6 +83,7 @@ def load_library() -> ctypes.CDLL:
     lib.cybq_weight_fuse_pairs.argtypes = [vp, vp, vp, ctypes.POINTER(vp)]
     lib.cybq_matmul_many_ex.argtypes = [vp, i64, vp, vp, vp, vp, vp, ci, i64, ci, vp]
     lib.cybq_set_prefill_mode.argtypes = [vp, ci]
+    lib.cybq_set_decode_mode.argtypes = [vp, ci]
     lib.cybq_matmul_many.argtypes = [vp, i64, vp, vp, vp, ci, i64, ci, vp]
     lib.cybq_dequant.argtypes = [vp, vp, vp, vp]
     lib.cybq_quantize.argtypes = [vp, ci, vp, i64, i64, vp, vp, vp]
@@ -337,6 +338,14 @@ class Backend:
         if mode not in codes:
             raise CybqError(-1, "invalid argument", f"prefill mode {mode!r}")
         self._check(self._lib.cybq_set_prefill_mode(self._ctx, codes[mode]))
+
+    def set_decode_mode(self, mode: str) -> None:
+        """'stream' (default): one f16 row multiplies subnormal weight operands straight from memory;
+        'exact': exact integer weight operands."""
+        codes = {"stream": 0, "exact": 1}
+        if mode not in codes:
+            raise CybqError(-1, "invalid argument", f"decode mode {mode!r}")
+        self._check(self._lib.cybq_set_decode_mode(self._ctx, codes[mode]))
 
     def set_gemv_tuning(self, waves: int = 0, rows_kernel: int = 0, unroll: int = 0) -> None:
         """Diagnostics: waves per workgroup; decode kernel choice (0 auto, 1 always the

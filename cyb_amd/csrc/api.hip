@@ -15,6 +15,7 @@ struct cybq_ctx {
     int device = 0;
     int num_cus = 0;
     bool prefill_exact = false;
+    bool decode_exact = false;
     void* workspace = nullptr;          // scratch for the prefill path, allocated once at init
     size_t workspace_bytes = 0;
     std::string last_error;
@@ -321,7 +322,7 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
     cybq::WeightView v = view_of(w);
     hipError_t e;
     if (M <= 16) {
-        e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, epi, st);
+        e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->decode_exact, epi, st);
     } else if (xdt == CYBQ_F32 ? !ctx->prefill_exact : M > 32) {
         e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, ctx->workspace, ctx->workspace_bytes,
                               epi, st);
@@ -340,7 +341,7 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
             const size_t yoff = (size_t)m0 * n_out * dtype_size(ydt);
             cybq::Epilogue ec = epi;
             if (epi.kind == cybq::kEpiAdd) ec.residual = static_cast<const char*>(residual) + yoff;
-            e = cybq::launch_gemv(v, xp, xdt, mm, static_cast<char*>(y) + yoff, ydt, ctx->num_cus, ec, st);
+            e = cybq::launch_gemv(v, xp, xdt, mm, static_cast<char*>(y) + yoff, ydt, ctx->num_cus, ctx->decode_exact, ec, st);
         }
     }
     if (e != hipSuccess) return fail_hip(ctx, e, "matmul launch");
@@ -403,6 +404,14 @@ int cybq_set_prefill_mode(cybq_ctx* ctx, cybq_prefill_mode mode)
     if (!ctx) return CYBQ_ERR_INVALID;
     if (mode != CYBQ_PREFILL_FAST && mode != CYBQ_PREFILL_EXACT) return fail(ctx, CYBQ_ERR_INVALID, "unknown prefill mode");
     ctx->prefill_exact = mode == CYBQ_PREFILL_EXACT;
+    return CYBQ_OK;
+}
+
+int cybq_set_decode_mode(cybq_ctx* ctx, cybq_decode_mode mode)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (mode != CYBQ_DECODE_STREAM && mode != CYBQ_DECODE_EXACT) return fail(ctx, CYBQ_ERR_INVALID, "unknown decode mode");
+    ctx->decode_exact = mode == CYBQ_DECODE_EXACT;
     return CYBQ_OK;
 }
 

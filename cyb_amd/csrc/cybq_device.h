@@ -16,7 +16,7 @@
 //     nibble), and (w & 0x000F000F), ((w >> 8) & 0x000F000F) are the slots (0,1),
 //     (2,3) of the even group as two 16-bit integers each - which, read as IEEE f16,
 //     are the subnormals u * 2^-24 - while the mask 0x00F000F0 yields the odd
-//     group as 16u * 2^-24.  One shift and four ANDs turn a word into operands.
+//     group as 16u * 2^-24.  A shift or two and four ANDs turn a word into operands.
 //   Q8 q part  : 2 halves x 64 lanes x 16 B (2048 B).  Half h, lane l
 //     holds groups 4*kt + 2*h and 4*kt + 2*h + 1, 8 bytes each, byte s =
 //     q + 128 for k = 32*g + 8*(l >> 4) + s.
@@ -95,20 +95,29 @@ __device__ __forceinline__ void unpack_q4_f16(uint32_t wa, uint32_t wb, int t, u
     }
 }
 
-// The same group as f16 subnormals: u * 2^-24 (t = 0) or 16u * 2^-24 (t = 1), u = q + 8.
+// The same group as f16 subnormals: 4u * 2^-24 (t = 0) or 64u * 2^-24 (t = 1), u = q + 8.
 // The matrix cores of gfx950 take f16 subnormals at face value, so these ARE operands; a
 // caller takes the bias off with one more MFMA of its activations against the constant
-// operand kSubBiasL / kSubBiasH (-8 * 2^-24, -128 * 2^-24) and folds 2^24 (and the 16 of
-// an odd group) into the scale.
-constexpr uint32_t kSubBiasL = 0x80088008u, kSubBiasH = 0x80808080u;
+// operand kSubBiasL / kSubBiasH (-32 * 2^-24, -512 * 2^-24) and folds 2^22 (and the 16 of
+// an odd group) into the scale.  Two shifts and four ANDs per word.  (The nibbles are moved
+// two bits up the mantissa on the way: the matrix pipe aligns the 32 products of an
+// instruction by their operands' exponent fields and drops what falls below its adder,
+// always downwards, so every leading zero of a subnormal operand costs a bit of the sum -
+// with the nibbles where memory has them, u * 2^-24 and 16u * 2^-24, that showed as a common
+// offset of 2e-6 .. 3e-5 of the result's size, growing with K; two bits up it is 3e-7.)
+constexpr uint32_t kSubBiasL = 0x80208020u, kSubBiasH = 0x82008200u;
+constexpr float kSubUnscale = 4194304.0f;          // 2^22
 __device__ __forceinline__ void unpack_q4_sub(uint32_t wa, uint32_t wb, int t, uint32_t out[4])
 {
-    const uint32_t m = t ? 0x00F000F0u : 0x000F000Fu;
-    out[0] = wa & m;
-    out[1] = (wa >> 8) & m;
-    out[2] = wb & m;
-    out[3] = (wb >> 8) & m;
+    const uint32_t m = t ? 0x03C003C0u : 0x003C003Cu;
+    out[0] = (wa << 2) & m;
+    out[1] = (wa >> 6) & m;
+    out[2] = (wb << 2) & m;
+    out[3] = (wb >> 6) & m;
 }
+// Q8: bytes u = q + 128 as subnormals u * 2^-24 (one byte permute per pair), bias -128 * 2^-24
+constexpr uint32_t kSubBiasQ8 = 0x80808080u;
+constexpr float kSubUnscaleQ8 = 16777216.0f;       // 2^24
 
 // The bf16 counterpart: 0x4300 | u is the bf16 number 128 + u (7 mantissa bits, so
 // only a nibble in the low bits fits: every pair is shifted down first).  There is no

@@ -19,8 +19,14 @@ hipError_t launch_repack(int bits, int layout, const void* q, const void* scales
 hipError_t launch_dequant(const WeightView& w, float* out, hipStream_t st);
 
 // decode path, 1 <= M <= 16 per call (api.hip walks 17..32 rows as two calls)
+// exact_operands: keep the weight operands exact integers for one f16 row too (the LDS kernel)
+// instead of the subnormal-operand kernel of gemv1.hip
 hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
-                       int num_cus, const Epilogue& epi, hipStream_t st);
+                       int num_cus, bool exact_operands, const Epilogue& epi, hipStream_t st);
+// one-row decode kernel (f16 activations, no folded norm): weight operands are f16 subnormals,
+// the +8 / +128 bias comes off inside the MFMA accumulation (gemv1.hip)
+bool gemv1_serves(const WeightView& w, int xdt, int M, const Epilogue& epi);
+hipError_t launch_gemv1(const WeightView& w, const void* x, void* y, int ydt, const Epilogue& epi, hipStream_t st);
 // prefill path (api.hip sends 16-bit activations with M > 32 here)
 // exact: two MFMAs per group with losslessly split weights; otherwise one f16 MFMA
 // per group with weights rounded once to f16
@@ -50,5 +56,6 @@ inline hipError_t raise_lds_limit_once(const void* kernel, int bytes, unsigned l
 
 // test/bench hook: overrides the decode kernel's launch heuristics (0 = automatic)
 void set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll);
+
 
 }  // namespace cybq

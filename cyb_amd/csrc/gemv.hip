@@ -845,7 +845,8 @@ hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int y
 
 int g_tune_waves = 0, g_tune_unroll = 0, g_tune_rows = 0;
 
-constexpr int kLdsBudget = 64 * 1024;
+constexpr int kLdsBudget = 64 * 1024;      // what a slab of x aims for
+constexpr int kLdsCap = 150 * 1024;         // what a launch may ask for
 
 template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT, int PAIR, bool NORM>
 hipError_t launch_p(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
@@ -869,9 +870,12 @@ hipError_t launch_p(const WeightView& w, const void* x, int M, void* y, int ydt,
     // x, then the waves' partial sums, then 16 row sums of squares and their 16 x 16 per-wave parts (folded RMSNorm)
     const size_t lds = xbytes + (size_t)PAIR * nwaves * RMAX * 64 * sizeof(float) + (16 + 256) * sizeof(float);
     auto kern = gemv_kernel<BITS, XMODE, RMAX, U, ONESHOT, PAIR, NORM>;
-    // M = 16 fp32 activations with 8 waves need 66 KB, just over the default cap
+    // A slab is at least one tile per wave, whatever the budget says: 16 rows of fp32 activations
+    // (two 16-bit planes) on 16 waves stage 16 x 2056 x 4 B = 129 KB, plus 16 KB of partial sums
+    // and the norm's row sums - the largest request there is, 146 KB.
     static unsigned long long lds_raised = 0;
-    if (hipError_t e = raise_lds_limit_once(reinterpret_cast<const void*>(kern), 96 * 1024, lds_raised); e != hipSuccess) return e;
+    if (hipError_t e = raise_lds_limit_once(reinterpret_cast<const void*>(kern), kLdsCap, lds_raised); e != hipSuccess) return e;
+    if (lds > (size_t)kLdsCap) return hipErrorInvalidValue;
     hipLaunchKernelGGL(kern, dim3(w.NT / PAIR), dim3(nwaves * PAIR * 64), lds, st, w, x, M, y, ydt, slab_tiles, ldx, (int)xbytes,
                        epi);
     return hipGetLastError();
@@ -922,7 +926,7 @@ void set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll)
 }
 
 hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
-                       int num_cus, const Epilogue& epi, hipStream_t st)
+                       int num_cus, bool exact_operands, const Epilogue& epi, hipStream_t st)
 {
     // Waves per workgroup (= split of a strip's K tiles).  Depends on the weight
     // shape only, never on M, so that the summation order is the same for every
@@ -930,6 +934,10 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
     // more if that is what it takes to bring a wave's share down to 8 tiles, all requested
     // up front.  (K = 4096 is 4 waves x 8 tiles for every N: with few strips 8 waves x 4 tiles
     // measured 2 - 4 % slower.)
+    // one f16 row: the kernel of gemv1.hip (unless the caller asked for exact integer weight
+    // operands, or a test forces one of the kernels below)
+    if (!exact_operands && g_tune_waves == 0 && g_tune_rows == 0 && g_tune_unroll == 0 && gemv1_serves(w, xdt, M, epi))
+        return launch_gemv1(w, x, y, ydt, epi, st);
     int nwaves = g_tune_waves;
     if (nwaves <= 0) {
         nwaves = 2;
@@ -955,7 +963,10 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
     // 27.6 us at 4096 -> 28672)
     const bool wide_q8 = w.bits == 8 && (w.NT + num_cus / 2) / num_cus >= 3;
     const bool rows_kernel = g_tune_rows == 1 || (g_tune_rows == 0 && M >= (wide_q8 ? 5 : 3));
-    if (rows_kernel && xdt != kF32) {
+    // (a folded norm keeps gamma as fp32 in LDS next to the exchange areas: beyond K = 23552 that no
+    // longer fits and the LDS kernel, which stages x in slabs, takes the call)
+    const bool gamma_fits = !epi.gamma || w.K <= 23552;
+    if (rows_kernel && xdt != kF32 && gamma_fits) {
         if (w.bits == 4) {
             if (xdt == kF16) return launch_rows<4, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
             return launch_rows<4, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);

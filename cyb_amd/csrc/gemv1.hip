@@ -14,15 +14,15 @@
 //    ignored).  Output row g = 4*b + r lives in register r of lane block b (lanes 16b..16b+15):
 //    lane block b ends up with tile b of the set, register r with scale group r - exactly
 //    the four scales a lane gets from one 8-byte load of the tile's scale record.
-//  * Weight operands cost one shift and four ANDs per eight weights: the native nibble
-//    order makes (w & 0x000F000F) two f16 subnormals u * 2^-24 (u = q + 8), which the matrix
-//    cores take at face value.  The bias comes off inside the same accumulation: the MFMA's C
-//    operand is x times the constant -8 * 2^-24 (one extra MFMA per set, its row g is exactly
-//    -8 * sum of group g's activations).  Odd groups sit in the high nibbles (16u * 2^-24,
-//    constant -128 * 2^-24); the 16 and the 2^24 are folded into the final scaling.
+//  * Weight operands cost two shifts and four ANDs per eight weights: the native nibble
+//    order makes ((w << 2) & 0x003C003C) two f16 subnormals 4u * 2^-24 (u = q + 8), which the
+//    matrix cores take at face value.  The bias comes off inside the same accumulation: the
+//    MFMA's C operand is x times the constant -32 * 2^-24 (one extra MFMA per set, its row g is
+//    exactly -8 * 4 * sum of group g's activations).  Odd groups sit in the high nibbles (64u *
+//    2^-24, constant -512 * 2^-24); the 16 and the 2^22 are folded into the final scaling.
 //    Q8 bytes u = q + 128 become subnormals with one byte permute per pair.
 //  * Per-group f16 scales are applied in fp32 on the MFMA results; lanes add up what their
-//    block owns, blocks meet through two cross-lane moves, waves through LDS in wave order:
+//    block owns, blocks meet through a 16x16x4 fp32 MFMA against ones, waves through LDS:
 //    the order of all additions is fixed, results are reproducible.
 #include "cybq_device.h"
 #include "cybq_internal.h"
@@ -65,8 +65,8 @@ __device__ __forceinline__ Frag16 sub_operand(const u32x4_t (&q)[BITS == 4 ? 1 :
 
 // SETS: sets a wave owns (set index wv + nwaves * h).  NS: strips per workgroup (2 = a gate strip
 // and its up strip, SwiGLU epilogue).  EVEN: K is a multiple of 512 and every wave has SETS
-// whole sets, so nothing needs clamping.
-template <int BITS, int SETS, int NS, bool EVEN>
+// whole sets, so nothing needs clamping.  NW: waves per workgroup when known at compile time (0 = any).
+template <int BITS, int SETS, int NS, bool EVEN, int NW>
 __global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float16* __restrict__ x, void* __restrict__ y, int ydt,
                                                      Epilogue epi)
 {
@@ -74,7 +74,7 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float1
     __shared__ float red[NS * 16 * 16];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nwaves = (int)blockDim.x >> 6;
+    const int nwaves = NW ? NW : (int)blockDim.x >> 6;          // NW = 0: whatever the launch says
     const int row = lane & 15, blk = lane >> 4;
     const int KT = w.KT;
 
@@ -93,25 +93,46 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float1
             tile_ok[h] = 4 * set + blk < KT;
         }
     }
+    // Addresses: one wave-uniform 64-bit base per (strip, set) plus a 32-bit lane offset, so the
+    // requests go out after a handful of scalar instructions.
+    constexpr int TB = kTileBytes<BITS>, QB = kTileQBytes<BITS>;
+    const uint32_t lane_q = (uint32_t)lane * 16u;
+    const uint32_t lane_s = (uint32_t)QB + (uint32_t)row * 8u;
 #pragma unroll
     for (int st = 0; st < NS; st++) {
-        const int64_t strip = (int64_t)(blockIdx.x * NS + st) * KT;
+        const int strip_tile = ((int)blockIdx.x * NS + st) * KT;           // tile indices fit 32 bits
 #pragma unroll
         for (int h = 0; h < SETS; h++) {
             const int t0 = 4 * (wv + nwaves * h);
-            sc[st][h] = __builtin_nontemporal_load(tile_s<BITS>(w, strip + (EVEN ? t0 + blk : min(t0 + blk, KT - 1))) + row);
-        }
+            if (EVEN) {
+                const uint8_t* sb = w.base + (int64_t)(strip_tile + t0) * TB;
+                sc[st][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(sb + ((uint32_t)blk * TB + lane_s)));
 #pragma unroll
-        for (int h = 0; h < SETS; h++) {
-            const int t0 = 4 * (wv + nwaves * h);
+                for (int b = 0; b < 4; b++)
 #pragma unroll
-            for (int b = 0; b < 4; b++) {
-                const u32x4_t* qp = tile_q<BITS>(w, strip + (EVEN ? t0 + b : min(t0 + b, KT - 1)));
+                    for (int v = 0; v < QV; v++)
+                        q[st][h][b][v] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(sb + (b * TB + v * 1024) + lane_q));
+            } else {
+                const uint8_t* strip = w.base + (int64_t)strip_tile * TB;
+                sc[st][h] = __builtin_nontemporal_load(
+                    reinterpret_cast<const u32x2_t*>(strip + ((uint32_t)min(t0 + blk, KT - 1) * TB + lane_s)));
 #pragma unroll
-                for (int v = 0; v < QV; v++) q[st][h][b][v] = __builtin_nontemporal_load(qp + v * 64 + lane);
+                for (int b = 0; b < 4; b++) {
+                    const uint8_t* tp = strip + (int64_t)min(t0 + b, KT - 1) * TB;
+#pragma unroll
+                    for (int v = 0; v < QV; v++)
+                        q[st][h][b][v] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(tp + v * 1024 + lane_q));
+                }
             }
         }
     }
+    // Everything the tail needs from the kernel arguments is fetched now, next to the requests:
+    // left to itself the compiler loads each argument where it is first used, i.e. after the
+    // final barrier, and the kernel would end with two more round trips to memory.
+    const int n_rows = w.N, out_dt = ydt, epi_kind = epi.kind;
+    const void* const residual = epi.residual;
+    asm volatile("" ::"s"(n_rows), "s"(out_dt), "s"(epi_kind), "s"(residual), "s"(y));
+    if (!NW) asm volatile("" ::"s"(nwaves));
     __builtin_amdgcn_sched_barrier(0);       // every request is out before any arithmetic
 
     if (!EVEN) {
@@ -131,8 +152,10 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float1
     }
 
     Frag16 kL, kH;
+    constexpr uint32_t cH = BITS == 4 ? kSubBiasH : kSubBiasQ8;
+    constexpr float unscale = BITS == 4 ? kSubUnscale : kSubUnscaleQ8;
     kL.u = (u32x4_t){kSubBiasL, kSubBiasL, kSubBiasL, kSubBiasL};
-    kH.u = (u32x4_t){kSubBiasH, kSubBiasH, kSubBiasH, kSubBiasH};
+    kH.u = (u32x4_t){cH, cH, cH, cH};
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
     float4_t biasL[SETS], biasH[SETS];
 #pragma unroll
@@ -179,39 +202,44 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float1
         __builtin_amdgcn_sched_barrier(0);
     }
 
-    // blocks meet across lanes, waves through LDS (wave order), then the epilogue
+    // Blocks meet inside the matrix pipe: with B[k = block][n] = the block's sum and A = ones, a
+    // 16x16x4 fp32 MFMA leaves sum_k B[k][n] in every row - one instruction instead of two
+    // cross-lane round trips.  Waves meet through LDS; the last sum is the same trick again: lane
+    // block j adds the partial sums of waves 4i + j in order of i, the MFMA adds the four blocks.
+    const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int st = 0; st < NS; st++) {
         float tb[4];
 #pragma unroll
         for (int b = 0; b < 4; b++) tb[b] = BITS == 4 ? accL[st][b] + accH[st][b] * 0.0625f : accL[st][b];
-        float t = blk == 0 ? tb[0] : (blk == 1 ? tb[1] : (blk == 2 ? tb[2] : tb[3]));
-        t += __shfl_xor(t, 16, 64);
-        t += __shfl_xor(t, 32, 64);
-        if (lane < 16) red[(st * 16 + wv) * 16 + lane] = t;
+        const float t = blk == 0 ? tb[0] : (blk == 1 ? tb[1] : (blk == 2 ? tb[2] : tb[3]));
+        const float4_t sum = __builtin_amdgcn_mfma_f32_16x16x4f32(1.0f, t, zero4, 0, 0, 0);
+        if (lane < 16) red[(st * 16 + wv) * 16 + lane] = sum[0];
     }
     __syncthreads();
+    if (tid >= 64) return;
+    constexpr int SLOTS = NW ? (NW + 3) / 4 : 4;
+    float outv[NS];
+#pragma unroll
+    for (int st = 0; st < NS; st++) {
+        float t[SLOTS];
+#pragma unroll
+        for (int i = 0; i < SLOTS; i++) t[i] = red[(st * 16 + min(4 * i + blk, 15)) * 16 + row];
+        float v = 0.f;
+#pragma unroll
+        for (int i = 0; i < SLOTS; i++) v += 4 * i + blk < nwaves ? t[i] : 0.f;
+        outv[st] = __builtin_amdgcn_mfma_f32_16x16x4f32(1.0f, v, zero4, 0, 0, 0)[0] * unscale;
+    }
+    if (lane >= 16) return;
+    const int n = blockIdx.x * 16 + lane;
     if (NS == 2) {               // SwiGLU: strips 2i / 2i+1 are gate / up of output strip i
-        if (tid < 16) {
-            float g = 0.f, u = 0.f;
-            for (int k = 0; k < nwaves; k++) {
-                g += red[k * 16 + tid];
-                u += red[(16 + k) * 16 + tid];
-            }
-            const int n = blockIdx.x * 16 + tid;
-            if (n < (w.N >> 1)) store_out1(y, ydt, n, silu_mul(g * 16777216.0f, u * 16777216.0f));
-        }
+        if (n < (n_rows >> 1)) store_out1(y, out_dt, n, silu_mul(outv[0], outv[NS - 1]));
         return;
     }
-    if (tid < 16) {
-        float v = 0.f;
-        for (int k = 0; k < nwaves; k++) v += red[k * 16 + tid];
-        v *= 16777216.0f;
-        const int n = blockIdx.x * 16 + tid;
-        if (n < w.N) {
-            if (epi.kind == kEpiAdd) v += load_out1(epi.residual, ydt, n);
-            store_out1(y, ydt, n, v);
-        }
+    if (n < n_rows) {
+        float v = outv[0];
+        if (epi_kind == kEpiAdd) v += load_out1(residual, out_dt, n);
+        store_out1(y, out_dt, n, v);
     }
 }
 
@@ -220,36 +248,48 @@ hipError_t launch1_e(const WeightView& w, const void* x, void* y, int ydt, int n
                      hipStream_t st)
 {
     const dim3 grid((unsigned)(w.NT / NS)), block((unsigned)nwaves * 64);
-    if (even)
-        hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, true>), grid, block, 0, st, w, reinterpret_cast<const _Float16*>(x), y, ydt,
+    if (even && nwaves == 8 && SETS == 1)          // K = 4096: the shape most decode launches have
+        hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, true, SETS == 1 ? 8 : 0>), grid, block, 0, st, w,
+                           reinterpret_cast<const _Float16*>(x), y, ydt, epi);
+    else if (even)
+        hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, true, 0>), grid, block, 0, st, w, reinterpret_cast<const _Float16*>(x), y, ydt,
                            epi);
     else
-        hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, false>), grid, block, 0, st, w, reinterpret_cast<const _Float16*>(x), y, ydt,
+        hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, false, 0>), grid, block, 0, st, w, reinterpret_cast<const _Float16*>(x), y, ydt,
                            epi);
     return hipGetLastError();
 }
 
+// sets of four K tiles a wave may own (all of them in registers, 16 waves per workgroup at
+// most: 128 registers per lane): two, three for Q4 with one strip per workgroup, one for
+// Q8 gate / up pairs
+constexpr int max_sets_per_wave(int bits, int ns) { return bits == 4 ? (ns == 1 ? 3 : 2) : (ns == 1 ? 2 : 1); }
+
 template <int BITS, int NS>
 hipError_t launch1_s(const WeightView& w, const void* x, void* y, int ydt, const Epilogue& epi, hipStream_t st)
 {
-    // sets of four K tiles; a wave takes up to four of them, a workgroup has up to 16 waves
     const int nsets = (w.KT + 3) / 4;
     const int per_wave = (nsets + 15) / 16;
     const int nwaves = (nsets + per_wave - 1) / per_wave;
     const bool even = w.K % 512 == 0 && nsets % nwaves == 0;
-    switch (per_wave) {
-        case 1: return launch1_e<BITS, 1, NS>(w, x, y, ydt, nwaves, even, epi, st);
-        case 2: return launch1_e<BITS, 2, NS>(w, x, y, ydt, nwaves, even, epi, st);
-        case 3: return launch1_e<BITS, 3, NS>(w, x, y, ydt, nwaves, even, epi, st);
-        default: return launch1_e<BITS, 4, NS>(w, x, y, ydt, nwaves, even, epi, st);
+    constexpr int MAXS = max_sets_per_wave(BITS, NS);
+    if (per_wave == 1) return launch1_e<BITS, 1, NS>(w, x, y, ydt, nwaves, even, epi, st);
+    if constexpr (MAXS >= 2) {
+        if (per_wave == 2) return launch1_e<BITS, 2, NS>(w, x, y, ydt, nwaves, even, epi, st);
     }
+    if constexpr (MAXS >= 3) {
+        if (per_wave == 3) return launch1_e<BITS, 3, NS>(w, x, y, ydt, nwaves, even, epi, st);
+    }
+    return hipErrorInvalidValue;         // gemv1_serves() said no
 }
 
 }  // namespace
 
 bool gemv1_serves(const WeightView& w, int xdt, int M, const Epilogue& epi)
 {
-    return M == 1 && xdt == kF16 && !epi.gamma && w.KT <= 4 * 4 * 16;
+    if (M != 1 || xdt != kF16 || epi.gamma) return false;
+    const int nsets = (w.KT + 3) / 4;
+    return (nsets + 15) / 16 <= max_sets_per_wave(w.bits, epi.kind == kEpiSwiglu ? 2 : 1);
 }
 
 hipError_t launch_gemv1(const WeightView& w, const void* x, void* y, int ydt, const Epilogue& epi, hipStream_t st)

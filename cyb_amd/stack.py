@@ -59,12 +59,12 @@ def fused_shapes(shapes: Dict[str, tuple] = None) -> Dict[str, tuple]:
             "down_proj": shapes["down_proj"]}
 
 
-def build(backend: Backend, layers: int = 32, bits: int = formats.Q4, seed: int = 5, keep_planar: int = 0,
+def build(backend: Backend, layers: int = 32, bits: int = formats.Q4, seed: int = 5, keep_planar=0,
           shapes: Dict[str, tuple] = None, order: List[str] = None, epilogues: bool = False) -> LinearStack:
     """Random-init stack with N(0, 0.02) weights quantised on the device.
 
-    keep_planar: for the first that many layers, the PLANAR device buffers are kept in
-    `stack.planar` so that a checker can pull them back and recompute outputs.
+    keep_planar: for the first that many layers (or for the layers listed), the PLANAR device
+    buffers are kept in `stack.planar` so that a checker can pull them back and recompute outputs.
     epilogues: with the fused shapes, `gate_up_proj` becomes a strip-interleaved pair run with the
     SwiGLU epilogue (its output has half the columns) and `o_proj` / `down_proj` add a residual."""
     import torch
@@ -73,6 +73,7 @@ def build(backend: Backend, layers: int = 32, bits: int = formats.Q4, seed: int 
     gen = torch.Generator(device="cuda")
     gen.manual_seed((synth.BASE_SEED ^ seed) & 0x7FFFFFFF)
     order = order or [l for l in LINEAR_ORDER if l in shapes] or list(shapes)
+    kept = set(range(keep_planar)) if isinstance(keep_planar, int) else set(keep_planar)
     for layer in range(layers):
         for lin in order:
             K, N = shapes[lin]
@@ -102,7 +103,7 @@ def build(backend: Backend, layers: int = 32, bits: int = formats.Q4, seed: int 
             st.nodes.append(QMatMul(w=name, x=f"in.{K}", y=f"out.{lin}", quant=bits, M=1, N=N, K=K))
             if epilogues:
                 st.epilogues.append(epi)
-            if layer < keep_planar:
+            if layer in kept:
                 st.planar[name] = (qd, sd)
             del w
     return st

@@ -85,6 +85,15 @@ typedef enum cybq_dtype { CYBQ_F32 = 0, CYBQ_F16 = 1, CYBQ_BF16 = 2 } cybq_dtype
  *          the fp32 CPU path only by accumulation order.  Half the throughput. */
 typedef enum cybq_prefill_mode { CYBQ_PREFILL_FAST = 0, CYBQ_PREFILL_EXACT = 1 } cybq_prefill_mode;
 
+/* How the one-row decode kernel (M = 1, f16 activations) forms its weight operands.  Both
+ * accumulate in fp32 and stay far inside the 1e-3 tolerance.
+ *   STREAM (default) the packed nibbles / bytes are used as f16 subnormals (q + bias) * 2^-24
+ *          straight from memory and the bias is removed inside the same fp32 accumulation;
+ *          about 3e-6 relative L2 (the sums carry the bias until it cancels), the quickest form.
+ *   EXACT  the weight operand is the exact integer q (more unpack arithmetic per byte);
+ *          about 1e-7 relative L2, and a tensor of zeros gives exact zeros. */
+typedef enum cybq_decode_mode { CYBQ_DECODE_STREAM = 0, CYBQ_DECODE_EXACT = 1 } cybq_decode_mode;
+
 /* ---- context ---------------------------------------------------------- */
 
 /* Replaces: backend construction when the runtime is spawned
@@ -136,6 +145,9 @@ int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype x
  * `--backend honeycrisp|wgpu|cpu`, shell/src/worlds/models/mod.rs:113-115); here
  * it selects the numeric mode of the prefill kernel for this context. */
 int cybq_set_prefill_mode(cybq_ctx* ctx, cybq_prefill_mode mode);
+
+/* Same knob for the decode kernel (see cybq_decode_mode). */
+int cybq_set_decode_mode(cybq_ctx* ctx, cybq_decode_mode mode);
 
 /* Replaces: the executor's walk over the quantised-matmul nodes of one decode
  * step (7 linears per layer x layers + LM head - decide/pipeline.md:51): `count`

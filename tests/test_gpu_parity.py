@@ -218,6 +218,72 @@ def test_decode_batched_rows_equal_single_rows_bitwise(backend, oracle):
     assert torch.equal(_run(backend, qw, x), y16)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("shape", [(64, 128), (48, 160), (100, 4096 + 96), (4096, 4096), (256, 14336), (64, 11008),
+                                   (32, 16384), (16, 24576), (16, 32768)])
+def test_one_row_kernel_shapes(backend, oracle, bits, shape):
+    """One f16 row (subnormal weight operands, bias removed inside the accumulation): whole and
+    ragged sets of K tiles, one to three sets per wave, and K beyond what it serves."""
+    N, K = shape
+    q, s = _quant(oracle, bits, N, K)
+    qw = backend.upload_quantized(q, s, bits, formats.BLOCK_AOS if N % 32 else formats.PLANAR)
+    x = _x(1, K, "f16", outliers=0.001)
+    y = _run(backend, qw, x)
+    assert oracle.rel_l2(y.cpu().numpy(), oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT
+    assert torch.equal(_run(backend, qw, x), y)                 # reproducible
+    for ydt in ("f16", "bf16"):
+        assert torch.equal(_run(backend, qw, x, ydt), y.to(TDT[ydt]))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_decode_modes(backend, oracle, bits):
+    """STREAM (default) and EXACT weight operands for one f16 row: both inside the tight bar;
+    EXACT returns exact zeros for a tensor of zeros."""
+    N, K = 320, 4096
+    q, s = _quant(oracle, bits, N, K)
+    qw = backend.upload_quantized(q, s, bits)
+    qz = backend.upload_quantized(np.zeros((N, K), np.int8), s, bits)
+    x = _x(1, K, "f16")
+    ref = oracle.matmul_f64(q, s, x.float().cpu().numpy())
+    scale = float(np.abs(ref).mean())
+    try:
+        errs = {}
+        for mode in ("stream", "exact"):
+            backend.set_decode_mode(mode)
+            errs[mode] = oracle.rel_l2(_run(backend, qw, x).cpu().numpy(), ref)
+            assert errs[mode] < TIGHT, (mode, errs)
+            z = _run(backend, qz, x).cpu().numpy()
+            if mode == "exact":
+                assert not z.any()
+            else:
+                assert np.abs(z).max() < 1e-4 * scale       # the bias cancels to rounding, not to the bit
+        assert errs["exact"] < 1e-6
+    finally:
+        backend.set_decode_mode("stream")
+    with pytest.raises(CybqError):
+        backend.set_decode_mode("loose")
+
+
+def test_decode_lds_kernel_largest_request(backend, oracle):
+    """fp32 activations, 10..16 rows, K long enough for 16 waves: the slab of x is one tile per
+    wave whatever the budget says (up to 146 KB of LDS); and exact-mode fp32 prefill walks it."""
+    K = 14336
+    for N in (64, 4096):
+        q, s = _quant(oracle, 4, N, K)
+        qw = backend.upload_quantized(q, s, 4)
+        for M in (12, 16):
+            x = _x(M, K, "f32")
+            y = _run(backend, qw, x).cpu().numpy()
+            assert oracle.rel_l2(y, oracle.matmul_f64(q, s, x.cpu().numpy())) < TIGHT, (N, M)
+    backend.set_prefill_mode("exact")
+    try:
+        x = _x(40, K, "f32")
+        y = _run(backend, qw, x).cpu().numpy()
+        assert oracle.rel_l2(y, oracle.matmul_f64(q, s, x.cpu().numpy())) < TIGHT
+    finally:
+        backend.set_prefill_mode("fast")
+
+
 def test_decode_special_cases(backend, oracle):
     N, K = 64, 256
     ones = np.full((N, K // 32), 0x3C00, np.uint16)
@@ -385,7 +451,7 @@ def test_prefill_more_rows_than_the_stage_holds(backend, oracle, prefill_mode):
     assert oracle.rel_l2(y[rows].cpu().numpy(), ref) < _bar(prefill_mode)
 
 
-@pytest.mark.parametrize("M", [128, 512])
+@pytest.mark.parametrize("M", [128, 512, 2048])
 @pytest.mark.parametrize("shape", [(4096, 14336), (14336, 4096)])
 def test_config4_full_size(backend, oracle, prefill_mode, M, shape):
     K, N = shape
@@ -786,6 +852,80 @@ def test_decode_stack_with_epilogues(backend, oracle):
             got = edges[node.y].cpu().numpy()
             assert got.shape == ref.shape
             assert oracle.rel_l2(got, ref) < bar, (M, node.w, epi)
+    for w in st.weights:
+        w.free()
+
+
+def _node_reference(oracle, st, node, epi, edges, rows=None):
+    """float64 oracle output of one stack node from the PLANAR buffers the stack kept."""
+    qd, sd = st.planar[node.w]
+    q = formats.unpack_planar(qd.cpu().numpy(), 4, node.N, node.K)
+    s = sd.cpu().numpy().view(np.uint16).reshape(node.N, node.K // 32)
+    x = edges[node.x] if rows is None else edges[node.x][rows]
+    ref = oracle.matmul_f64(q, s, x.float().cpu().numpy())
+    if epi == "add":
+        r = edges[f"res.{node.N}"] if rows is None else edges[f"res.{node.N}"][rows]
+        ref = ref + r.double().cpu().numpy()
+    elif epi == "swiglu":
+        h = node.N // 2
+        ref = _silu_mul(ref[:, :h], ref[:, h:])
+    return ref
+
+
+@pytest.mark.timeout(900)
+@pytest.mark.parametrize("form", ["per_linear", "fused", "fused_epilogues"])
+def test_config5_full_size_stack(backend, oracle, form):
+    """The 32-layer Llama-3-8B-shaped decode step through cybq_matmul_many at full size, batch 1 and 8:
+    every node of the first, a middle and the last layer against the oracle; for the fused forms also
+    one 512-token bf16 prefill chunk through the same node list."""
+    from cyb_amd import stack
+    shapes = None if form == "per_linear" else stack.fused_shapes()
+    checked = (0, 15, 31)
+    st = stack.build(backend, layers=32, seed=5, keep_planar=checked, shapes=shapes,
+                     order=list(shapes) if shapes else None, epilogues=form == "fused_epilogues")
+    per_layer = len(st.nodes) // 32
+    assert per_layer == (7 if shapes is None else 4)
+    epis = st.epilogues or ["none"] * len(st.nodes)
+    mine = [i for i in range(len(st.nodes)) if i // per_layer in checked]
+    for M in (1, 8, 512) if shapes is not None else (1, 8):
+        edges = stack.edges_for(st, M, shapes=shapes, xdtype=torch.bfloat16 if M > 16 else None)
+        xs, ys = [edges[n.x] for n in st.nodes], [edges[n.y] for n in st.nodes]
+        for i in mine:                                  # the checked nodes write buffers of their own
+            ys[i] = torch.full_like(ys[i], float("nan"))
+        res = None
+        if st.epilogues:
+            res = [edges[f"res.{n.N}"] if e == "add" else None for n, e in zip(st.nodes, st.epilogues)]
+        pl = backend.plan_many(st.weights, xs, ys, st.epilogues or None, res)
+        backend.matmul_many(pl, M)
+        torch.cuda.synchronize()
+        for i in mine:
+            node, epi = st.nodes[i], epis[i]
+            if M <= 16:
+                ref = _node_reference(oracle, st, node, epi, edges)
+                assert oracle.rel_l2(ys[i].cpu().numpy(), ref) < TIGHT, (M, node.w, epi)
+            else:
+                rows = [0, M // 2, M - 1]
+                ref = _node_reference(oracle, st, node, epi, edges, rows)
+                assert oracle.rel_l2(ys[i][rows].cpu().numpy(), ref) < 2 * FAST, (M, node.w, epi)
+                assert torch.isfinite(ys[i]).all()
+        if M > 16:
+            # every row of the widest and of the longest-K node of the last layer: float64 matmul on the
+            # oracle's dequantised weights
+            for i in mine[-per_layer:]:
+                node, epi = st.nodes[i], epis[i]
+                if epi == "swiglu" or node.N * node.K < 4096 * 14336:
+                    continue
+                qd, sd = st.planar[node.w]
+                q = formats.unpack_planar(qd.cpu().numpy(), 4, node.N, node.K)
+                s = sd.cpu().numpy().view(np.uint16).reshape(node.N, node.K // 32)
+                wd = torch.from_numpy(oracle.dequant(q, s)).cuda().double()
+                full = edges[node.x].double() @ wd.T
+                if epi == "add":
+                    full = full + edges[f"res.{node.N}"].double()
+                err = ((ys[i].double() - full).norm() / full.norm()).item()
+                assert err < 2 * FAST, (M, node.w, err)
+                del wd, full
+    assert st.weight_bytes == 32 * 122_683_392
     for w in st.weights:
         w.free()
 
