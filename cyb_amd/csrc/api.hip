@@ -7,6 +7,7 @@
 #include <cstring>
 #include <new>
 #include <string>
+#include <vector>
 
 #include "../../include/cybq.h"
 #include "cybq_internal.h"
@@ -30,6 +31,33 @@ struct cybq_weight {
     size_t bytes = 0;
     bool paired = false;                // made by cybq_weight_fuse_pairs: strips alternate gate / up
 };
+
+namespace cybq {
+
+namespace {
+struct LdsEntry {
+    const void* kernel;
+    int bytes;
+};
+std::vector<LdsEntry>& lds_requests()
+{
+    static std::vector<LdsEntry> list;        // built on first use: registrations come from static initialisers
+    return list;
+}
+}  // namespace
+
+void register_lds_request(const void* kernel, int bytes) { lds_requests().push_back({kernel, bytes}); }
+
+hipError_t raise_all_lds_limits()
+{
+    for (const LdsEntry& r : lds_requests()) {
+        hipError_t e = hipFuncSetAttribute(r.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, r.bytes);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+}  // namespace cybq
 
 namespace {
 
@@ -138,6 +166,10 @@ int cybq_init(int device, cybq_ctx** out)
     if (e != hipSuccess) { (void)hipGetLastError(); return CYBQ_ERR_NO_DEVICE; }
     if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) return CYBQ_ERR_NO_DEVICE;
     e = hipSetDevice(device);
+    if (e != hipSuccess) { (void)hipGetLastError(); return CYBQ_ERR_HIP; }
+    // every kernel that wants more than the default dynamic LDS gets its limit raised now, for
+    // this device: launches never touch function attributes
+    e = cybq::raise_all_lds_limits();
     if (e != hipSuccess) { (void)hipGetLastError(); return CYBQ_ERR_HIP; }
     cybq_ctx* ctx = new (std::nothrow) cybq_ctx();
     if (!ctx) return CYBQ_ERR_NOMEM;
@@ -287,7 +319,7 @@ int cybq_weight_info(const cybq_weight* w, int* quant, int64_t* N, int64_t* K, i
 namespace {
 int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M, const void* gamma,
                  cybq_dtype gdt, float eps, void* y, cybq_dtype ydt, cybq_epilogue epilogue, const void* residual,
-                 void* stream)
+                 void* stream, void* workspace, size_t workspace_bytes)
 {
     if (!ctx) return CYBQ_ERR_INVALID;
     if (!w || !x || !y) return fail(ctx, CYBQ_ERR_INVALID, "w / x / y is NULL");
@@ -324,7 +356,7 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
     if (M <= 16) {
         e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->decode_exact, epi, st);
     } else if (xdt == CYBQ_F32 ? !ctx->prefill_exact : M > 32) {
-        e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, ctx->workspace, ctx->workspace_bytes,
+        e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, workspace, workspace_bytes,
                               epi, st);
     } else {
         // fp32 activations keep full precision through the decode kernel's hi/lo split:
@@ -352,7 +384,8 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
 int cybq_matmul_ex(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M, void* y,
                    cybq_dtype ydt, cybq_epilogue epilogue, const void* residual, void* stream)
 {
-    return matmul_fused(ctx, w, x, xdt, M, nullptr, CYBQ_F32, 0.f, y, ydt, epilogue, residual, stream);
+    return matmul_fused(ctx, w, x, xdt, M, nullptr, CYBQ_F32, 0.f, y, ydt, epilogue, residual, stream, ctx ? ctx->workspace : nullptr,
+                        ctx ? ctx->workspace_bytes : 0);
 }
 
 int cybq_matmul_norm(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M, const void* gamma,
@@ -361,7 +394,7 @@ int cybq_matmul_norm(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dt
 {
     if (!ctx) return CYBQ_ERR_INVALID;
     if (!gamma) return fail(ctx, CYBQ_ERR_INVALID, "gamma is NULL");
-    return matmul_fused(ctx, w, x, xdt, M, gamma, gdt, eps, y, ydt, epilogue, residual, stream);
+    return matmul_fused(ctx, w, x, xdt, M, gamma, gdt, eps, y, ydt, epilogue, residual, stream, ctx->workspace, ctx->workspace_bytes);
 }
 
 int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M, void* y,

@@ -39,20 +39,17 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
 hipError_t launch_quantize(int bits, const float* src, int N, int K, void* q_out, void* s_out,
                            hipStream_t st);
 
-// Raises a kernel's dynamic LDS limit, once per kernel and device: `done` is the caller's
-// static bit mask of devices already served (the attribute belongs to the kernel as loaded on
-// one device; a process may drive several).
-inline hipError_t raise_lds_limit_once(const void* kernel, int bytes, unsigned long long& done)
-{
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    const unsigned long long bit = 1ull << (dev & 63);
-    if (done & bit) return hipSuccess;
-    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (e == hipSuccess) done |= bit;
-    return e;
-}
+// Kernels that need more dynamic LDS than the default 64 KB say so when the library is loaded:
+// naming LdsRequest<&kernel, bytes>::registered anywhere in a launcher puts the pair on a list
+// (a static initialiser, run before any call).  cybq_init walks the list for its device, so
+// no launch ever changes a function attribute: first calls behave like all others and may sit
+// inside a stream capture.
+void register_lds_request(const void* kernel, int bytes);
+hipError_t raise_all_lds_limits();              // for the current device
+template <auto Kernel, int Bytes>
+struct LdsRequest {
+    static inline const bool registered = (register_lds_request(reinterpret_cast<const void*>(Kernel), Bytes), true);
+};
 
 // test/bench hook: overrides the decode kernel's launch heuristics (0 = automatic)
 void set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll);

@@ -485,10 +485,9 @@ hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt,
                     size_t part_bytes, int num_cus, const Epilogue& epi, const NormStats& ns, hipStream_t st)
 {
     constexpr int BM = WAVES * MF * 16;
-    const size_t lds = (size_t)2 * NF * (4 * (EXACT ? 2 : 1) * 64) * 16;     // operand buffers, 56 .. 128 KB
+    constexpr int lds = 2 * NF * (4 * (EXACT ? 2 : 1) * 64) * 16;     // operand buffers, 56 .. 128 KB
     auto kern = gemm_kernel<BITS, XBF, NF, EXACT, MF, WAVES>;
-    static unsigned long long lds_raised = 0;
-    if (hipError_t e = raise_lds_limit_once(reinterpret_cast<const void*>(kern), (int)lds, lds_raised); e != hipSuccess) return e;
+    (void)LdsRequest<&gemm_kernel<BITS, XBF, NF, EXACT, MF, WAVES>, lds>::registered;
     const int n_tiles = (w.NT + NF - 1) / NF, m_tiles = (M + BM - 1) / BM;
     // Too few tiles to fill the chip: split K over workgroups.  Every split adds its
     // K range in fp32 into its own slab of `part`; a second kernel adds the slabs in

@@ -783,9 +783,8 @@ hipError_t launch_rows_x(const WeightView& w, const void* x, int M, void* y, int
     if (epi.gamma) {
         lds += (size_t)w.K * sizeof(float);            // gamma as fp32
         auto kern = gemv_rows_kernel<BITS, XMODE, TS, NS, true, XR>;
-        static unsigned long long lds_raised = 0;
-        if (hipError_t e = raise_lds_limit_once(reinterpret_cast<const void*>(kern), 150 * 1024, lds_raised); e != hipSuccess) return e;
-        if (lds > 150 * 1024) return hipErrorInvalidValue;      // K beyond ~30 k with a folded norm
+        (void)LdsRequest<&gemv_rows_kernel<BITS, XMODE, TS, NS, true, XR>, 150 * 1024>::registered;
+        if (lds > 150 * 1024) return hipErrorInvalidValue;      // (launch_gemv keeps such K away from this kernel)
         hipLaunchKernelGGL(kern, dim3(groups), dim3(nwaves * 64), lds, st, w, reinterpret_cast<const uint16_t*>(x), M, y, ydt,
                            epi);
     } else
@@ -873,8 +872,7 @@ hipError_t launch_p(const WeightView& w, const void* x, int M, void* y, int ydt,
     // A slab is at least one tile per wave, whatever the budget says: 16 rows of fp32 activations
     // (two 16-bit planes) on 16 waves stage 16 x 2056 x 4 B = 129 KB, plus 16 KB of partial sums
     // and the norm's row sums - the largest request there is, 146 KB.
-    static unsigned long long lds_raised = 0;
-    if (hipError_t e = raise_lds_limit_once(reinterpret_cast<const void*>(kern), kLdsCap, lds_raised); e != hipSuccess) return e;
+    (void)LdsRequest<&gemv_kernel<BITS, XMODE, RMAX, U, ONESHOT, PAIR, NORM>, kLdsCap>::registered;
     if (lds > (size_t)kLdsCap) return hipErrorInvalidValue;
     hipLaunchKernelGGL(kern, dim3(w.NT / PAIR), dim3(nwaves * PAIR * 64), lds, st, w, x, M, y, ydt, slab_tiles, ldx, (int)xbytes,
                        epi);
