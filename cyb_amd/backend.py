@@ -78,6 +78,7 @@ def load_library() -> ctypes.CDLL:
     lib.cybq_weight_info.argtypes = [vp, ctypes.POINTER(ci), ctypes.POINTER(i64), ctypes.POINTER(i64),
                                      ctypes.POINTER(i64)]
     lib.cybq_matmul.argtypes = [vp, vp, vp, ci, i64, vp, ci, vp]
+    lib.cybq_matmul_static.argtypes = [vp, vp, vp, ci, i64, vp, ci, vp]
     lib.cybq_matmul_ex.argtypes = [vp, vp, vp, ci, i64, vp, ci, ci, vp, vp]
     lib.cybq_matmul_norm.argtypes = [vp, vp, vp, ci, i64, vp, ci, ctypes.c_float, vp, ci, ci, vp, vp]
     lib.cybq_weight_fuse_pairs.argtypes = [vp, vp, vp, ctypes.POINTER(vp)]
@@ -267,6 +268,13 @@ class Backend:
             M = int(x.shape[0]) if x.dim() == 2 else 1
         self._check(self._lib.cybq_matmul(self._ctx, w.handle, _ptr(x), _dtype_code(x, xdt), M, _ptr(y),
                                           _dtype_code(y, ydt), stream))
+
+    def matmul_static(self, w: QWeight, x, y, M: Optional[int] = None, stream: int = 0) -> None:
+        """cybq_matmul_static: the same op with its scratch in a static device array (allocates nothing)."""
+        if M is None:
+            M = int(x.shape[0]) if x.dim() == 2 else 1
+        self._check(self._lib.cybq_matmul_static(self._ctx, w.handle, _ptr(x), _dtype_code(x, None), M, _ptr(y),
+                                                 _dtype_code(y, None), stream))
 
     def matmul_ex(self, w: QWeight, x, y, epilogue: str = "none", residual=None, M: Optional[int] = None,
                   stream: int = 0) -> None:

@@ -61,6 +61,17 @@ hipError_t raise_all_lds_limits()
 
 namespace {
 
+// Scratch of cybq_matmul_static, the entry point that allocates nothing: the prefill path's
+// staging area and K-split slabs live in this array instead of a hipMalloc'ed workspace.
+// Every device the library runs on holds its own copy at its own address until the process
+// ends; the name below is only the host-side handle of the symbol, never a device address:
+// cybq_init asks the runtime for the address on its device and kernels receive that pointer.
+constexpr size_t kStaticScratchBytes = (size_t)64 << 20;
+constexpr int64_t kStaticMaxK = 32768;          // 256 staged rows of 2-byte activations fit half the scratch with room to spare
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+void* g_scratch_ptr[kMaxDevices] = {};
+
 int fail(cybq_ctx* ctx, int code, const char* what)
 {
     if (ctx) ctx->last_error = what ? what : "";
@@ -171,6 +182,12 @@ int cybq_init(int device, cybq_ctx** out)
     // this device: launches never touch function attributes
     e = cybq::raise_all_lds_limits();
     if (e != hipSuccess) { (void)hipGetLastError(); return CYBQ_ERR_HIP; }
+    if (device < kMaxDevices && !g_scratch_ptr[device]) {       // this device's copy of the static scratch
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) { (void)hipGetLastError(); return CYBQ_ERR_HIP; }
+        g_scratch_ptr[device] = p;
+    }
     cybq_ctx* ctx = new (std::nothrow) cybq_ctx();
     if (!ctx) return CYBQ_ERR_NOMEM;
     ctx->device = device;
@@ -401,6 +418,18 @@ int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype x
                 cybq_dtype ydt, void* stream)
 {
     return cybq_matmul_ex(ctx, w, x, xdt, M, y, ydt, CYBQ_EPI_NONE, nullptr, stream);
+}
+
+int cybq_matmul_static(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt, int64_t M, void* y,
+                       cybq_dtype ydt, void* stream)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (ctx->device >= kMaxDevices || !g_scratch_ptr[ctx->device])
+        return fail(ctx, CYBQ_ERR_UNSUPPORTED, "no static scratch on this device");
+    if (w && M > 16 && w->K > kStaticMaxK)
+        return fail(ctx, CYBQ_ERR_UNSUPPORTED, "cybq_matmul_static: K beyond 32768 does not fit the static scratch for more than 16 rows");
+    return matmul_fused(ctx, w, x, xdt, M, nullptr, CYBQ_F32, 0.f, y, ydt, CYBQ_EPI_NONE, nullptr, stream,
+                        g_scratch_ptr[ctx->device], kStaticScratchBytes);
 }
 
 int cybq_weight_fuse_pairs(cybq_ctx* ctx, const cybq_weight* gate, const cybq_weight* up, cybq_weight** out)

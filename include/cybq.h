@@ -141,6 +141,17 @@ int cybq_weight_info(const cybq_weight* w, int* quant, int64_t* N, int64_t* K,
 int cybq_matmul(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt,
                 int64_t M, void* y, cybq_dtype ydt, void* stream);
 
+/* cybq_matmul for callers that cannot allocate or cannot let a callee allocate: code under
+ * stream capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
+ * reference.  Same arguments, same results to within summation order; the prefill path's
+ * scratch (staged activations, partial sums of a K split) is a 64 MiB array inside the
+ * library's code object, one copy per device, instead of the context's allocated workspace,
+ * and the call makes no hipMalloc / hipFree and no call that allocates.  Limits: for M > 16,
+ * K <= 32768 (CYBQ_ERR_UNSUPPORTED beyond).  All calls on one device share that array, whatever
+ * context or stream they use: calls that overlap in time on one device race. */
+int cybq_matmul_static(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype xdt,
+                       int64_t M, void* y, cybq_dtype ydt, void* stream);
+
 /* Replaces: a backend configuration knob (the reference picks a backend per run:
  * `--backend honeycrisp|wgpu|cpu`, shell/src/worlds/models/mod.rs:113-115); here
  * it selects the numeric mode of the prefill kernel for this context. */
