@@ -9,6 +9,11 @@ distinct device copies of the weight tensor (more bytes than the 256 MB
 last-level cache), so every step streams its weights from HBM.  Inputs are
 resident in HBM before the timed region starts.
 
+A timed pass is exactly `--steps` back-to-back launches between two HIP events on the
+launch stream; passes are repeated (the walk over the weight copies simply continues)
+until at least 50 ms of device time have been measured, and the per-step mean over all
+passes is reported, so the figure does not depend on how small `--steps` is.
+
 Prints ONE JSON line on stdout; progress goes to stderr.
 """
 from __future__ import annotations
@@ -24,54 +29,74 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
-MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / f16, published
 MALL_BYTES = 256 << 20
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain
-# 256 MiB copy: FETCH x 1.9997, WRITE x 1.0000); profiles/decode_gemv_q4_4096x14336_m1.md
+MIN_TIMED_S = 0.050
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the
+# same counter reads for a plain 256 MiB copy; profiles/decode_gemv_q4_4096x14336_m1.md and
+# profiles/prefill_gemm_q4_4096x14336_m512.md
 TRAFFIC_DECODE_BYTES = 33_270_500
-TRAFFIC_PREFILL_M512_BYTES = 121_950_000     # multiply 113.5 MB + activation staging pass 8.4 MB
+TRAFFIC_PREFILL_M512_BYTES = 121_950_000
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def timed_many(be, plan, M, stream, torch):
-    a = torch.cuda.Event(enable_timing=True)
-    b = torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    a.record()
-    be.matmul_many(plan, M, stream)
-    b.record()
-    torch.cuda.synchronize()
-    return a.elapsed_time(b) * 1e-3      # seconds
+class Timer:
+    """HIP events on the launch stream around a callable that only enqueues work."""
+
+    def __init__(self, torch):
+        self.torch = torch
+
+    def once(self, fn):
+        t = self.torch
+        a, b = t.cuda.Event(enable_timing=True), t.cuda.Event(enable_timing=True)
+        t.cuda.synchronize()
+        a.record()
+        fn()
+        b.record()
+        t.cuda.synchronize()
+        return a.elapsed_time(b) * 1e-3      # seconds
+
+    def until(self, make_pass, min_s=MIN_TIMED_S, max_passes=400):
+        """make_pass(i) enqueues pass i; returns (mean seconds per pass, per-pass list)."""
+        times = []
+        while sum(times) < min_s and len(times) < max_passes:
+            i = len(times)
+            times.append(self.once(lambda: make_pass(i)))
+        return sum(times) / len(times), times
 
 
 def cpu_baseline(q, s, x32, alg_bytes, budget_s=12.0):
-    """The CPU restatement (oracle, row-parallel fp32) timed on the host cores."""
+    """The optimised CPU restatement (oracle/cybq_cpu_baseline.c: packed Q4_0 blocks, SIMD, all host
+    cores), checked against the float64 oracle, then timed on a bounded sample."""
     import numpy as np
+    from cyb_amd import formats
     from tests.oracle_lib import Oracle
     ora = Oracle()
     try:
         cores = len(os.sched_getaffinity(0))
     except AttributeError:
         cores = os.cpu_count() or 1
-    threads = max(1, min(16, cores))
-    copies = [(q, s)] + [(q.copy(), s.copy()) for _ in range(3)]   # > L3 of any one CCD
-    ora.matmul_mt(q, s, x32, threads)                               # warm-up, page-in
+    N, K = q.shape
+    blocks = np.ascontiguousarray(formats.pack_blocks(q, s, formats.Q4)).view(np.uint8).reshape(-1)
+    y, used = ora.cpu_baseline_q4_0(blocks, N, K, x32, cores)
+    err = ora.rel_l2(y, ora.matmul_f64(q, s, x32))
+    if not err < 1e-5:
+        raise RuntimeError(f"cpu baseline disagrees with the oracle: rel_l2 = {err}")
+    copies = [blocks] + [blocks.copy() for _ in range(31)]          # 1.06 GB of blocks: more than the L3 of the whole socket
+    out = np.empty_like(y)
     reps, t0 = 0, time.perf_counter()
     while True:
-        qq, ss = copies[reps % len(copies)]
-        ora.matmul_mt(qq, ss, x32, threads)
+        ora.cpu_baseline_q4_0(copies[reps % len(copies)], N, K, x32, cores, out)
         reps += 1
         el = time.perf_counter() - t0
-        if el >= budget_s or reps >= 4000:
+        if el >= budget_s or reps >= 200000:
             break
-    # the same restatement on one thread (fixed summation order), a few passes
     r1, t1 = 0, time.perf_counter()
-    while r1 < 40 and time.perf_counter() - t1 < 3.0:
-        qq, ss = copies[r1 % len(copies)]
-        ora.matmul_f32(qq, ss, x32)
+    while r1 < 200 and time.perf_counter() - t1 < 3.0:
+        ora.cpu_baseline_q4_0(copies[r1 % len(copies)], N, K, x32, 1, out)
         r1 += 1
     el1 = time.perf_counter() - t1
     model = ""
@@ -80,13 +105,14 @@ def cpu_baseline(q, s, x32, alg_bytes, budget_s=12.0):
             model = next((l.split(":", 1)[1].strip() for l in f if l.startswith("model name")), "")
     except OSError:
         pass
-    return {"value": round(alg_bytes * reps / el / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": f"{reps} passes of the same 4096->14336 Q4 batch-1 matmul over {len(copies)} weight copies, "
-                      f"{el:.1f} s, C restatement (fp32, per-group scale, rows split over {threads} threads)",
+    return {"value": round(alg_bytes * reps / el / 1e9, 3), "unit": "GB/s", "cores": used, "kind": "port",
+            "sample": f"{reps} passes of the same 4096->14336 Q4 batch-1 matmul over {len(copies)} copies of the packed "
+                      f"Q4_0 blocks, {el:.1f} s; C restatement with {ora.cpu_baseline_isa()} intrinsics, fp32 accumulate, "
+                      f"rows split over {used} threads; rel_l2 vs the float64 oracle {err:.1e}",
             "us_per_pass": round(el / reps * 1e6, 1),
             "one_thread": {"value": round(alg_bytes * r1 / el1 / 1e9, 3), "unit": "GB/s", "us_per_pass": round(el1 / r1 * 1e6, 1),
                            "passes": r1},
-            "host": {"cpus_available": cores, "cpu_model": model}}
+            "host": {"cpus_available": cores, "cpu_model": model, "isa": ora.cpu_baseline_isa()}}
 
 
 def main():
@@ -95,7 +121,7 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--no-extra", action="store_true", help="skip the prefill / sweep extras")
+    ap.add_argument("--no-extra", action="store_true", help="skip the prefill / sweep / stack extras")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="no timing: a plain 256 MiB device copy (calibration), then the decode and prefill "
                          "kernels, for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
@@ -115,6 +141,7 @@ def main():
     dev = torch.device("cuda:0")
     be = Backend(0)                      # raises if libcybq.so is missing
     stream = torch.cuda.current_stream().cuda_stream
+    timer = Timer(torch)
 
     K, N, M, bits = 4096, 14336, 1, formats.Q4
     t0 = time.time()
@@ -143,8 +170,10 @@ def main():
         print(f"parity failed: rel_l2 = {rel_l2}", file=sys.stderr)
         sys.exit(1)
 
-    def plan_of(n):
-        return be.plan_many([ws[i % copies] for i in range(n)], [x] * n, [ys[i % 2] for i in range(n)])
+    def plan_of(n, first=0, weights=None, xs=None, youts=None):
+        wl = weights or ws
+        return be.plan_many([wl[(first + i) % len(wl)] for i in range(n)], [xs if xs is not None else x] * n,
+                            [(youts or ys)[i % len(youts or ys)] for i in range(n)])
 
     if args.traffic_probe:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
@@ -160,29 +189,69 @@ def main():
         log("traffic probe done")
         return
 
+    # Every timed walk starts on the copy after the last one touched and simply goes on around the ring:
+    # a launch always meets the copy that was used longest ago (24 launches = 793 MB earlier).
+    cursor = [0]
+    plans = {}
+
+    def walk(n, run):
+        key = (n, cursor[0])
+        if key not in plans:                    # built once, outside any timed region (see prepare)
+            plans[key] = plan_of(n, cursor[0])
+        run(plans[key])
+        cursor[0] = (cursor[0] + n) % copies
+
+    def prepare(n):
+        """Builds the plans the next walks of n steps will need (a walk's start only depends on n mod copies)."""
+        c = cursor[0]
+        for _ in range(copies):
+            if (n, c) not in plans:
+                plans[(n, c)] = plan_of(n, c)
+            c = (c + n) % copies
+
+    # everything still cached from the set-up (clones, parity) is pushed out first
+    flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    flush.fill_(1)
+    torch.cuda.synchronize()
+    del flush
     if args.warmup > 0:
-        be.matmul_many(plan_of(args.warmup), M, stream)
-    plan = plan_of(args.steps)
-    el = timed_many(be, plan, M, stream, torch)
-    us = el / args.steps * 1e6
-    gbs = alg_bytes / (el / args.steps) / 1e9
-    log(f"decode GEMV: {us:.2f} us/launch, {gbs:.0f} GB/s")
+        walk(args.warmup, lambda p: be.matmul_many(p, M, stream))
+    prepare(args.steps)
+    mean_pass, passes = timer.until(lambda i: walk(args.steps, lambda p: be.matmul_many(p, M, stream)))
+    us = mean_pass / args.steps * 1e6
+    gbs = alg_bytes / (mean_pass / args.steps) / 1e9
+    log(f"decode GEMV: {us:.2f} us/launch, {gbs:.0f} GB/s ({len(passes)} passes of {args.steps} steps)")
+
+    # ---- ceilings on this box, same footprint, same walk over the copies --------------------------
+    ceil_n = 1000
+    ceilings = {}
+    walk(200, lambda p: be.matmul_many(p, M, stream))
+    prepare(ceil_n)
+    for label, io in (("bare_read_of_the_weight_bytes", False), ("read_plus_x_load_and_y_store", True)):
+        walk(200, lambda p: be.debug_read_weights(p, io, x, ys[0], stream))
+        t, _ = timer.until(lambda i: walk(ceil_n, lambda p: be.debug_read_weights(p, io, x, ys[0], stream)))
+        cus = t / ceil_n * 1e6
+        ceilings[label] = {"us": round(cus, 3), "GB/s": round((alg_bytes if io else alg_w) / (t / ceil_n) / 1e9, 1),
+                           "frac_of_hbm_peak": round((alg_bytes if io else alg_w) / (t / ceil_n) / 1e9 / HBM_PEAK_GBS, 4)}
+        log(f"ceiling {label}: {cus:.2f} us")
+    ceilings["what"] = ("the one-row kernel's own memory requests (one workgroup per 16-row strip, whole strip requested "
+                        "up front) with no arithmetic; second line adds its activation read and its 57 KB of stores")
+    ceilings["kernel_over_bare_read"] = round(us / ceilings["bare_read_of_the_weight_bytes"]["us"], 4)
+    ceilings["kernel_over_read_with_io"] = round(us / ceilings["read_plus_x_load_and_y_store"]["us"], 4)
+    # the same launches with exact integer weight operands (cybq_set_decode_mode EXACT)
+    be.set_decode_mode("exact")
+    walk(200, lambda p: be.matmul_many(p, M, stream))
+    t, _ = timer.until(lambda i: walk(ceil_n, lambda p: be.matmul_many(p, M, stream)))
+    be.set_decode_mode("stream")
+    exact_us = t / ceil_n * 1e6
+    log(f"exact-operand kernel: {exact_us:.2f} us")
 
     # one isolated launch (idle GPU before and after)
-    lat = []
-    one = plan_of(1)
-    for _ in range(20):
-        lat.append(timed_many(be, one, M, stream, torch) * 1e6)
-    lat.sort()
-
-    # spread: batches of 25 back-to-back launches (one pass over the weight copies), each timed on its own
-    per = []
-    batch = plan_of(copies)
-    for _ in range(40):
-        per.append(timed_many(be, batch, M, stream, torch) / copies * 1e6)
-    per.sort()
-    spread = {"min": round(per[0], 2), "median": round(per[len(per) // 2], 2), "p95": round(per[int(len(per) * 0.95) - 1], 2),
-              "of": f"{len(per)} batches of {copies} back-to-back launches, us per launch"}
+    prepare(1)
+    lat = sorted(timer.once(lambda: walk(1, lambda p: be.matmul_many(p, M, stream))) * 1e6 for _ in range(20))
+    per = sorted(t / args.steps * 1e6 for t in passes)
+    spread = {"min": round(per[0], 3), "median": round(per[len(per) // 2], 3), "max": round(per[-1], 3),
+              "of": f"{len(per)} timed passes of {args.steps} back-to-back launches, us per launch"}
 
     result = {
         "metric": "Q4 GEMV GB/s at 4096x14336 b=1",
@@ -195,96 +264,182 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32 (f16 activations x exact int4 weights on f16 MFMA, fp32 accumulate, f16 scale applied in fp32)",
+        "dtype": "f32 (f16 activations x int4 weights as f16 subnormals (q+8)*2^-22 on the f16 MFMA, bias removed inside the "
+                 "fp32 accumulation, f16 scale applied in fp32; decode mode STREAM)",
         "data": "synthetic (seeded Philox: W~N(0,0.02) quantised per 32-group, x~N(0,1))",
         "config": {"workload": "Q4 decode GEMV, K=4096 -> N=14336, M=1, x f16, y f32 (BASELINE configs[1])",
-                   "weight_copies_rotated": int(copies), "algorithmic_bytes_per_step": int(alg_bytes)},
+                   "weight_copies_rotated": int(copies), "algorithmic_bytes_per_step": int(alg_bytes),
+                   "timed_passes": len(passes), "timed_device_ms": round(sum(passes) * 1e3, 2)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_DECODE_BYTES},
         "parity_rel_l2": rel_l2,
         "single_launch_us": round(lat[len(lat) // 2], 2),
         "us_per_launch_spread": spread,
+        "ceilings": ceilings,
+        "decode_mode_exact_us": round(exact_us, 3),
     }
 
     if not args.no_extra:
         extra = {}
-        # prefill GEMM, M = 512, bf16 activations (the second kernel of the path)
+        run_many = lambda Mx: (lambda p: be.matmul_many(p, Mx, stream))
+        # ---- prefill GEMM, M = 512, bf16 activations (the second kernel of the path)
         Mp = 512
         xp = torch.from_numpy(synth.activations(4, Mp, K)).to(dev).to(torch.bfloat16)
         yp = torch.empty((Mp, N), dtype=torch.float32, device=dev)
         be.matmul(w0, xp, yp, stream=stream)
         torch.cuda.synchronize()
-        refp = xp.double() @ torch.from_numpy(formats.dequantize(q, s)).to(dev).double().T
+        wdq = torch.from_numpy(formats.dequantize(q, s)).to(dev)
+        refp = xp.double() @ wdq.double().T
         relp = float(((yp.double() - refp).norm() / refp.norm()).item())
         del refp
         nrep = 50
-        planp = be.plan_many([ws[i % copies] for i in range(nrep)], [xp] * nrep, [yp] * nrep)
-        be.matmul_many(planp, Mp, stream)
-        elp = timed_many(be, planp, Mp, stream, torch) / nrep
+
+        pplans = {c: be.plan_many([ws[(c + j) % copies] for j in range(nrep)], [xp] * nrep, [yp] * nrep) for c in range(copies)}
+
+        def prefill_pass(i):
+            pl = pplans[cursor[0]]
+            cursor[0] = (cursor[0] + nrep) % copies
+            be.matmul_many(pl, Mp, stream)
+
+        prefill_pass(0)
+        tp, _ = timer.until(prefill_pass)
+        elp = tp / nrep
         tfl = 2.0 * Mp * N * K / elp / 1e12
+        # yardsticks on the same box: the vendor's dense bf16 GEMM of the same shape (no dequantisation),
+        # and what a loop of nothing but MFMAs sustains
+        wb = wdq.to(torch.bfloat16)
+        wbs = [wb] + [wb.clone() for _ in range(7)]          # 8 x 117 MB: dense weights also come from HBM
+        for j in range(8):
+            torch.matmul(xp, wbs[j].T)
+        tt, _ = timer.until(lambda i: [torch.matmul(xp, wbs[j % 8].T) for j in range(40)])
+        dense_us = tt / 40 * 1e6
+        del wb, wbs, wdq
+        sink = torch.zeros(4, dtype=torch.float32, device=dev)
+        be.debug_mfma_loop(2, 2000, sink, stream)
+        tm = min(timer.once(lambda: be.debug_mfma_loop(2, 20000, sink, stream)) for _ in range(3))
+        cus = torch.cuda.get_device_properties(0).multi_processor_count
+        mfma_tfl = cus * 4 * 2 * 20000 * 16 * 16384 / tm / 1e12
         extra["prefill_gemm_M512"] = {
-            "workload": "Q4 prefill GEMM, M=512, K=4096 -> N=14336, X bf16, Y f32 (BASELINE configs[3])",
+            "workload": "Q4 prefill GEMM, M=512, K=4096 -> N=14336, X bf16, Y f32 (BASELINE configs[3]), weights rotating "
+                        "through HBM; per call = activation staging pass + multiply",
             "us": round(elp * 1e6, 1), "tflops": round(tfl, 1), "parity_rel_l2": relp,
             "roofline": {"bound": "mfma", "achieved": round(tfl, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
-                         "unit": "TFLOP/s", "frac": round(tfl / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": TRAFFIC_PREFILL_M512_BYTES}}
-        log(f"prefill GEMM M=512: {elp * 1e6:.1f} us, {tfl:.1f} TFLOP/s, rel_l2 {relp:.2e}")
-        # batch sweep of the decode kernel on the same shape
-        sweep = {}
-        for Mb in (4, 8, 16):
-            xb = torch.from_numpy(synth.activations(3, Mb, K, outliers=0.001)).to(dev).to(torch.float16)
-            yb = torch.empty((Mb, N), dtype=torch.float32, device=dev)
-            n = 240
-            pl = be.plan_many([ws[i % copies] for i in range(n)], [xb] * n, [yb] * n)
-            be.matmul_many(pl, Mb, stream)
-            e = timed_many(be, pl, Mb, stream, torch) / n
-            sweep[f"M{Mb}"] = {"us": round(e * 1e6, 2),
-                               "GB/s": round(formats.matmul_bytes(bits, N, K, Mb, 2, 4) / e / 1e9, 1)}
-        extra["decode_batch_sweep_4096x14336"] = sweep
-        # the sweep's second shape, the down projection (BASELINE configs[2]): 256 strips of 112 K tiles
+                         "unit": "TFLOP/s", "frac": round(tfl / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": TRAFFIC_PREFILL_M512_BYTES},
+            "yardsticks_same_box": {
+                "torch_matmul_bf16_dense_512x4096x14336_us": round(dense_us, 1),
+                "torch_matmul_bf16_dense_tflops": round(2.0 * Mp * N * K / (dense_us * 1e-6) / 1e12, 1),
+                "pure_mfma_f16_loop_tflops": round(mfma_tfl, 1),
+                "pure_mfma_loop_frac_of_published_peak": round(mfma_tfl / MFMA_BF16_PEAK_TFLOPS, 4)}}
+        log(f"prefill GEMM M=512: {elp * 1e6:.1f} us, {tfl:.1f} TFLOP/s, rel_l2 {relp:.2e}; dense bf16 {dense_us:.1f} us; "
+            f"MFMA loop {mfma_tfl:.0f} TFLOP/s")
+
+        # ---- batch sweep of the decode kernels on the same shape
+        def sweep_shape(wl, Kx, Nx, Ms, bitsx=bits):
+            out = {}
+            for Mb in Ms:
+                xb = torch.from_numpy(synth.activations(3, Mb, Kx, outliers=0.001)).to(dev).to(torch.float16)
+                yb = [torch.empty((Mb, Nx), dtype=torch.float32, device=dev)]
+                n = 240
+                cur = [0]
+                spl = {}
+                c = 0
+                for _ in range(len(wl)):
+                    spl.setdefault(c, plan_of(n, c, wl, xb, yb))
+                    c = (c + n) % len(wl)
+
+                def one(i):
+                    pl = spl[cur[0]]
+                    cur[0] = (cur[0] + n) % len(wl)
+                    be.matmul_many(pl, Mb, stream)
+
+                one(0)
+                t, _ = timer.until(one)
+                e = t / n
+                g = formats.matmul_bytes(bitsx, Nx, Kx, Mb, 2, 4) / e / 1e9
+                out[f"M{Mb}"] = {"us": round(e * 1e6, 2), "GB/s": round(g, 1), "frac_of_hbm_peak": round(g / HBM_PEAK_GBS, 4)}
+            return out
+
+        extra["decode_batch_sweep_4096x14336"] = sweep_shape(ws, K, N, (2, 4, 8, 16, 32))
         for t in ws[1:]:
             t.free()
         del ws[1:]
+        # the sweep's second shape, the down projection (BASELINE configs[2]): 256 strips of 112 K tiles
         qd, sd = formats.quantize(synth.weights(6, K, N), bits)
         wd = [be.upload_quantized(qd, sd, bits)]
         wd += [wd[0].clone() for _ in range(copies - 1)]
         del qd, sd
-        sweep_d = {}
-        for Mb in (1, 4, 8, 16):
-            xb = torch.from_numpy(synth.activations(3, Mb, N, outliers=0.001)).to(dev).to(torch.float16)
-            yb = torch.empty((Mb, K), dtype=torch.float32, device=dev)
-            n = 240
-            pl = be.plan_many([wd[i % copies] for i in range(n)], [xb] * n, [yb] * n)
-            be.matmul_many(pl, Mb, stream)
-            e = timed_many(be, pl, Mb, stream, torch) / n
-            sweep_d[f"M{Mb}"] = {"us": round(e * 1e6, 2),
-                                 "GB/s": round(formats.matmul_bytes(bits, K, N, Mb, 2, 4) / e / 1e9, 1)}
-        extra["decode_batch_sweep_14336x4096"] = sweep_d
+        extra["decode_batch_sweep_14336x4096"] = sweep_shape(wd, N, K, (1, 4, 8, 16, 32))
         for t in wd:
             t.free()
         del wd
-        # the same kernel on Q8 blocks (twice the bytes per weight, half the unpack work per byte):
-        # shows how much of the Q4 time is arithmetic rather than memory
+        # the same kernels on Q8 blocks (twice the bytes per weight)
         q8, s8 = formats.quantize(synth.weights(2, N, K), formats.Q8)
         n8 = max(2, (3 * MALL_BYTES) // formats.weight_bytes(formats.Q8, N, K) + 1)
         w8 = [be.upload_quantized(q8, s8, formats.Q8)]
         w8 += [w8[0].clone() for _ in range(n8 - 1)]
         del q8, s8
-        q8res = {}
-        for Mb in (1, 8):
-            xb = torch.from_numpy(synth.activations(3, Mb, K)).to(dev).to(torch.float16)
-            yb = torch.empty((Mb, N), dtype=torch.float32, device=dev)
-            n = 240
-            pl = be.plan_many([w8[i % n8] for i in range(n)], [xb] * n, [yb] * n)
-            be.matmul_many(pl, Mb, stream)
-            e = timed_many(be, pl, Mb, stream, torch) / n
-            gbs = formats.matmul_bytes(formats.Q8, N, K, Mb, 2, 4) / e / 1e9
-            q8res[f"M{Mb}"] = {"us": round(e * 1e6, 2), "GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
-        extra["q8_decode_4096x14336"] = q8res
+        extra["q8_decode_4096x14336"] = sweep_shape(w8, K, N, (1, 8), formats.Q8)
         for t in w8:
             t.free()
         del w8
-        # the reference-shaped decode step: 32 layers x (q,k,v,o,gate,up,down), Q4, random init,
-        # one native walk over the 224 linear nodes per step (BASELINE configs[4])
+
+        # ---- LM head: 4096 -> 128256 (/root/reference/decide/pipeline.md:51), weights made on the device
+        NL = 128256
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(1234)
+        wl = torch.empty((NL, K), dtype=torch.float32, device=dev).normal_(0.0, 0.02, generator=gen)
+        ql = torch.empty(NL * K // 2, dtype=torch.uint8, device=dev)
+        sl = torch.empty(NL * (K // 32), dtype=torch.int16, device=dev)
+        be.quantize(bits, wl, NL, K, ql, sl)
+        lm = [be.weight_from_device(bits, NL, K, ql, sl)]
+        torch.cuda.synchronize()
+        # ---- import stage (f2): f32 [N,K] on the device -> quantise -> native layout, timed here on the
+        # LM-head tensor (2.1 GB of f32 in, 295 MB out) and, from host blocks, on the headline tensor
+        def import_once():
+            be.quantize(bits, wl, NL, K, ql, sl, stream)
+            h = be.weight_from_device(bits, NL, K, ql, sl, stream)
+            return h
+        hs = []
+        ti, _ = timer.until(lambda i: hs.append(import_once()), min_s=0.02, max_passes=6)
+        for h in hs:
+            h.free()
+        imp_bytes = 4 * NL * K + formats.weight_bytes(bits, NL, K)
+        tq = min(timer.once(lambda: be.quantize(bits, wl, NL, K, ql, sl, stream)) for _ in range(3))
+        blocks = np.ascontiguousarray(formats.pack_blocks(q, s, bits))
+        tu0 = time.perf_counter()
+        hu = be.upload(bits, formats.BLOCK_AOS, N, K, blocks)
+        tu = time.perf_counter() - tu0
+        hu.free()
+        extra["import_stage"] = {
+            "workload": f"f32 [{NL},{K}] resident in HBM -> cybq_quantize (PLANAR) -> cybq_weight_from_device (native tiles)",
+            "us": round(ti * 1e6, 1), "algorithmic_bytes": int(imp_bytes),
+            "GB/s": round(imp_bytes / ti / 1e9, 1), "frac_of_hbm_peak": round(imp_bytes / ti / 1e9 / HBM_PEAK_GBS, 4),
+            "quantize_only_us": round(tq * 1e6, 1), "repack_only_us": round((ti - tq) * 1e6, 1),
+            "repack_GB/s": round(2 * formats.weight_bytes(bits, NL, K) / max(ti - tq, 1e-9) / 1e9, 1),
+            "upload_from_host_blocks_4096x14336_ms": round(tu * 1e3, 2),
+            "note": "algorithmic bytes = the f32 source read once + the packed tensor written once; the PLANAR intermediate "
+                    "(written, read again) is extra traffic the stage pays; the host upload includes the PCIe copy"}
+        log(f"import stage: {ti * 1e6:.0f} us for {imp_bytes / 1e9:.2f} GB = {imp_bytes / ti / 1e9:.0f} GB/s "
+            f"(quantise {tq * 1e6:.0f} us); host upload {tu * 1e3:.1f} ms")
+        del wl
+        lm += [lm[0].clone() for _ in range(3)]              # 4 x 295 MB
+        extra["lm_head_4096x128256"] = sweep_shape(lm, K, NL, (1, 8))
+        # parity of the LM-head shape on a sample of rows (the full tensor is checked by the test-suite)
+        xb = torch.from_numpy(synth.activations(3, 1, K)).to(dev).to(torch.float16)
+        yb = torch.empty((1, NL), dtype=torch.float32, device=dev)
+        be.matmul(lm[0], xb, yb, stream=stream)
+        rows = torch.arange(0, NL, 997, device=dev)
+        qrows = formats.unpack_planar(ql.view(NL, K // 2)[rows].cpu().numpy().reshape(-1), bits, len(rows), K)
+        srows = sl.view(NL, K // 32)[rows].cpu().numpy().view(np.uint16)
+        refl = xb.float().cpu().numpy().astype(np.float64) @ formats.dequantize(qrows, srows).astype(np.float64).T
+        gotl = yb[0, rows].cpu().numpy().astype(np.float64)
+        extra["lm_head_4096x128256"]["parity_rel_l2_sampled_rows"] = float(np.linalg.norm(gotl - refl[0]) / np.linalg.norm(refl))
+        for t in lm:
+            t.free()
+        del lm, ql, sl
+
+        # ---- the reference-shaped decode step: 32 layers x (q,k,v,o,gate,up,down), Q4, random init,
+        # one native walk over the linear nodes per step (BASELINE configs[4])
         from cyb_amd import stack as stk
         stack_out = {}
         for label, shapes, epis in (("per_linear_224_launches", None, False),
@@ -298,20 +453,39 @@ def main():
                 edges = stk.edges_for(st, Ms, shapes=shapes)
                 pl = stk.plan(st, edges)
                 be.matmul_many(pl, Ms, stream)
-                reps = 20
-                torch.cuda.synchronize()
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                a.record()
-                for _ in range(reps):
-                    be.matmul_many(pl, Ms, stream)
-                b.record()
-                torch.cuda.synchronize()
-                per = a.elapsed_time(b) * 1e-3 / reps
+                per, _ = timer.until(lambda i: be.matmul_many(pl, Ms, stream))
                 res[f"M{Ms}"] = {"us_per_step": round(per * 1e6, 1),
                                  "GB/s": round(st.step_bytes(Ms) / per / 1e9, 1),
                                  "frac_of_hbm_peak": round(st.step_bytes(Ms) / per / 1e9 / HBM_PEAK_GBS, 4),
                                  "linear_stack_tok_per_s": round(Ms / per, 1)}
                 log(f"decode stack {label} M={Ms}: {per * 1e6:.0f} us/step")
+                if shapes is not None and not epis:
+                    # what the epilogues replace: the same step with SwiGLU and the two residual adds as
+                    # launches of their own between the linears (plain torch ops on the same buffers)
+                    gu, res_o, res_d = edges["out.gate_up_proj"], edges["out.o_proj"], edges["out.down_proj"]
+                    h = gu.shape[1] // 2
+                    act = torch.empty((Ms, h), dtype=torch.float32, device=dev)
+                    r0 = torch.zeros_like(res_o)
+
+                    def step_with_elementwise():
+                        for layer in range(32):
+                            be.matmul_many(layer_plans[layer][0], Ms, stream)       # qkv, o
+                            torch.add(res_o, r0, out=res_o)
+                            be.matmul_many(layer_plans[layer][1], Ms, stream)       # gate_up
+                            torch.mul(torch.nn.functional.silu(gu[:, :h]), gu[:, h:], out=act)
+                            be.matmul_many(layer_plans[layer][2], Ms, stream)       # down
+                            torch.add(res_d, r0, out=res_d)
+
+                    xs_all, ys_all = [edges[n.x] for n in st.nodes], [edges[n.y] for n in st.nodes]
+                    layer_plans = []
+                    for layer in range(32):
+                        b0 = layer * 4
+                        layer_plans.append([be.plan_many(st.weights[b0 + a:b0 + b], xs_all[b0 + a:b0 + b], ys_all[b0 + a:b0 + b])
+                                            for a, b in ((0, 2), (2, 3), (3, 4))])
+                    step_with_elementwise()
+                    per2, _ = timer.until(lambda i: step_with_elementwise())
+                    res[f"M{Ms}"]["us_per_step_with_swiglu_and_residual_as_separate_launches"] = round(per2 * 1e6, 1)
+                    log(f"  ... with SwiGLU / residual adds as separate launches: {per2 * 1e6:.0f} us/step")
             if shapes is not None and not epis:
                 # prefill of one 512-token chunk through the same stack (bf16 activations), and both
                 # phases in the units the reference's UI reports (tok_in_s / tok_out_s,
@@ -320,14 +494,7 @@ def main():
                 edges = stk.edges_for(st, Mp2, shapes=shapes, xdtype=torch.bfloat16)
                 pl = stk.plan(st, edges)
                 be.matmul_many(pl, Mp2, stream)
-                torch.cuda.synchronize()
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                a.record()
-                for _ in range(3):
-                    be.matmul_many(pl, Mp2, stream)
-                b.record()
-                torch.cuda.synchronize()
-                per = a.elapsed_time(b) * 1e-3 / 3
+                per, _ = timer.until(lambda i: be.matmul_many(pl, Mp2, stream), max_passes=6)
                 flops = sum(2.0 * Mp2 * w.N * w.K for w in st.weights)
                 res["prefill_M512"] = {"ms_per_chunk": round(per * 1e3, 3), "TFLOP/s": round(flops / per / 1e12, 1),
                                        "frac_of_mfma_peak": round(flops / per / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}

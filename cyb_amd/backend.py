@@ -88,7 +88,10 @@ def load_library() -> ctypes.CDLL:
     lib.cybq_matmul_many.argtypes = [vp, i64, vp, vp, vp, ci, i64, ci, vp]
     lib.cybq_dequant.argtypes = [vp, vp, vp, vp]
     lib.cybq_quantize.argtypes = [vp, ci, vp, i64, i64, vp, vp, vp]
+    # diagnostics (cyb_amd/csrc/cybq_debug.h), not part of the operator interface
     lib.cybq_debug_set_gemv_tuning.argtypes = [ci, ci, ci]
+    lib.cybq_debug_read_weight.argtypes = [vp, i64, vp, ci, vp, vp, vp]
+    lib.cybq_debug_mfma_loop.argtypes = [vp, ci, ci, vp, vp]
     _lib = lib
     return lib
 
@@ -354,6 +357,16 @@ class Backend:
         if mode not in codes:
             raise CybqError(-1, "invalid argument", f"decode mode {mode!r}")
         self._check(self._lib.cybq_set_decode_mode(self._ctx, codes[mode]))
+
+    def debug_read_weights(self, plan: "MatmulPlan", with_io: bool, x=None, y=None, stream: int = 0) -> None:
+        """Diagnostics: the one-row decode kernel's memory requests without its arithmetic, one launch per
+        weight of `plan` (with_io: also the activation read and a 16-float store per strip)."""
+        self._check(self._lib.cybq_debug_read_weight(self._ctx, plan.count, plan.w, 1 if with_io else 0, _ptr(x), _ptr(y),
+                                                     stream))
+
+    def debug_mfma_loop(self, waves_per_simd: int, iters: int, sink, stream: int = 0) -> None:
+        """Diagnostics: `iters` x 16 independent v_mfma_f32_16x16x32_f16 per wave on every SIMD."""
+        self._check(self._lib.cybq_debug_mfma_loop(self._ctx, waves_per_simd, iters, _ptr(sink), stream))
 
     def set_gemv_tuning(self, waves: int = 0, rows_kernel: int = 0, unroll: int = 0) -> None:
         """Diagnostics: waves per workgroup; decode kernel choice (0 auto, 1 always the

@@ -10,6 +10,7 @@
 #include <vector>
 
 #include "../../include/cybq.h"
+#include "cybq_debug.h"
 #include "cybq_internal.h"
 
 struct cybq_ctx {
@@ -533,11 +534,41 @@ int cybq_quantize(cybq_ctx* ctx, cybq_quant quant, const float* src, int64_t N, 
     return CYBQ_OK;
 }
 
-/* Test and benchmark hook (not part of the operator interface): overrides the
- * decode kernel's launch heuristics; 0 restores the automatic choice. */
+/* ---- diagnostics declared in cybq_debug.h (not part of the operator interface) ---- */
+
 int cybq_debug_set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll)
 {
     cybq::set_gemv_tuning(waves_per_group, rows_kernel, unroll);
+    return CYBQ_OK;
+}
+
+int cybq_debug_read_weight(cybq_ctx* ctx, int64_t count, const cybq_weight* const* w, int with_io, const void* x, void* y,
+                           void* stream)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (count < 0 || (count > 0 && !w) || (with_io && (!x || !y))) return fail(ctx, CYBQ_ERR_INVALID, "w / x / y is NULL");
+    DeviceGuard guard(ctx->device);
+    if (guard.err != hipSuccess) return fail_hip(ctx, guard.err, "hipSetDevice");
+    for (int64_t i = 0; i < count; i++) {
+        if (!w[i]) return fail(ctx, CYBQ_ERR_INVALID, "w[i] is NULL");
+        hipError_t e = cybq::launch_read_probe(view_of(w[i]), with_io != 0, x, y, static_cast<hipStream_t>(stream));
+        if (e == hipErrorInvalidValue) {
+            (void)hipGetLastError();
+            return fail(ctx, CYBQ_ERR_UNSUPPORTED, "probe needs K % 512 == 0 and K <= 16384");
+        }
+        if (e != hipSuccess) return fail_hip(ctx, e, "probe launch");
+    }
+    return CYBQ_OK;
+}
+
+int cybq_debug_mfma_loop(cybq_ctx* ctx, int waves_per_simd, int iters, float* sink, void* stream)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (!sink) return fail(ctx, CYBQ_ERR_INVALID, "sink is NULL");
+    DeviceGuard guard(ctx->device);
+    if (guard.err != hipSuccess) return fail_hip(ctx, guard.err, "hipSetDevice");
+    hipError_t e = cybq::launch_mfma_loop(ctx->num_cus, waves_per_simd, iters, sink, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail_hip(ctx, e, "mfma loop launch");
     return CYBQ_OK;
 }
 

@@ -1,0 +1,41 @@
+/*
+ * cybq_debug.h - diagnostics exported by libcybq.so for the tests and the benchmark of this
+ * repository.  NOT part of the operator interface (include/cybq.h): nothing a runtime binds,
+ * no stability promise.  The tuning override is process-wide mutable state; use it from one
+ * thread, with no launches in flight.
+ */
+#ifndef CYBQ_DEBUG_H
+#define CYBQ_DEBUG_H
+
+#include "../../include/cybq.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Overrides the decode kernels' launch heuristics for experiments: waves per
+ * workgroup (1..16); which decode kernel runs (0 automatic, 1 always the
+ * x-in-registers kernel, 2 never); tiles in flight per wave of the streaming
+ * variant (2 or 4).  0 restores the automatic choice.  Any non-zero value also keeps
+ * one-row calls away from the kernel of gemv1.hip. */
+int cybq_debug_set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll);
+
+/* Ceiling probes for the one-row decode kernel: a kernel that issues exactly that kernel's
+ * memory requests for tensor `w` (one workgroup per 16-row strip, whole strip requested up
+ * front) and does nothing with the data.
+ *   with_io = 0  weights and scales only, nothing stored
+ *   with_io = 1  also reads the activations x [K] f16 the way the kernel does and stores
+ *                16 floats per strip to y [N]
+ * `count` launches back to back, one per tensor of w[] (like cybq_matmul_many).
+ * Needs K a multiple of 512 and at most 16384. */
+int cybq_debug_read_weight(cybq_ctx* ctx, int64_t count, const cybq_weight* const* w, int with_io, const void* x, void* y,
+                           void* stream);
+
+/* A loop of independent v_mfma_f32_16x16x32_f16 on every SIMD of the chip: `waves_per_simd`
+ * waves each issue `iters` x 16 instructions.  flops = CUs * 4 * waves_per_simd * iters * 16 * 16384. */
+int cybq_debug_mfma_loop(cybq_ctx* ctx, int waves_per_simd, int iters, float* sink, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

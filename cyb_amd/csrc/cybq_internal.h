@@ -51,6 +51,10 @@ struct LdsRequest {
     static inline const bool registered = (register_lds_request(reinterpret_cast<const void*>(Kernel), Bytes), true);
 };
 
+// measurement probes (debug.hip)
+hipError_t launch_read_probe(const WeightView& w, bool io, const void* x, void* y, hipStream_t st);
+hipError_t launch_mfma_loop(int num_cus, int waves_per_simd, int iters, float* sink, hipStream_t st);
+
 // test/bench hook: overrides the decode kernel's launch heuristics (0 = automatic)
 void set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll);
 

@@ -236,14 +236,6 @@ int cybq_weight_from_device(cybq_ctx* ctx, cybq_quant quant, int64_t N, int64_t 
                             const void* q_dev, const void* scales_dev, void* stream,
                             cybq_weight** out);
 
-/* ---- diagnostics (not part of the operator interface) ------------------- */
-
-/* Overrides the decode kernel's launch heuristics for experiments: waves per
- * workgroup (1..16); which decode kernel runs (0 automatic, 1 always the
- * x-in-registers kernel, 2 never); tiles in flight per wave of the streaming
- * variant (2 or 4).  0 restores the automatic choice.  Process-wide. */
-int cybq_debug_set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll);
-
 #ifdef __cplusplus
 }
 #endif

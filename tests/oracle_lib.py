@@ -13,6 +13,7 @@ import numpy as np
 
 _ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 _SO = os.path.join(_ROOT, "oracle", "_build", "libcybq_oracle.so")
+_SO_CPU = os.path.join(_ROOT, "oracle", "_build", "libcybq_cpu_baseline.so")
 
 
 def _arr(a, dtype):
@@ -22,7 +23,7 @@ def _arr(a, dtype):
 
 class Oracle:
     def __init__(self):
-        if not os.path.exists(_SO):
+        if not os.path.exists(_SO) or not os.path.exists(_SO_CPU):
             subprocess.run(["make"], cwd=os.path.join(_ROOT, "oracle"), check=True,
                            stdout=subprocess.DEVNULL)
         L = ctypes.CDLL(_SO)
@@ -142,6 +143,29 @@ class Oracle:
 
     def matmul_mt(self, q, s, x, threads):
         return self._mm(self.L.cybq_oracle_matmul_blocked_mt, q, s, x, np.float32, threads)
+
+    # the optimised CPU path that bench.py times beside the GPU (oracle/cybq_cpu_baseline.c) ----
+    def _cpu(self):
+        if getattr(self, "_C", None) is None:
+            C = ctypes.CDLL(_SO_CPU)
+            C.cybq_cpu_q4_0_matmul.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_void_p,
+                                               ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int]
+            C.cybq_cpu_baseline_isa.restype = ctypes.c_char_p
+            self._C = C
+        return self._C
+
+    def cpu_baseline_isa(self) -> str:
+        return self._cpu().cybq_cpu_baseline_isa().decode()
+
+    def cpu_baseline_q4_0(self, blocks, N, K, x, threads, out=None):
+        """y [M,N] f32 = x [M,K] f32 times the Q4_0 BLOCK_AOS tensor `blocks` (uint8, N*K/32*18 bytes)."""
+        assert blocks.dtype == np.uint8 and blocks.flags.c_contiguous and blocks.size == N * (K // 32) * 18
+        x, xp = _arr(x, np.float32)
+        M = x.shape[0]
+        if out is None:
+            out = np.empty((M, N), np.float32)
+        used = self._cpu().cybq_cpu_q4_0_matmul(blocks.ctypes.data, N, K, xp, M, out.ctypes.data, threads)
+        return out, used
 
     def rel_l2(self, a, b):
         a, ap = _arr(a, np.float32)
