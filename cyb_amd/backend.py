@@ -177,6 +177,7 @@ class MatmulPlan:
         if not (n == len(xs) == len(ys)):
             raise CybqError(-1, "invalid argument", "weights / xs / ys differ in length")
         self.count = n
+        self.checked = set()                            # batch sizes whose buffers were validated
         self.keep = (list(weights), list(xs), list(ys), list(residuals or []))      # keeps tensors and handles alive
         arr = ctypes.c_void_p * n
         self.w = arr(*[w.handle.value for w in weights])
@@ -236,6 +237,14 @@ class Backend:
         q = np.ascontiguousarray(q)
         qp = q.ctypes.data_as(ctypes.c_void_p)
         sp = None
+        if N >= 1 and K >= 32 and K % 32 == 0 and quant in (formats.Q4, formats.Q8):
+            groups = N * (K // 32)
+            if layout == formats.PLANAR:
+                need_q, need_s = N * K * quant // 8, groups * 2
+            else:
+                need_q, need_s = groups * (18 if quant == formats.Q4 else 34), 0
+            if q.nbytes < need_q or (need_s and scales is not None and np.asarray(scales).nbytes < need_s):
+                raise CybqError(-2, "bad shape", f"host buffers are smaller than a [{N},{K}] Q{quant} tensor in this layout")
         if scales is not None:
             scales = np.ascontiguousarray(scales)
             sp = scales.ctypes.data_as(ctypes.c_void_p)
@@ -265,10 +274,30 @@ class Backend:
         return w
 
     # ---- ops (x / y / out: torch tensors on this device, or raw device addresses)
+    def _check_tensor(self, t, what: str, elems: int) -> None:
+        """A tensor handed to the C ABI must be contiguous, on this context's device and large enough:
+        the library only sees a raw pointer.  (Raw integer addresses are the caller's responsibility.)"""
+        if t is None or isinstance(t, int):
+            return
+        if not t.is_contiguous():
+            raise CybqError(-2, "bad shape", f"{what} must be contiguous")
+        if not t.is_cuda or (t.device.index or 0) != self.device:
+            raise CybqError(-1, "invalid argument", f"{what} must live on cuda:{self.device}")
+        if t.numel() < elems:
+            raise CybqError(-2, "bad shape", f"{what} holds {t.numel()} elements, the call needs {elems}")
+
+    def _check_call(self, w: QWeight, x, y, M: int, epilogue: str = "none", residual=None, gamma=None) -> None:
+        n_out = w.N // 2 if epilogue == "swiglu" else w.N
+        self._check_tensor(x, "x", M * w.K)
+        self._check_tensor(y, "y", M * n_out)
+        self._check_tensor(residual, "residual", M * n_out)
+        self._check_tensor(gamma, "gamma", w.K)
+
     def matmul(self, w: QWeight, x, y, M: Optional[int] = None, xdt: Optional[int] = None,
                ydt: Optional[int] = None, stream: int = 0) -> None:
         if M is None:
             M = int(x.shape[0]) if x.dim() == 2 else 1
+        self._check_call(w, x, y, M)
         self._check(self._lib.cybq_matmul(self._ctx, w.handle, _ptr(x), _dtype_code(x, xdt), M, _ptr(y),
                                           _dtype_code(y, ydt), stream))
 
@@ -276,6 +305,7 @@ class Backend:
         """cybq_matmul_static: the same op with its scratch in a static device array (allocates nothing)."""
         if M is None:
             M = int(x.shape[0]) if x.dim() == 2 else 1
+        self._check_call(w, x, y, M)
         self._check(self._lib.cybq_matmul_static(self._ctx, w.handle, _ptr(x), _dtype_code(x, None), M, _ptr(y),
                                                  _dtype_code(y, None), stream))
 
@@ -287,6 +317,7 @@ class Backend:
             raise CybqError(-1, "invalid argument", f"unknown epilogue {epilogue!r}")
         if M is None:
             M = int(x.shape[0]) if x.dim() == 2 else 1
+        self._check_call(w, x, y, M, epilogue, residual)
         self._check(self._lib.cybq_matmul_ex(self._ctx, w.handle, _ptr(x), _dtype_code(x, None), M, _ptr(y),
                                              _dtype_code(y, None), EPILOGUES[epilogue], _ptr(residual), stream))
 
@@ -297,6 +328,7 @@ class Backend:
             raise CybqError(-1, "invalid argument", f"unknown epilogue {epilogue!r}")
         if M is None:
             M = int(x.shape[0]) if x.dim() == 2 else 1
+        self._check_call(w, x, y, M, epilogue, residual, gamma)
         self._check(self._lib.cybq_matmul_norm(self._ctx, w.handle, _ptr(x), _dtype_code(x, None), M, _ptr(gamma),
                                                _dtype_code(gamma, None), ctypes.c_float(eps), _ptr(y),
                                                _dtype_code(y, None), EPILOGUES[epilogue], _ptr(residual), stream))
@@ -315,6 +347,14 @@ class Backend:
         return MatmulPlan(self, weights, xs, ys, epilogues, residuals)
 
     def matmul_many(self, plan: "MatmulPlan", M: int, stream: int = 0) -> None:
+        if M not in plan.checked:                      # once per plan and batch size, not per step
+            ws, xs, ys, rs = plan.keep
+            for i, w in enumerate(ws):
+                epi = "none"
+                if plan.epi is not None:
+                    epi = next(k for k, v in EPILOGUES.items() if v == plan.epi[i])
+                self._check_call(w, xs[i], ys[i], M, epi, rs[i] if rs else None)
+            plan.checked.add(M)
         if plan.epi is not None:
             self._check(self._lib.cybq_matmul_many_ex(self._ctx, plan.count, plan.w, plan.x, plan.y, plan.epi, plan.res,
                                                       plan.xdt, M, plan.ydt, stream))

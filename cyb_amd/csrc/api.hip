@@ -3,6 +3,7 @@
 // this boundary.
 #include <hip/hip_runtime.h>
 
+#include <cmath>
 #include <cstdio>
 #include <cstring>
 #include <new>
@@ -31,6 +32,9 @@ struct cybq_weight {
     uint8_t* data = nullptr;            // native tiles (q words + scales per tile), strip-major
     size_t bytes = 0;
     bool paired = false;                // made by cybq_weight_fuse_pairs: strips alternate gate / up
+    // some |scale| * qmax exceeds what f16 holds: the prefill kernels, which form scale * q in
+    // f16, would overflow; such a tensor takes the decode kernels (scale applied in fp32) for any M
+    bool wide_scales = false;
 };
 
 namespace cybq {
@@ -105,6 +109,30 @@ cybq::WeightView view_of(const cybq_weight* w)
     v.KT = w->KT;
     v.bits = w->bits;
     return v;
+}
+
+// largest finite f16 magnitude a scale may have for scale * q to stay inside f16: 65504 / qmax
+bool scale_is_wide(uint16_t bits, int quant)
+{
+    const int e = (bits >> 10) & 31, m = bits & 1023;
+    if (e == 31) return true;                                  // Inf / NaN
+    const float v = e == 0 ? (float)m * (1.0f / 16777216.0f) : std::ldexp((float)(m + 1024), e - 25);
+    return v * (quant == CYBQ_Q4 ? 8.0f : 128.0f) > 65504.0f;
+}
+
+bool any_wide_scale(int quant, int layout, int64_t groups, const void* q, const void* scales)
+{
+    if (layout == CYBQ_LAYOUT_PLANAR) {
+        const uint16_t* s = static_cast<const uint16_t*>(scales);
+        for (int64_t g = 0; g < groups; g++)
+            if (scale_is_wide(s[g], quant)) return true;
+        return false;
+    }
+    const size_t bs = quant == CYBQ_Q4 ? 18 : 34;
+    const uint8_t* b = static_cast<const uint8_t*>(q);
+    for (int64_t g = 0; g < groups; g++)
+        if (scale_is_wide((uint16_t)(b[g * bs] | (b[g * bs + 1] << 8)), quant)) return true;
+    return false;
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -261,6 +289,7 @@ int cybq_weight_upload(cybq_ctx* ctx, cybq_quant quant, cybq_layout layout, int6
     (void)hipFree(q_tmp);
     if (s_tmp) (void)hipFree(s_tmp);
     if (rc) return rc;
+    w->wide_scales = any_wide_scale(quant, layout, groups, q, scales);
     *out = w;
     return CYBQ_OK;
 }
@@ -310,6 +339,7 @@ int cybq_weight_clone(cybq_ctx* ctx, const cybq_weight* src, cybq_weight** out)
         return fail_hip(ctx, e, "weight clone");
     }
     w->paired = src->paired;
+    w->wide_scales = src->wide_scales;
     *out = w;
     return CYBQ_OK;
 }
@@ -373,7 +403,7 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
     hipError_t e;
     if (M <= 16) {
         e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->decode_exact, epi, st);
-    } else if (xdt == CYBQ_F32 ? !ctx->prefill_exact : M > 32) {
+    } else if (!w->wide_scales && (xdt == CYBQ_F32 ? !ctx->prefill_exact : M > 32)) {
         e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, workspace, workspace_bytes,
                               epi, st);
     } else {
@@ -458,6 +488,7 @@ int cybq_weight_fuse_pairs(cybq_ctx* ctx, const cybq_weight* gate, const cybq_we
         return fail_hip(ctx, e, "weight fuse");
     }
     w->paired = true;
+    w->wide_scales = gate->wide_scales || up->wide_scales;
     *out = w;
     return CYBQ_OK;
 }

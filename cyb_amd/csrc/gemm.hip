@@ -10,7 +10,7 @@
 //      kernel first restages X once per call in operand order - row block, scale
 //      group, lane - and the multiply streams it global -> registers with
 //      contiguous 1 KB loads, one K tile (four scale groups) ahead of its use.
-//      The same pass widens bf16 to f16 for FAST mode.
+//      The same pass turns bf16 / fp32 rows into f16 operands for FAST mode.
 //   W  is shared by the waves of a workgroup: per K tile (128 k = 4 groups) the NF native
 //      weight tiles are read once with 128-bit loads and dequantised to
 //      w = f32(scale) * q, which is exact in fp32 (11-bit x 4-bit significand).
@@ -30,9 +30,9 @@
 //   EXACT  as described above: two MFMAs per scale group in the type of X.
 //   FAST   one f16 MFMA per scale group.  The weight operand is round_f16(scale * q)
 //          (one rounding, relative error <= 2^-11, about 2e-4 relative L2 on Y -
-//          inside the operator's 1e-3 tolerance); bf16 activations are widened
-//          to f16 by the staging pass after a 2^-4 prescale that is undone in the
-//          epilogue, exact for 2^-10 <= |x| < 2^20.
+//          inside the operator's 1e-3 tolerance); bf16 and fp32 activations become
+//          f16 operands in the staging pass behind a power-of-two scale per row that is
+//          undone in the epilogue.
 //
 // Shapes with fewer tiles than CUs split K over workgroups: each split leaves fp32
 // partial sums in its own slab of the workspace and a last kernel adds the slabs in a
@@ -70,9 +70,12 @@ __device__ __forceinline__ float load_out_g(const void* p, int dt, int64_t idx)
 
 // Folded RMSNorm on the prefill path: the staging pass leaves, per row of the chunk, `nblk`
 // partial sums of squares; rstd of a row adds them in index order.
+// `unscale` (FAST mode with widened activations): the power of two every staged row was
+// divided by on its way to f16, to be multiplied back onto the finished sums.
 struct NormStats {
     const float* part;
     int nblk;
+    const float* unscale;
 };
 
 __device__ __forceinline__ float rstd_of(const NormStats& ns, int row, int K, float eps)
@@ -80,6 +83,14 @@ __device__ __forceinline__ float rstd_of(const NormStats& ns, int row, int K, fl
     float t = 0.f;
     for (int j = 0; j < ns.nblk; j++) t += ns.part[(int64_t)row * ns.nblk + j];
     return 1.0f / sqrtf(t / (float)K + eps);
+}
+
+// what a finished sum of row `row` is multiplied by before the epilogue
+__device__ __forceinline__ float row_factor(const NormStats& ns, bool norm, int row, int K, float eps)
+{
+    float f = ns.unscale ? ns.unscale[row] : 1.0f;
+    if (norm) f *= rstd_of(ns, row, K, eps);
+    return f;
 }
 
 // gamma[k0 .. k0+8) as fp32 (k0 a multiple of 8, gamma 16-byte aligned)
@@ -177,20 +188,6 @@ __device__ __forceinline__ float4_t mma(const Frag16& a, const Frag16& b, float4
 {
     if (XBF) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, c, 0, 0, 0);
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, c, 0, 0, 0);
-}
-
-// bf16 A operand -> f16 A operand, prescaled by 2^-4
-__device__ __forceinline__ Frag16 bf16_to_f16_frag(const Frag16& a)
-{
-    Frag16 o;
-#pragma unroll
-    for (int p = 0; p < 4; p++) {
-        float f0 = __builtin_bit_cast(float, a.u[p] << 16);
-        float f1 = __builtin_bit_cast(float, a.u[p] & 0xffff0000u);
-        half2_t h = {(_Float16)(f0 * 0.0625f), (_Float16)(f1 * 0.0625f)};
-        o.u[p] = as_u32(h);
-    }
-    return o;
 }
 
 // XBF = 1: X is bf16, 0: X is f16.  EXACT: see the header comment.
@@ -381,12 +378,12 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
             }
         return;
     }
-    if (epi.gamma) {                   // folded RMSNorm: scale every row by its rstd before the epilogue
+    if (epi.gamma || ns.unscale) {     // folded RMSNorm: rstd of the row; widened activations: the row's power of two
 #pragma unroll
         for (int i = 0; i < MF; i++)
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const float rs = rstd_of(ns, min(m0 + i * 16 + oct * 4 + r, M - 1), K, epi.eps);
+                const float rs = row_factor(ns, epi.gamma != nullptr, min(m0 + i * 16 + oct * 4 + r, M - 1), K, epi.eps);
 #pragma unroll
                 for (int f = 0; f < NF; f++) acc[i][f][r] *= rs;
             }
@@ -442,7 +439,7 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ part, int splits,
             g += part[s * slab + ig];
             u += part[s * slab + ig + 16];
         }
-        const float sc = epi.gamma ? out_scale * rstd_of(ns, m, K, epi.eps) : out_scale;
+        const float sc = out_scale * row_factor(ns, epi.gamma != nullptr, m, K, epi.eps);
         store_out_g(y, ydt, i, silu_mul(g * sc, u * sc));
         return;
     }
@@ -450,7 +447,7 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ part, int splits,
     float v = part[i];
     for (int s = 1; s < splits; s++) v += part[s * slab + i];
     v *= out_scale;
-    if (epi.gamma) v *= rstd_of(ns, (int)(i / N), K, epi.eps);
+    if (epi.gamma || ns.unscale) v *= row_factor(ns, epi.gamma != nullptr, (int)(i / N), K, epi.eps);
     if (epi.kind == kEpiAdd) v += load_out_g(epi.residual, ydt, i);
     store_out_g(y, ydt, i, v);
 }
@@ -468,7 +465,7 @@ __global__ void splitk_reduce4_kernel(const float* __restrict__ part, int splits
 #pragma unroll
     for (int e = 0; e < 4; e++) {
         float t = v[e] * out_scale;
-        if (epi.gamma) t *= rstd_of(ns, (int)((i + e) / N), K, epi.eps);
+        if (epi.gamma || ns.unscale) t *= row_factor(ns, epi.gamma != nullptr, (int)((i + e) / N), K, epi.eps);
         if (epi.kind == kEpiAdd) t += load_out_g(epi.residual, ydt, i + e);
         v[e] = t;
     }
@@ -548,25 +545,20 @@ hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt
     return hipErrorInvalidValue;
 }
 
-// X [M, K] row major -> A-operand order: for row block rb (16 rows, zero padded) and
-// scale group g, 64 x 16 B where slot (oct, r) = oct*16 + r holds row 16*rb + r,
-// k = 32*g + 8*oct .. +8.  WIDEN: bf16 -> f16 scaled by 2^-4 on the way (exact for
-// 2^-10 <= |x| < 2^20).  A workgroup moves one row block x 16 groups through LDS:
+// X [M, K] row major (16-bit elements, used as they are) -> A-operand order: for row block rb
+// (16 rows, zero padded) and scale group g, 64 x 16 B where slot (oct, r) = oct*16 + r holds row
+// 16*rb + r, k = 32*g + 8*oct .. +8.  A workgroup moves one row block x 16 groups through LDS:
 // waves read 1 KB runs of a row and write whole 1 KB units.
 constexpr int kStageGroups = 16;                       // scale groups per workgroup
 constexpr int kStagePitch = kStageGroups * 4 + 1;      // 16 B slots per LDS row (odd: no bank conflicts)
 
-// NORM: RMSNorm folded in.  x * gamma is formed in fp32 and rounded once to the operand type
-// (XBF: the input is bf16; WIDEN: bf16 in, f16 * 2^-4 out); the squares of the unscaled row are
-// summed per (row, workgroup) in a fixed butterfly order into ssq_part[row * gridDim.y + blockIdx.y].
-// XT: element type of X (0 f16, 1 bf16, 2 f32).  fp32 rows are rounded once to f16 * 2^-4 (WIDEN),
-// two 16 B chunks in, one out.
-template <bool WIDEN, int XT, bool NORM>
+// NORM: RMSNorm folded in.  x * gamma is formed in fp32 and rounded once to the operand type (XBF:
+// bf16, else f16); the squares of the unscaled row are summed per (row, workgroup) in a fixed
+// butterfly order into ssq_part[row * gridDim.y + blockIdx.y].
+template <bool XBF, bool NORM>
 __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict__ src, u32x4_t* __restrict__ dst, int M, int K8,
                                                       Epilogue epi, float* __restrict__ ssq_part)
 {
-    constexpr bool XBF = XT == 1;
-    static_assert(XT != 2 || WIDEN, "fp32 activations are staged as prescaled f16");
     __shared__ u32x4_t tile[16 * kStagePitch];
     const int rb = blockIdx.x;
     const int c0 = blockIdx.y * (kStageGroups * 4);     // first 16 B chunk of the row handled here
@@ -577,26 +569,7 @@ __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict_
         const int row = rb * 16 + r;
         Frag16 a;
         a.u = (u32x4_t){0u, 0u, 0u, 0u};
-        float xf[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};       // XT == 2: the chunk as loaded
-        if (row < M && c < K8) {
-            if (XT == 2) {
-                const u32x4_t lo = src[((int64_t)row * K8 + c) * 2], hi = src[((int64_t)row * K8 + c) * 2 + 1];
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    xf[e] = __builtin_bit_cast(float, (uint32_t)lo[e]);
-                    xf[4 + e] = __builtin_bit_cast(float, (uint32_t)hi[e]);
-                }
-            } else {
-                a.u = src[(int64_t)row * K8 + c];
-            }
-        }
-        if (XT == 2 && !NORM) {
-#pragma unroll
-            for (int p = 0; p < 4; p++) {
-                const half2_t h = {(_Float16)(xf[2 * p] * 0.0625f), (_Float16)(xf[2 * p + 1] * 0.0625f)};
-                a.u[p] = as_u32(h);
-            }
-        }
+        if (row < M && c < K8) a.u = src[(int64_t)row * K8 + c];
         if (NORM) {
             float sq = 0.f;
             if (c < K8) {
@@ -605,10 +578,7 @@ __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict_
 #pragma unroll
                 for (int p = 0; p < 4; p++) {
                     float v0, v1;
-                    if (XT == 2) {
-                        v0 = xf[2 * p];
-                        v1 = xf[2 * p + 1];
-                    } else if (XBF) {
+                    if (XBF) {
                         v0 = __builtin_bit_cast(float, a.u[p] << 16);
                         v1 = __builtin_bit_cast(float, a.u[p] & 0xffff0000u);
                     } else {
@@ -617,10 +587,9 @@ __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict_
                         v1 = (float)h.y;
                     }
                     sq = fmaf(v1, v1, fmaf(v0, v0, sq));
-                    const float sc = WIDEN ? 0.0625f : 1.0f;
-                    v0 *= g[2 * p] * sc;
-                    v1 *= g[2 * p + 1] * sc;
-                    if (XBF && !WIDEN) {
+                    v0 *= g[2 * p];
+                    v1 *= g[2 * p + 1];
+                    if (XBF) {
                         a.u[p] = pack_bf16x2(v0, v1);
                     } else {
                         const half2_t h = {(_Float16)v0, (_Float16)v1};
@@ -631,8 +600,6 @@ __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict_
 #pragma unroll
             for (int off = 32; off >= 1; off >>= 1) sq += __shfl_xor(sq, off, 64);
             if ((t & 63) == 0) ssq_part[(int64_t)row * gridDim.y + blockIdx.y] = sq;      // (rows past M: zeros, never read)
-        } else if (WIDEN && XT == 1) {
-            a = bf16_to_f16_frag(a);
         }
         tile[r * kStagePitch + (t & 63)] = a.u;
     }
@@ -646,6 +613,148 @@ __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict_
     }
 }
 
+// The same restaging for FAST mode when the activations are not f16 (bf16 or fp32 in, f16 operands
+// out), with a power-of-two scale PER ROW: a workgroup owns four rows, wave r owns row r.  First
+// the wave reads its row for the largest magnitude (of x, or of x * gamma with a folded norm,
+// whose sum of squares it also takes), picks the power of two s that brings it just under 2^14 and
+// leaves 1 / s in `unscale` for the multiply's epilogue; then the four rows go through LDS in
+// pieces of 512 k, every value multiplied by its row's s on the way to f16, and leave as 64-byte
+// runs (four neighbouring rows of one k octet in operand order).
+// Whatever the magnitude of a row, its largest element lands in [2^13, 2^14) and elements down to
+// 2^-27 of it stay normal f16 numbers.  Rows of up to CH * 512 elements stay in registers between
+// the two steps (CH chunks of 8 values per lane, all requested at once); longer rows are read
+// again, CH chunks at a time (the second read hits the L2).
+template <int XT>
+struct RowChunk {                 // 8 consecutive activations of a row as loaded
+    u32x4_t v[XT == 2 ? 2 : 1];
+};
+
+template <int XT>
+__device__ __forceinline__ RowChunk<XT> load_row_chunk(const void* src, int64_t row, int K, int c)
+{
+    RowChunk<XT> o;
+    if (XT == 2) {
+        const u32x4_t* p = reinterpret_cast<const u32x4_t*>(reinterpret_cast<const float*>(src) + row * K + c * 8);
+        o.v[0] = p[0];
+        o.v[XT == 2 ? 1 : 0] = p[1];
+    } else {
+        o.v[0] = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const uint16_t*>(src) + row * K + c * 8);
+    }
+    return o;
+}
+
+template <int XT>
+__device__ __forceinline__ void row_chunk_values(const RowChunk<XT>& c, float v[8])
+{
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        if (XT == 2) {
+            v[e] = __builtin_bit_cast(float, (uint32_t)c.v[0][e]);
+            v[4 + e] = __builtin_bit_cast(float, (uint32_t)c.v[XT == 2 ? 1 : 0][e]);
+        } else {
+            v[2 * e] = __builtin_bit_cast(float, c.v[0][e] << 16);
+            v[2 * e + 1] = __builtin_bit_cast(float, c.v[0][e] & 0xffff0000u);
+        }
+    }
+}
+
+template <int XT, bool NORM, int CH>
+__global__ __launch_bounds__(256) void stage_rows_kernel(const void* __restrict__ src, u32x4_t* __restrict__ dst, int M, int K,
+                                                         Epilogue epi, float* __restrict__ ssq, float* __restrict__ unscale)
+{
+    static_assert(XT == 1 || XT == 2, "bf16 or fp32 activations");
+    __shared__ u32x4_t tile[2][4 * kStagePitch];
+    const int rb = blockIdx.x >> 2, r0 = (blockIdx.x & 3) * 4;          // row block, first of this workgroup's rows in it
+    const int t = threadIdx.x, lane = t & 63, r = t >> 6;
+    const int64_t row = min(rb * 16 + r0 + r, M - 1);      // (rows past M repeat the last one and are never read back)
+    const int K8 = K >> 3, G = K8 >> 2;
+    const bool resident = K8 <= 64 * CH;
+
+    // ---- the row's largest magnitude (and sum of squares)
+    RowChunk<XT> keep[CH];
+    float amax = 0.f, sq = 0.f;
+    for (int c0 = 0; c0 < K8; c0 += 64 * CH) {
+#pragma unroll
+        for (int i = 0; i < CH; i++)
+            if (c0 + i * 64 < K8) keep[i] = load_row_chunk<XT>(src, row, K, min(c0 + i * 64 + lane, K8 - 1));
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const int c = c0 + i * 64 + lane;
+            float v[8];
+            if (c < K8) {
+                row_chunk_values<XT>(keep[i], v);
+                if (NORM) {
+                    float g[8];
+                    load_gamma8_g(epi.gamma, epi.gamma_dt, c * 8, g);
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        sq = fmaf(v[e], v[e], sq);
+                        v[e] *= g[e];
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[e]));
+            }
+        }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+        if (NORM) sq += __shfl_xor(sq, off, 64);
+    }
+    // amax = f * 2^e with f in [0.5, 1): s = 2^(14 - e) puts it in [2^13, 2^14); zero, Inf and NaN rows keep s = 1
+    float s = 1.0f;
+    if (amax > 0.f && amax < __builtin_inff()) {
+        int e;
+        (void)frexpf(amax, &e);
+        s = ldexpf(1.0f, 14 - e);
+    }
+    if (lane == 0 && rb * 16 + r0 + r < M) {
+        unscale[row] = 1.0f / s;
+        if (NORM) ssq[row] = sq;
+    }
+
+    // ---- scale, round to f16, through LDS into operand order (two tiles: one barrier per piece)
+    auto convert = [&](const RowChunk<XT>& ch, int c) {
+        float v[8];
+        row_chunk_values<XT>(ch, v);
+        if (NORM) {
+            float g[8];
+            load_gamma8_g(epi.gamma, epi.gamma_dt, min(c, K8 - 1) * 8, g);
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[e] *= g[e];
+        }
+        Frag16 a;
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const half2_t h = {(_Float16)(v[2 * p] * s), (_Float16)(v[2 * p + 1] * s)};
+            a.u[p] = as_u32(h);
+        }
+        return a.u;
+    };
+    const int gl = t >> 4, oct = (t >> 2) & 3, rr = t & 3;  // when writing out: group within the piece, k octet, row
+    int piece = 0;
+    for (int c0 = 0; c0 < K8; c0 += 64 * CH) {
+        if (!resident) {
+#pragma unroll
+            for (int i = 0; i < CH; i++)
+                if (c0 + i * 64 < K8) keep[i] = load_row_chunk<XT>(src, row, K, min(c0 + i * 64 + lane, K8 - 1));
+        }
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const int cb = c0 + i * 64;
+            if (cb < K8) {                                   // (uniform over the workgroup)
+                u32x4_t* tl = tile[piece & 1];
+                tl[r * kStagePitch + lane] = convert(keep[i], cb + lane);
+                __syncthreads();
+                const int g = (cb >> 2) + gl;
+                if (g < G) dst[((int64_t)rb * G + g) * 64 + oct * 16 + r0 + rr] = tl[rr * kStagePitch + gl * 4 + oct];
+                piece++;
+            }
+        }
+    }
+}
+
 }  // namespace
 
 hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
@@ -654,22 +763,25 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
 {
     if (xdt == kF32 && exact) return hipErrorNotSupported;   // api.hip walks exact fp32 prefill through the decode kernel
     // FAST multiplies in f16: bf16 activations are widened, fp32 activations rounded to f16
-    // (both with a 2^-4 prescale that is undone in the epilogue)
+    // (both behind a power-of-two scale per row that the epilogue undoes)
     const bool widen = !exact && xdt != kF16;
-    const float out_scale = widen ? 16.0f : 1.0f;
+    const float out_scale = 1.0f;
     const int kdt = widen ? kF16 : xdt;
     // Rows are staged through the workspace in chunks that fit it; work on one stream is
     // ordered, so a chunk's multiply is done before the next chunk overwrites the stage.
     // First half of the workspace: staged X; second half: partial sums of a K split.
     const size_t half = workspace_bytes / 2;
     float* part = reinterpret_cast<float*>(static_cast<char*>(workspace) + half);
-    // The last MiB of the first half: per-row partial sums of squares of a folded RMSNorm
-    // (rows of a chunk x K / 512 floats: at most half / 256 bytes).
+    // The last MiB of the first half: per-row statistics - partial sums of squares of a folded
+    // RMSNorm (rows of a chunk x K / 512 floats: less than half / 256 bytes) and, in its last
+    // quarter, the per-row power of two of widened activations (at most 65536 rows per chunk).
     const size_t stats_bytes = (size_t)1 << 20;
     if (!workspace || half <= stats_bytes) return hipErrorOutOfMemory;
     float* ssq_part = reinterpret_cast<float*>(static_cast<char*>(workspace) + half - stats_bytes);
+    float* unscale = reinterpret_cast<float*>(static_cast<char*>(workspace) + half - stats_bytes / 4);
     const int64_t row_bytes = (int64_t)w.K * (xdt == kF32 ? 4 : 2);        // a row of the caller's X
-    const int64_t max_rows = (int64_t)((half - stats_bytes) / (size_t)(w.K * 2)) / 256 * 256;    // staged rows are 16-bit
+    const int64_t max_rows =
+        std::min<int64_t>(65536, (int64_t)((half - stats_bytes) / (size_t)(w.K * 2)) / 256 * 256);    // staged rows are 16-bit
     if (max_rows < 256) return hipErrorOutOfMemory;
     const size_t ysize = ydt == kF32 ? 4 : 2;
     for (int64_t m_lo = 0; m_lo < M; m_lo += max_rows) {
@@ -682,18 +794,33 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
         const int K8 = w.K / 8;
         const dim3 grid((unsigned)((mc + 15) / 16), (unsigned)((K8 / 4 + kStageGroups - 1) / kStageGroups));
         u32x4_t* xst = reinterpret_cast<u32x4_t*>(workspace);
-        const NormStats ns = {ssq_part, (int)grid.y};
-        if (epi.gamma) {
-            if (xdt == kF32) hipLaunchKernelGGL((stage_x_kernel<true, 2, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
-            else if (widen) hipLaunchKernelGGL((stage_x_kernel<true, 1, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
-            else if (xdt == kBF16) hipLaunchKernelGGL((stage_x_kernel<false, 1, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
-            else hipLaunchKernelGGL((stage_x_kernel<false, 0, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
-        } else if (xdt == kF32) {
-            hipLaunchKernelGGL((stage_x_kernel<true, 2, false>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
-        } else if (widen) {
-            hipLaunchKernelGGL((stage_x_kernel<true, 1, false>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+        NormStats ns = {ssq_part, (int)grid.y, nullptr};
+        if (widen) {
+            // per-row scaled f16 operands; one sum of squares per row
+            ns = NormStats{ssq_part, 1, unscale};
+            const dim3 rgrid((unsigned)((mc + 15) / 16) * 4);
+            // chunks of 512 k a lane keeps in registers: the whole row when it has at most 16384 (bf16) or
+            // 8192 (fp32) elements
+            const int batches = (K8 + 63) / 64;
+#define CYBQ_STAGE_ROWS(XT, NORM, CH) \
+    hipLaunchKernelGGL((stage_rows_kernel<XT, NORM, CH>), rgrid, dim3(256), 0, st, xs, xst, mc, w.K, epi, ssq_part, unscale)
+#define CYBQ_STAGE_ROWS_CH(XT, NORM, C1, C2, C3)              \
+    do {                                                      \
+        if (batches <= C1) CYBQ_STAGE_ROWS(XT, NORM, C1);     \
+        else if (batches <= C2) CYBQ_STAGE_ROWS(XT, NORM, C2); \
+        else CYBQ_STAGE_ROWS(XT, NORM, C3);                   \
+    } while (0)
+            if (xdt == kF32 && epi.gamma) CYBQ_STAGE_ROWS_CH(2, true, 4, 8, 16);
+            else if (xdt == kF32) CYBQ_STAGE_ROWS_CH(2, false, 4, 8, 16);
+            else if (epi.gamma) CYBQ_STAGE_ROWS_CH(1, true, 8, 16, 32);
+            else CYBQ_STAGE_ROWS_CH(1, false, 8, 16, 32);
+#undef CYBQ_STAGE_ROWS_CH
+#undef CYBQ_STAGE_ROWS
+        } else if (epi.gamma) {
+            if (xdt == kBF16) hipLaunchKernelGGL((stage_x_kernel<true, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+            else hipLaunchKernelGGL((stage_x_kernel<false, true>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
         } else {
-            hipLaunchKernelGGL((stage_x_kernel<false, 0, false>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
+            hipLaunchKernelGGL((stage_x_kernel<false, false>), grid, dim3(256), 0, st, xs, xst, mc, K8, epi, ssq_part);
         }
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;

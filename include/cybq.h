@@ -78,8 +78,10 @@ typedef enum cybq_dtype { CYBQ_F32 = 0, CYBQ_F16 = 1, CYBQ_BF16 = 2 } cybq_dtype
  * operator's 1e-3 relative-L2 tolerance; the decode kernels (M <= 32) are always exact.
  *   FAST   (default) one f16 MFMA per 32-group; the weight operand is
  *          round_f16(scale * q), relative error <= 2^-11 per weight (about 2e-4
- *          relative L2 on y).  bf16 activations are widened to f16 after a 2^-4
- *          prescale (undone on output): |x| must stay below 2^20.
+ *          relative L2 on y).  bf16 and fp32 activations become f16 operands behind a
+ *          power-of-two scale per row (taken from the row's largest magnitude and undone on
+ *          output): rows of any finite magnitude keep that accuracy; within a row, elements
+ *          below 2^-27 of the largest lose bits.  f16 activations are used as they are.
  *   EXACT  two MFMAs per 32-group in the activation type; scale * q is split
  *          without loss into a high and a low 16-bit operand, so y differs from
  *          the fp32 CPU path only by accumulation order.  Half the throughput. */
@@ -113,7 +115,10 @@ const char* cybq_version(void);
  * model-switch time (use_model, lazy load - shell/src/worlds/models/mod.rs:7-8,386;
  * "all conversion happens at import" - decide/pipeline.md:59: the repack to the
  * device layout happens here, once, never in cybq_matmul).
- * `q` / `scales` are host pointers (see cybq_layout); requires K % 32 == 0. */
+ * `q` / `scales` are host pointers (see cybq_layout); requires K % 32 == 0.
+ * A tensor with a scale so large that |scale| * 8 (Q4) or |scale| * 128 (Q8) leaves f16's range
+ * (or a non-finite scale) is marked at upload and served by the decode kernels for every M: the
+ * prefill kernels form scale * q in f16. */
 int cybq_weight_upload(cybq_ctx* ctx, cybq_quant quant, cybq_layout layout,
                        int64_t N, int64_t K, const void* q, const void* scales,
                        cybq_weight** out);
@@ -231,7 +236,12 @@ int cybq_dequant(cybq_ctx* ctx, const cybq_weight* w, float* out, void* stream);
 int cybq_quantize(cybq_ctx* ctx, cybq_quant quant, const float* src, int64_t N, int64_t K,
                   void* q_out, void* scales_out, void* stream);
 /* Builds a weight handle from PLANAR buffers that already live on the device
- * (the output of cybq_quantize); stream-ordered, allocates the handle. */
+ * (the output of cybq_quantize); stream-ordered, allocates the handle.  The buffers must stay
+ * valid until the work queued on `stream` has run; other calls that read the new weight
+ * (cybq_weight_clone, cybq_weight_fuse_pairs, a matmul on another stream) must be ordered after it
+ * by the caller.  The scales are not inspected here: they must keep |scale| * 8 (Q4) or
+ * |scale| * 128 (Q8) within f16's range, which the output of cybq_quantize does for finite
+ * weights up to 65504. */
 int cybq_weight_from_device(cybq_ctx* ctx, cybq_quant quant, int64_t N, int64_t K,
                             const void* q_dev, const void* scales_dev, void* stream,
                             cybq_weight** out);

@@ -157,16 +157,19 @@ public:
         auto xi = edges.find(node.x), yi = edges.find(node.y);
         if (xi == edges.end() || yi == edges.end()) return fail(CYBQ_ERR_INVALID, "edge not bound");
         if (xi->second.rows < node.M || yi->second.rows < node.M) return fail(CYBQ_ERR_SHAPE, "edge has too few rows");
+        if (Status s = check_cols(*w, node, xi->second, yi->second); !s) return s;
         const void* res = nullptr;
         if (node.epilogue == CYBQ_EPI_ADD) {
             auto ri = edges.find(node.residual);
-            if (ri == edges.end() || ri->second.dtype != yi->second.dtype || ri->second.rows < node.M)
-                return fail(CYBQ_ERR_INVALID, "residual edge not bound or of another type");
+            if (ri == edges.end() || ri->second.dtype != yi->second.dtype || ri->second.rows < node.M ||
+                ri->second.cols != yi->second.cols)
+                return fail(CYBQ_ERR_INVALID, "residual edge not bound, of another type or of another shape");
             res = ri->second.ptr;
         }
         if (!node.norm_gamma.empty()) {
             auto gi = edges.find(node.norm_gamma);
             if (gi == edges.end()) return fail(CYBQ_ERR_INVALID, "gamma edge not bound");
+            if (gi->second.rows * gi->second.cols != w->cols()) return fail(CYBQ_ERR_SHAPE, "gamma must hold K elements");
             return matmul_norm(*w, xi->second.ptr, xi->second.dtype, node.M, gi->second.ptr, gi->second.dtype, node.norm_eps,
                                yi->second.ptr, yi->second.dtype, node.epilogue, res, stream);
         }
@@ -183,14 +186,17 @@ public:
         std::vector<const void*> xs, rs;
         std::vector<void*> ys;
         std::vector<int> es;
-        const Edge& x0 = edges.at(nodes[0].x);
-        const Edge& y0 = edges.at(nodes[0].y);
+        auto x0i = edges.find(nodes[0].x), y0i = edges.find(nodes[0].y);
+        if (x0i == edges.end() || y0i == edges.end()) return fail(CYBQ_ERR_INVALID, "unresolved node '" + nodes[0].w + "'");
+        const Edge &x0 = x0i->second, &y0 = y0i->second;
         for (const auto& n : nodes) {
             const Weight* w = find(n.w);
             auto xi = edges.find(n.x), yi = edges.find(n.y);
             if (!w || xi == edges.end() || yi == edges.end()) return fail(CYBQ_ERR_INVALID, "unresolved node '" + n.w + "'");
             if (xi->second.dtype != x0.dtype || yi->second.dtype != y0.dtype || n.M != nodes[0].M)
                 return fail(CYBQ_ERR_INVALID, "run_all needs one M and one dtype pair");
+            if (xi->second.rows < n.M || yi->second.rows < n.M) return fail(CYBQ_ERR_SHAPE, "edge has too few rows");
+            if (Status s = check_cols(*w, n, xi->second, yi->second); !s) return s;
             if (!n.norm_gamma.empty()) return fail(CYBQ_ERR_INVALID, "run_all does not take folded norms: use run()");
             const void* res = nullptr;
             if (n.epilogue == CYBQ_EPI_ADD) {
@@ -209,6 +215,15 @@ public:
     }
 
 private:
+    // an edge's columns must be what the weight reads (K) and writes (N, or N / 2 behind SwiGLU)
+    Status check_cols(const Weight& w, const QMatMulNode& node, const Edge& x, const Edge& y)
+    {
+        if (!x.ptr || !y.ptr) return fail(CYBQ_ERR_INVALID, "edge without a buffer");
+        const int64_t n_out = node.epilogue == CYBQ_EPI_SWIGLU ? w.rows() / 2 : w.rows();
+        if (x.cols != w.cols() || y.cols != n_out)
+            return fail(CYBQ_ERR_SHAPE, "edges of node '" + node.w + "' do not have the weight's K / N columns");
+        return Status{};
+    }
     Status wrap(int rc)
     {
         Status s;

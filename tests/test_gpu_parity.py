@@ -381,23 +381,58 @@ def test_prefill_ragged_shapes(backend, oracle, prefill_mode, shape):
         assert oracle.rel_l2(y, oracle.matmul_f64(q, s, x.float().cpu().numpy())) < _bar(prefill_mode)
 
 
-def test_prefill_fast_mode_activation_range(backend, oracle):
-    # FAST widens bf16 activations to f16 behind a 2^-4 prescale: large outliers
-    # (up to 2^20) and tiny values must both survive
+@pytest.mark.parametrize("xdt", ["bf16", "f32"])
+def test_prefill_fast_mode_activation_range(backend, oracle, xdt):
+    # FAST turns bf16 / fp32 activations into f16 operands behind a power-of-two scale per row:
+    # rows of any magnitude keep the mode's accuracy, outliers far beyond f16's range survive
     N, K = 128, 1024
     q, s = _quant(oracle, 4, N, K)
     qw = backend.upload_quantized(q, s, 4)
-    x = _x(40, K, "bf16")
+    x = _x(40, K, xdt)
     x[0, 5] = 3.0e5
     x[1, 77] = -9.0e5
     x[2] *= 1e-3
     x[3] *= 300.0
+    x[4] *= 1e-4
+    x[5] *= 1e-5
+    x[6] *= 1e-6
+    x[7] *= 1e-12
+    x[8] *= 1e12
+    x[9] = 0.0
+    x[10, 1:] = 0.0
     backend.set_prefill_mode("fast")
     y = _run(backend, qw, x).cpu().numpy()
     assert np.isfinite(y).all()
+    assert not y[9].any()
     ref = oracle.matmul_f64(q, s, x.float().cpu().numpy())
-    for rows in ([0], [1], [2], [3], list(range(4, 40))):
+    for rows in ([0], [1], [2], [3], [4], [5], [6], [7], [8], [10], list(range(11, 40))):
         assert oracle.rel_l2(y[rows], ref[rows]) < FAST, rows
+    # a folded norm sees the same rows (gamma of mixed magnitudes)
+    gamma = torch.from_numpy(np.abs(synth.activations(22, 1, K))[0] * 10.0 + 1e-3).cuda()
+    yn = torch.empty((40, N), dtype=torch.float32, device="cuda")
+    backend.matmul_norm(qw, x, gamma, 1e-30, yn)           # 40 rows: the prefill kernel
+    torch.cuda.synchronize()
+    xf = x[:9].double().cpu().numpy()
+    rstd = 1.0 / np.sqrt((xf ** 2).mean(axis=1, keepdims=True) + 1e-30)
+    refn = oracle.matmul_f64(q, s, (xf * gamma.double().cpu().numpy()).astype(np.float32)) * rstd
+    for r in range(9):
+        assert oracle.rel_l2(yn[r:r + 1].cpu().numpy(), refn[r:r + 1]) < 2 * FAST, r
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_scales_beyond_f16_products(backend, oracle, bits):
+    """scale * q would leave f16's range: such tensors take the decode kernels (scale in fp32) on both
+    sides of the prefill boundary."""
+    N, K = 64, 256
+    q, s = _quant(oracle, bits, N, K)
+    s = s.copy()
+    s[::3, ::2] = np.float16(30000.0).view(np.uint16)
+    qw = backend.upload_quantized(q, s, bits, formats.BLOCK_AOS)
+    for M in (4, 32, 33, 100):
+        x = _x(M, K, "f16")
+        y = _run(backend, qw, x).cpu().numpy()
+        assert np.isfinite(y).all(), M
+        assert oracle.rel_l2(y, oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT, M
 
 
 def test_prefill_rows_agree_with_decode_rows(backend, oracle, prefill_mode):
@@ -771,12 +806,20 @@ def test_error_codes(backend, oracle):
     with pytest.raises(CybqError) as e:
         backend.upload(5, formats.PLANAR, 16, 64, formats.pack_planar(q, 4), s)       # bad quant
     assert e.value.status == -1
+    with pytest.raises(CybqError) as e:
+        backend.upload(4, formats.PLANAR, 32, 64, formats.pack_planar(q, 4), s)       # buffers of a 16-row tensor
+    assert e.value.status == -2
     qw = backend.upload_quantized(q, s, 4)
     x = _x(2, 64, "f16")
     y = torch.empty((2, 16), dtype=torch.float32, device="cuda")
     with pytest.raises(CybqError) as e:
         backend.matmul(qw, x, y, M=0)
     assert e.value.status == -2
+    # the host wrapper refuses tensors the library could only see as raw pointers of the wrong size
+    for bad_x, bad_y in ((x[:1], y), (x, y[:1]), (x.t().contiguous().t(), y), (x.cpu(), y)):
+        with pytest.raises(CybqError) as e:
+            backend.matmul(qw, bad_x, bad_y, M=2)
+        assert e.value.status in (-1, -2)
     buf = torch.empty(2 * 64 + 8, dtype=torch.float16, device="cuda")
     with pytest.raises(CybqError) as e:
         backend.matmul(qw, buf.data_ptr() + 2, y, M=2, xdt=1)                         # misaligned x
