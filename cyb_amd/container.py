@@ -164,7 +164,7 @@ class Container:
             raise ContainerError("frontmatter lists no [[files]]")
         pos = first
         seen_binary = False
-        for ent in files:
+        for idx, ent in enumerate(files):
             name = ent.get("name")
             if not isinstance(name, str):
                 raise ContainerError("a [[files]] entry has no name")
@@ -182,7 +182,14 @@ class Container:
                 pos = body + n
             else:
                 if seen_binary:
-                    raise ContainerError(f"text part {name!r} after a binary part")
+                    # text goes before binary; the one exception the spec draws is a last part without
+                    # a size, which simply runs to the end of the file
+                    # (/root/reference/reference/format.md:24-31, "binary file (until EOF)")
+                    if idx != len(files) - 1:
+                        raise ContainerError(f"text part {name!r} after a binary part")
+                    self.parts[name] = (body, len(mm) - body)
+                    pos = len(mm)
+                    continue
                 nxt = self._find_delim(body)
                 end = nxt if nxt >= 0 else len(mm)
                 self.parts[name] = (body, end - body)

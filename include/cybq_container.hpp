@@ -194,10 +194,13 @@ private:
         if (!parse_toml_subset(reinterpret_cast<const char*>(map_), first, front, err)) return bad("frontmatter " + err);
         size_t pos = first;
         bool seen_binary = false, any = false;
+        size_t files_left = 0;
+        for (const auto& t : front) files_left += t.name == "files";
         for (const auto& t : front) {
             if (t.name == "cyb") { auto it = t.str.find("name"); if (it != t.str.end()) name_ = it->second; }
             if (t.name != "files") continue;
             any = true;
+            files_left--;
             auto nm = t.str.find("name");
             if (nm == t.str.end()) return bad("a [[files]] entry has no name");
             std::string head = "~~~" + nm->second + "\n";
@@ -212,7 +215,14 @@ private:
                 parts_[nm->second] = {body, (size_t)n};
                 pos = body + (size_t)n;
             } else {
-                if (seen_binary) return bad("text part '" + nm->second + "' after a binary part");
+                if (seen_binary) {
+                    // text goes before binary; a LAST part without a size runs to the end of the file
+                    // (/root/reference/reference/format.md:24-31)
+                    if (files_left != 0) return bad("text part '" + nm->second + "' after a binary part");
+                    parts_[nm->second] = {body, size_ - body};
+                    pos = size_;
+                    continue;
+                }
                 size_t end = find_delim(body);
                 parts_[nm->second] = {body, end - body};
                 pos = end;

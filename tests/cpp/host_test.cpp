@@ -3,6 +3,7 @@
 // with expected outputs written by the Python test (which gets them from the oracle).
 //
 //   host_test --parse FILE                     no GPU: print the tensor index
+//   host_test --parts FILE NAME...             no GPU: length and FNV-1a hash of the named parts
 //   host_test --run FILE X.bin Y.bin M [exact] GPU: X is f16 [M,K] (K of the first tensor),
 //                                              Y is f64 [tensors][M,N]; prints rel-L2 per tensor
 #include <hip/hip_runtime.h>
@@ -29,6 +30,17 @@ int main(int argc, char** argv)
     cybq::Container c;
     cybq::Status s = c.open(argv[2]);
     if (!s) { std::printf("ERROR %d %s\n", s.code, s.text.c_str()); return 1; }
+    if (!std::strcmp(argv[1], "--parts")) {          // no GPU: the named parts, by name
+        std::printf("name %s\n", c.name().c_str());
+        for (int i = 3; i < argc; i++) {
+            auto p = c.part(argv[i]);
+            if (!p.first) { std::printf("part %s missing\n", argv[i]); continue; }
+            unsigned long long sum = 1469598103934665603ull;     // FNV-1a of the bytes
+            for (size_t j = 0; j < p.second; j++) sum = (sum ^ p.first[j]) * 1099511628211ull;
+            std::printf("part %s %zu %016llx\n", argv[i], p.second, sum);
+        }
+        return 0;
+    }
     if (!std::strcmp(argv[1], "--parse")) {
         std::printf("name %s\n", c.name().c_str());
         for (const auto& t : c.tensors())

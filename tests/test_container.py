@@ -117,3 +117,72 @@ def test_cpp_reader_matches_python(tmp_path):
     for line, r in zip(out[1:], c.tensors()):
         assert line == f"tensor {r.name} {r.kind} {r.layout} {r.shape[0]} {r.shape[1]} {r.offset}"
     c.close()
+
+
+# ---- committed fixtures (tests/golden/, written by tests/golden/make_fixtures.py) -----------------
+
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+def _fnv1a(data: bytes) -> str:
+    h = 1469598103934665603
+    for b in data:
+        h = ((h ^ b) * 1099511628211) & 0xFFFFFFFFFFFFFFFF
+    return f"{h:016x}"
+
+
+def _cpp_parts(path, names):
+    out = subprocess.run([HOST_TEST, "--parts", path] + names, capture_output=True, text=True, check=True).stdout.split("\n")
+    return out[0], {l.split()[1]: (int(l.split()[2]), l.split()[3]) for l in out[1:] if l.startswith("part ") and "missing" not in l}
+
+
+def test_fixture_spec_example_is_read_by_both_readers():
+    """The format spec's own example (/root/reference/reference/format.md:40-72), assembled into a file."""
+    path = os.path.join(GOLDEN, "spec_example.cyb")
+    c = container.Container(path)
+    assert c.name == "qwen3-0.6b-abliterated"
+    assert c.front["cyb"]["types"] == ["model"]
+    assert list(c.parts) == ["config", "program", "weights", "image"]           # order of [[files]]
+    assert c.text("config") == 'architecture = "Qwen3ForCausalLM"\nhidden_size = 1024\n\n'
+    assert c.text("program") == "transformer_decoder { layers: 28 }\n\n"
+    w = bytes(c.view("weights"))
+    assert len(w) == c.front["files"][2]["size"] and b"\n~~~config\n" in w and b"\r\n" in w     # never scanned
+    img = bytes(c.view("image"))
+    assert img.startswith(b"\x89IMG\r\n") and len(img) == 40                      # last part: runs to the end of the file
+    raw = open(path, "rb").read()
+    assert raw.endswith(img)
+    with pytest.raises(container.ContainerError):
+        c.tensors()                                                              # not a tensor container: said so, not guessed
+    if os.path.exists(HOST_TEST):
+        name, parts = _cpp_parts(path, ["config", "program", "weights", "image", "nope"])
+        assert name == "name qwen3-0.6b-abliterated"
+        assert parts == {n: (c.parts[n][1], _fnv1a(bytes(c.view(n)))) for n in ("config", "program", "weights", "image")}
+    c.close()
+
+
+def test_fixture_of_the_reference_writer_is_read_by_both_readers():
+    """The byte stream the reference's own .cyb writer emits
+    (/root/reference/shell/src/worlds/snapshot.rs:71-103): frontmatter, ~~~config, ~~~cyberlinks + size bytes."""
+    path = os.path.join(GOLDEN, "snapshot_writer.graph")
+    raw = open(path, "rb").read()
+    c = container.Container(path)
+    assert c.name == "cyb-snapshot" and c.front["cyb"]["types"] == ["graph"]
+    assert [f["format"] for f in c.front["files"]] == ["toml", "records"]
+    cfg = c.text("config")
+    assert cfg.startswith('chain_id = "cyb-local"\nblock = 0\n') and cfg.endswith("weight = 1\n")
+    rec = bytes(c.view("cyberlinks"))
+    assert len(rec) == 3 * 96 == c.front["files"][1]["size"] and raw.endswith(rec) and b"\n~~~" in rec
+    if os.path.exists(HOST_TEST):
+        name, parts = _cpp_parts(path, ["config", "cyberlinks"])
+        assert name == "name cyb-snapshot"
+        assert parts == {"config": (len(cfg.encode()), _fnv1a(cfg.encode())), "cyberlinks": (len(rec), _fnv1a(rec))}
+    c.close()
+
+
+def test_fixtures_match_their_generator():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(GOLDEN, "make_fixtures.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    assert open(os.path.join(GOLDEN, "spec_example.cyb"), "rb").read() == mod.spec_example()
+    assert open(os.path.join(GOLDEN, "snapshot_writer.graph"), "rb").read() == mod.snapshot_writer()

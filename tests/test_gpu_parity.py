@@ -284,6 +284,19 @@ def test_decode_lds_kernel_largest_request(backend, oracle):
         backend.set_prefill_mode("fast")
 
 
+def test_known_answers_from_the_committed_fixture(backend):
+    """tests/golden/matmul_small.json through the C ABI: both interchange layouts, f16 activations."""
+    from tests.test_oracle_matmul import _golden_cases
+    for name, bits, q, s, x, want in _golden_cases():
+        for layout in (formats.PLANAR, formats.BLOCK_AOS):
+            qw = backend.upload_quantized(q, s, bits, layout)
+            xt = torch.from_numpy(x).cuda().to(torch.float16)
+            y = _run(backend, qw, xt).double().cpu().numpy()
+            assert np.linalg.norm(y - want) <= TIGHT * np.linalg.norm(want), (name, layout)
+            if name == "by_hand_q4":
+                assert np.allclose(y, [[16.0, 32.0, 48.0, 64.0]], rtol=1e-6)
+
+
 def test_decode_special_cases(backend, oracle):
     N, K = 64, 256
     ones = np.full((N, K // 32), 0x3C00, np.uint16)
@@ -1029,6 +1042,44 @@ def test_calls_can_be_captured_in_a_graph(backend, oracle, M, xdt):
         torch.cuda.synchronize()
         assert torch.equal(h, h0) and torch.equal(y, y0)
         assert (x1.float() @ x1.float().T).sum().isfinite()          # eager work between replays
+
+
+def test_first_call_of_a_kernel_may_sit_inside_a_capture(oracle):
+    """No launch path changes a function attribute (cybq_init raised every kernel's dynamic LDS limit): a
+    fresh context may record calls whose kernels it has never launched - kernels that need more than the
+    default 64 KB of LDS among them - and the replay matches an eager run made afterwards."""
+    from cyb_amd import Backend
+    be = Backend(0)
+    try:
+        be.set_prefill_mode("exact")                       # EXACT prefill tiles stage 112 - 128 KB of operands in LDS
+        N, K, M = 208, 2176, 77                            # shapes no other test uses
+        q, s = _quant(oracle, 8, N, K, cfg=91)
+        qw = be.upload_quantized(q, s, 8, formats.BLOCK_AOS)
+        x = _x(M, K, "bf16", cfg=92)
+        x32 = _x(12, K, "f32", cfg=93)                     # LDS decode kernel, fp32 rows: its largest LDS request
+        y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        y32 = torch.zeros((12, N), dtype=torch.float32, device="cuda")
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            st = torch.cuda.current_stream().cuda_stream
+            be.matmul(qw, x, y, stream=st)
+            be.matmul(qw, x32, y32, stream=st)
+        for _ in range(2):
+            y.zero_()
+            y32.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert oracle.rel_l2(y.cpu().numpy(), oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT
+            assert oracle.rel_l2(y32.cpu().numpy(), oracle.matmul_f64(q, s, x32.cpu().numpy())) < TIGHT
+        ye = torch.zeros_like(y)
+        be.matmul(qw, x, ye)
+        torch.cuda.synchronize()
+        assert torch.equal(ye, y)
+        qw.free()
+    finally:
+        be.close()
 
 
 def test_container_to_backend(backend, oracle, tmp_path):

@@ -98,3 +98,27 @@ def test_cpu_baseline_matches_the_oracle(oracle):
             assert 1 <= used <= threads
             assert oracle.rel_l2(y, ref) < 2e-6
     assert oracle.cpu_baseline_isa() in ("avx512", "avx2", "plain")
+
+
+def _golden_cases():
+    import json
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "matmul_small.json")
+    for c in json.load(open(path))["cases"]:
+        q = np.array(c["q"], np.int8)
+        s = np.array(c["scales_f16_bits"], np.uint16)
+        x = np.array(c["x_f16_bits"], np.uint16).view(np.float16).astype(np.float32)
+        yield c["name"], c["bits"], q, s, x, np.array(c["y"], np.float64)
+
+
+def test_oracle_reproduces_the_committed_known_answers(oracle):
+    """tests/golden/matmul_small.json: expected outputs computed with numpy float64 by the generator script,
+    one case small enough to follow by hand (y[n] = 16 (n + 1))."""
+    names = []
+    for name, bits, q, s, x, want in _golden_cases():
+        names.append(name)
+        assert np.allclose(oracle.matmul_f64(q, s, x), want, rtol=1e-12, atol=1e-12), name
+        assert oracle.rel_l2(oracle.matmul_f32(q, s, x), want) < 1e-6, name
+        if name == "by_hand_q4":
+            assert want.tolist() == [[16.0, 32.0, 48.0, 64.0]]
+    assert names == ["by_hand_q4", "seeded_q4", "seeded_q8"]
