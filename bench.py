@@ -35,8 +35,8 @@ MIN_TIMED_S = 0.050
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the
 # same counter reads for a plain 256 MiB copy; profiles/decode_gemv_q4_4096x14336_m1.md and
 # profiles/prefill_gemm_q4_4096x14336_m512.md
-TRAFFIC_DECODE_BYTES = 33_270_500
-TRAFFIC_PREFILL_M512_BYTES = 121_950_000
+TRAFFIC_DECODE_BYTES = 33_194_100
+TRAFFIC_PREFILL_M512_BYTES = 121_870_000      # multiply 113.4 MB + activation staging pass 8.5 MB
 
 
 def log(*a):
