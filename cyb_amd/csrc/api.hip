@@ -401,7 +401,7 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
     hipStream_t st = static_cast<hipStream_t>(stream);
     cybq::WeightView v = view_of(w);
     hipError_t e;
-    if (M <= 16) {
+    if (M <= 16 || (M <= 32 && cybq::gemv_serves_32((int)xdt, (int)M, epi))) {
         e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->decode_exact, epi, st);
     } else if (!w->wide_scales && (xdt == CYBQ_F32 ? !ctx->prefill_exact : M > 32)) {
         e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, workspace, workspace_bytes,
@@ -411,8 +411,9 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
         // exact-mode prefill in fp32 is walked 16 rows at a time (FAST mode rounds them to f16
         // in the staging pass and takes the MFMA kernel from 17 rows on: the LDS decode kernel
         // needs 52 - 65 us for 24 - 32 fp32 rows, the MFMA kernel 31).  So are 17..32
-        // rows of 16-bit activations: two passes of the batched-rows kernel stream the
-        // weights twice and are still quicker than a 128-row MFMA tile mostly empty.
+        // rows of 16-bit activations with a folded norm: two passes of the batched-rows
+        // kernel stream the weights twice and are still quicker than a 128-row MFMA tile
+        // mostly empty (without the norm they are one pass, two row blocks per weight operand).
         e = hipSuccess;
         const int64_t n_out = epi.kind == cybq::kEpiSwiglu ? w->N / 2 : w->N;
         for (int64_t m0 = 0; m0 < M && e == hipSuccess; m0 += 16) {

@@ -18,7 +18,9 @@ hipError_t launch_repack(int bits, int layout, const void* q, const void* scales
                          hipStream_t st);
 hipError_t launch_dequant(const WeightView& w, float* out, hipStream_t st);
 
-// decode path, 1 <= M <= 16 per call (api.hip walks 17..32 rows as two calls)
+// decode path, 1 <= M <= 16 per call, and 17 .. 32 rows where gemv_serves_32 says so (api.hip
+// walks the other 17..32-row calls 16 rows at a time)
+bool gemv_serves_32(int xdt, int M, const Epilogue& epi);
 // exact_operands: keep the weight operands exact integers for one f16 row too (the LDS kernel)
 // instead of the subnormal-operand kernel of gemv1.hip
 hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,

@@ -9,22 +9,23 @@ namespace {
 // The one-row decode kernel's requests without its arithmetic: wave wv of a strip's workgroup
 // owns the sets (four consecutive K tiles) wv, wv + nwaves, ...
 template <int BITS, int SETS, bool IO>
-__global__ __launch_bounds__(1024) void read_probe_kernel(WeightView w, const _Float16* __restrict__ x, float* __restrict__ y)
+// (scalar arguments, delivered in registers at wave start like the decode kernel's)
+__global__ __launch_bounds__(1024) void read_probe_kernel(const uint8_t* __restrict__ wbase, const _Float16* __restrict__ x, int KT,
+                                                          int nwaves, float* __restrict__ y)
 {
     constexpr int QV = BITS == 4 ? 1 : 2;
     constexpr int TB = kTileBytes<BITS>, QB = kTileQBytes<BITS>;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nwaves = (int)blockDim.x >> 6;
     const int row = lane & 15, blk = lane >> 4;
-    const int strip_tile = (int)blockIdx.x * w.KT;
+    const int strip_tile = (int)blockIdx.x * KT;
     u32x4_t a[SETS], q[SETS][4][QV];
     u32x2_t sc[SETS];
 #pragma unroll
     for (int h = 0; h < SETS; h++) {
         const int set = wv + nwaves * h;
         if (IO) a[h] = *reinterpret_cast<const u32x4_t*>(x + set * 512 + row * 32 + blk * 8);
-        const uint8_t* sb = w.base + (int64_t)(strip_tile + 4 * set) * TB;
+        const uint8_t* sb = wbase + (int64_t)(strip_tile + 4 * set) * TB;
         sc[h] = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(sb + ((uint32_t)blk * TB + QB + row * 8)));
 #pragma unroll
         for (int b = 0; b < 4; b++)
@@ -78,8 +79,8 @@ hipError_t launch_read_probe(const WeightView& w, bool io, const void* x, void* 
     float* yp = reinterpret_cast<float*>(y);
 #define CYBQ_PROBE(B, S)                                                                                            \
     do {                                                                                                            \
-        if (io) hipLaunchKernelGGL((read_probe_kernel<B, S, true>), grid, block, 0, st, w, xp, yp);                 \
-        else hipLaunchKernelGGL((read_probe_kernel<B, S, false>), grid, block, 0, st, w, xp, yp);                   \
+        if (io) hipLaunchKernelGGL((read_probe_kernel<B, S, true>), grid, block, 0, st, w.base, xp, w.KT, (int)block.x >> 6, yp); \
+        else hipLaunchKernelGGL((read_probe_kernel<B, S, false>), grid, block, 0, st, w.base, xp, w.KT, (int)block.x >> 6, yp);  \
     } while (0)
     if (w.bits == 4 && per_wave == 1) CYBQ_PROBE(4, 1);
     else if (w.bits == 4) CYBQ_PROBE(4, 2);

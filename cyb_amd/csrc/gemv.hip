@@ -398,15 +398,18 @@ __device__ __forceinline__ void norm_staged_slab(uint16_t* xs, int M, int slab_k
 // (one register set); otherwise two batches are live and ping-pong.
 // NORM: RMSNorm folded into the staged x (only instantiated for the streaming variant U = 2).
 template <int BITS, int XMODE, int RMAX, int U, bool ONESHOT, int PAIR, bool NORM>
-__global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __restrict__ x, int M, void* __restrict__ y,
-                            int ydt, int slab_tiles, int ldx, int red_offset, Epilogue epi)
+// (leading scalar arguments, in the order of their first use: they arrive in registers at wave start)
+// (the launch's thread count travels with them: the launch geometry is not among what is preloaded)
+__global__ __launch_bounds__(1024) void gemv_kernel(const uint8_t* __restrict__ wbase, const void* __restrict__ x, int KT, int K, int M,
+                            int nthreads, int slab_tiles, int ldx, int red_offset, void* __restrict__ y, int N, int ydt, int NT,
+                            Epilogue epi)
 {
+    const WeightView w = {wbase, N, K, NT, KT, BITS};
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t* xs = reinterpret_cast<uint16_t*>(smem);
     const uint32_t magic = (BITS == 4 && XMODE == XBF16) ? q4_magic_vgpr_bf16() : q4_magic_vgpr();
 
     const int tid = threadIdx.x;
-    const int nthreads = blockDim.x;
     const int lane = tid & 63;
     // SwiGLU: the workgroup owns a gate strip and its up strip; the first half of its
     // waves splits the K tiles of one, the second half those of the other, x is staged once
@@ -531,11 +534,8 @@ __global__ __launch_bounds__(1024) void gemv_kernel(WeightView w, const void* __
 // on the batch it is part of (within this kernel; the LDS kernel may split K over
 // a different number of waves).
 template <int BITS, int XMODE>
-__device__ __forceinline__ void tile_issue_regs(const TileRegs<BITS>& t, const Frag16 (&a)[4], uint32_t magic,
-                                                float4_t d[4])
+__device__ __forceinline__ void tile_operands(const TileRegs<BITS>& t, uint32_t magic, Frag16 (&b)[4])
 {
-    const float4_t zero = {0.f, 0.f, 0.f, 0.f};
-    Frag16 b[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         uint32_t bw[4];
@@ -549,6 +549,12 @@ __device__ __forceinline__ void tile_issue_regs(const TileRegs<BITS>& t, const F
         }
         b[j].u = (u32x4_t){bw[0], bw[1], bw[2], bw[3]};
     }
+}
+
+template <int BITS, int XMODE>
+__device__ __forceinline__ void tile_multiply(const Frag16 (&a)[4], const Frag16 (&b)[4], float4_t d[4])
+{
+    const float4_t zero = {0.f, 0.f, 0.f, 0.f};
     Frag16 off;
     const uint32_t offw = BITS == 4 ? kBf16Neg136x2 : kBf16Neg128x2;
     off.u = (u32x4_t){offw, offw, offw, offw};
@@ -559,6 +565,15 @@ __device__ __forceinline__ void tile_issue_regs(const TileRegs<BITS>& t, const F
             d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j].b, off.b, d[j], 0, 0, 0);
         } else d[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j].h, b[j].h, zero, 0, 0, 0);
     }
+}
+
+template <int BITS, int XMODE>
+__device__ __forceinline__ void tile_issue_regs(const TileRegs<BITS>& t, const Frag16 (&a)[4], uint32_t magic,
+                                                float4_t d[4])
+{
+    Frag16 b[4];
+    tile_operands<BITS, XMODE>(t, magic, b);
+    tile_multiply<BITS, XMODE>(a, b, d);
 }
 
 // NORM: RMSNorm folded into the activation load (epi.gamma / epi.eps): an operand fragment
@@ -600,17 +615,20 @@ __device__ __forceinline__ void norm_frag(Frag16& a, const float* gamma_lds, int
     }
 }
 
-template <int BITS, int XMODE, int TS, int NS, bool NORM, int XR>
+// MB: blocks of 16 batch rows (2 = 17..32 rows: every unpacked weight operand is multiplied with
+// two activation operands, the weights still stream once).
+template <int BITS, int XMODE, int TS, int NS, bool NORM, int XR, int MB = 1>
 // (waves_per_eu: the scheduler would otherwise trade the up-front loads for occupancy)
-__global__ __launch_bounds__(TS <= 2 ? 1024 : 512) __attribute__((amdgpu_waves_per_eu(2, TS <= 2 ? 4 : 2)))
-void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void* __restrict__ y, int ydt, Epilogue epi)
+__global__ __launch_bounds__((TS <= 2 && MB == 1) ? 1024 : 512) __attribute__((amdgpu_waves_per_eu(2, (TS <= 2 && MB == 1) ? 4 : 2)))
+void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restrict__ x, int KT_, int K, int NT, int M, int nwaves,
+                      void* __restrict__ y, int N, int ydt, Epilogue epi)
 {
+    const WeightView w = {wbase, N, K, NT, KT_, BITS};
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t magic = (BITS == 4 && XMODE == XBF16) ? q4_magic_vgpr_bf16() : q4_magic_vgpr();
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nwaves = (int)blockDim.x >> 6;
     const int oct = lane >> 4;
     const int strip0 = blockIdx.x * NS;
     const int KT = w.KT;
@@ -623,14 +641,16 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
     constexpr int P = 64 / XR;                  // 16 B pieces per row and load
     constexpr int L = 16 / P;                   // loads per tile: 1, 2, 4
     constexpr int GPL = 4 / L;                  // scale groups per load
+    static_assert(MB == 1 || (XR == 16 && !NORM), "two row blocks: full loads, no folded norm");
     const uint16_t* xrow = x + (int64_t)min(lane / P, M - 1) * w.K + (lane % P) * 8;
+    const int64_t xblock = MB > 1 ? (int64_t)(min(16 + lane / P, M - 1) - min(lane / P, M - 1)) * w.K : 0;     // to my row of the second block
     const int klast = w.K - 8 - (lane % P) * 8;          // last start at which this lane's piece is inside the row
     const int from_lane = ((((lane & 15) & (XR - 1)) * P) | oct) << 2;       // byte address for ds_bpermute (+ 16 per group)
     // NORM: gamma as fp32 in LDS behind the exchange areas (read per fragment with LDS loads, which
     // do not queue behind the weight requests the way global loads would)
-    float* gamma_lds = reinterpret_cast<float*>(smem) + NS * nwaves * 4 * 64 + nwaves * 16;
+    float* gamma_lds = reinterpret_cast<float*>(smem) + NS * MB * nwaves * 4 * 64 + nwaves * 16;
     if (NORM) {
-        for (int c = tid; c < (w.K >> 3); c += (int)blockDim.x) {
+        for (int c = tid; c < (w.K >> 3); c += nwaves * 64) {
             float g[8];
             load_gamma8(epi.gamma, epi.gamma_dt, c * 8, g);
             reinterpret_cast<float4_t*>(gamma_lds + c * 8)[0] = (float4_t){g[0], g[1], g[2], g[3]};
@@ -639,11 +659,13 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
         __syncthreads();
     }
 
-    float acc[NS][4];
+    float acc[NS][MB][4];
 #pragma unroll
     for (int s = 0; s < NS; s++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) acc[s][r] = 0.f;
+        for (int b = 0; b < MB; b++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[s][b][r] = 0.f;
     float ssq = 0.f;          // NORM: squares of the x values this lane holds (row lane % 16)
 
     int64_t sbase[NS];
@@ -654,7 +676,7 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
         // my K tiles of this slab and their x operands (clamped past the end; such tiles get scale 0)
         int kt[TS];
         bool valid[TS];
-        Frag16 a[TS][4];
+        Frag16 a[MB][TS][4];
 #pragma unroll
         for (int u = 0; u < TS; u++) {
             const int t = slab0 + wv + nwaves * u;
@@ -664,8 +686,11 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
             for (int h = 0; h < L; h++) {
                 // (past the end of K: any x inside the row will do, the padded weights are zero)
                 const int k0 = kt[u] * kTileK + h * (GPL * 32);
-                if (XR == 16) a[u][h].u = *reinterpret_cast<const u32x4_t*>(xrow + min(k0, w.K - 32));
-                else a[u][h].u = *reinterpret_cast<const u32x4_t*>(xrow + min(k0, klast));
+                if (XR == 16) {
+#pragma unroll
+                    for (int b = 0; b < MB; b++)
+                        a[b][u][h].u = *reinterpret_cast<const u32x4_t*>(xrow + b * xblock + min(k0, w.K - 32));
+                } else a[0][u][h].u = *reinterpret_cast<const u32x4_t*>(xrow + min(k0, klast));
             }
         }
         // The memory pipeline takes requests at its own pace: a wave that asks for all its
@@ -680,24 +705,26 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
 #pragma unroll
             for (int u = 0; u < TS; u++) load_tile<BITS>(buf[s][u], w, sbase[s] + kt[u], lane);
 #pragma unroll
-        for (int u = 0; u < TS; u++) {
-            u32x4_t raw[L];
+        for (int b = 0; b < MB; b++)
 #pragma unroll
-            for (int h = 0; h < L; h++) raw[h] = a[u][h].u;
+            for (int u = 0; u < TS; u++) {
+                u32x4_t raw[L];
 #pragma unroll
-            for (int j = 0; j < 4; j++)
+                for (int h = 0; h < L; h++) raw[h] = a[b][u][h].u;
 #pragma unroll
-                for (int p = 0; p < 4; p++)
-                    a[u][j].u[p] =
-                        (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane + (j % GPL) * 16, (int)raw[j / GPL][p]);
-        }
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int p = 0; p < 4; p++)
+                        a[b][u][j].u[p] =
+                            (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane + (j % GPL) * 16, (int)raw[j / GPL][p]);
+            }
         if (NORM) {
 #pragma unroll
             for (int u = 0; u < TS; u++)
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     const int kg = kt[u] * kTileK + j * 32;            // (a group past K repeats the last one: not counted)
-                    norm_frag<XMODE>(a[u][j], gamma_lds, min(kg, w.K - 32) + oct * 8, valid[u] && kg < w.K, ssq);
+                    norm_frag<XMODE>(a[0][u][j], gamma_lds, min(kg, w.K - 32) + oct * 8, valid[u] && kg < w.K, ssq);
                 }
         }
 #pragma unroll
@@ -708,33 +735,45 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
                 for (int u = 0; u < TS; u++) load_tile<BITS>(buf[s + AHEAD][u], w, sbase[s + AHEAD] + kt[u], lane);
             }
             if (NS > 2) __builtin_amdgcn_sched_barrier(0);
-            float4_t dprev[4];
+            float4_t dprev[MB][4];
             u32x2_t sprev = {0u, 0u};
 #pragma unroll
-            for (int j = 0; j < 4; j++) dprev[j] = (float4_t){0.f, 0.f, 0.f, 0.f};
+            for (int b = 0; b < MB; b++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) dprev[b][j] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int u = 0; u < TS; u++) {
-                float4_t d[4];
-                tile_issue_regs<BITS, XMODE>(buf[s][u], a[u], magic, d);
+                float4_t d[MB][4];
+                Frag16 bop[4];
+                tile_operands<BITS, XMODE>(buf[s][u], magic, bop);
+#pragma unroll
+                for (int b = 0; b < MB; b++) tile_multiply<BITS, XMODE>(a[b][u], bop, d[b]);
                 u32x2_t sc = buf[s][u].s;
                 sc[0] = valid[u] ? sc[0] : 0u;
                 sc[1] = valid[u] ? sc[1] : 0u;
-                tile_accum<4>(sprev, dprev, acc[s]);
 #pragma unroll
-                for (int j = 0; j < 4; j++) dprev[j] = d[j];
+                for (int b = 0; b < MB; b++) {
+                    tile_accum<4>(sprev, dprev[b], acc[s][b]);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) dprev[b][j] = d[b][j];
+                }
                 sprev = sc;
             }
-            tile_accum<4>(sprev, dprev, acc[s]);
+#pragma unroll
+            for (int b = 0; b < MB; b++) tile_accum<4>(sprev, dprev[b], acc[s][b]);
         }
     }
 
     // split-K partials -> LDS, summed in wave order
+    // (slot = strip * MB + row block)
     float* red = reinterpret_cast<float*>(smem);
 #pragma unroll
     for (int s = 0; s < NS; s++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) red[((s * nwaves + wv) * 4 + r) * 64 + lane] = acc[s][r];
-    float* ssq_part = red + NS * nwaves * 4 * 64;      // [wave][row]
+        for (int b = 0; b < MB; b++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) red[(((s * MB + b) * nwaves + wv) * 4 + r) * 64 + lane] = acc[s][b][r];
+    float* ssq_part = red + NS * MB * nwaves * 4 * 64;      // [wave][row]
     if (NORM) {
         ssq += __shfl_xor(ssq, 16, 64);
         ssq += __shfl_xor(ssq, 32, 64);
@@ -753,43 +792,49 @@ void gemv_rows_kernel(WeightView w, const uint16_t* __restrict__ x, int M, void*
     // wave v finishes (strip, output register) pairs v, v + waves, ...
     if (NS >= 2 && epi.kind == kEpiSwiglu) {       // strips 2j / 2j+1 of the group are gate / up of output strip (strip0 >> 1) + j
         const int n_out = w.N >> 1;
-        for (int p = wv; p < NS * 2; p += nwaves) {
-            const int j = p >> 2, r = p & 3;
+        for (int p = wv; p < NS * MB * 2; p += nwaves) {
+            const int r = p & 3, b = (p >> 2) % MB, j = (p >> 2) / MB;
             const int nt = (strip0 >> 1) + j;
             const int n = nt * 16 + (lane & 15);
-            const float g = sum_partials(red + ((2 * j) * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64) * rstd[r];
-            const float u = sum_partials(red + ((2 * j + 1) * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64) * rstd[r];
-            const int m = 4 * oct + r;
-            if (m < M && n < n_out) store_out(y, ydt, (int64_t)m * n_out + n, silu_mul(g, u));
+            const float g = sum_partials(red + (((2 * j) * MB + b) * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64) * rstd[r];
+            const float u = sum_partials(red + (((2 * j + 1) * MB + b) * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64) * rstd[r];
+            const int m = 16 * b + 4 * oct + r;
+            if (2 * nt + 1 < w.NT && m < M && n < n_out) store_out(y, ydt, (int64_t)m * n_out + n, silu_mul(g, u));
         }
         return;
     }
-    for (int p = wv; p < NS * 4; p += nwaves) {
-        const int s = p >> 2, r = p & 3;
+    for (int p = wv; p < NS * MB * 4; p += nwaves) {
+        const int r = p & 3, b = (p >> 2) % MB, s = (p >> 2) / MB;
         const int nt = strip0 + s;
         const int n = nt * 16 + (lane & 15);
-        const float v = sum_partials(red + (s * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64) * rstd[r];
-        const int m = 4 * oct + r;
+        const float v = sum_partials(red + ((s * MB + b) * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64) * rstd[r];
+        const int m = 16 * b + 4 * oct + r;
         if (nt < w.NT && m < M && n < w.N) emit(y, ydt, epi, (int64_t)m * w.N + n, v);
     }
 }
 
-template <int BITS, int XMODE, int TS, int NS, int XR>
+template <int BITS, int XMODE, int TS, int NS, int XR, int MB = 1>
 hipError_t launch_rows_x(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
                          hipStream_t st)
 {
-    size_t lds = (size_t)NS * nwaves * 4 * 64 * sizeof(float) + (size_t)nwaves * 16 * sizeof(float);
+    size_t lds = (size_t)NS * MB * nwaves * 4 * 64 * sizeof(float) + (size_t)nwaves * 16 * sizeof(float);
     const unsigned groups = (unsigned)((w.NT + NS - 1) / NS);
-    if (epi.gamma) {
-        lds += (size_t)w.K * sizeof(float);            // gamma as fp32
-        auto kern = gemv_rows_kernel<BITS, XMODE, TS, NS, true, XR>;
-        (void)LdsRequest<&gemv_rows_kernel<BITS, XMODE, TS, NS, true, XR>, 150 * 1024>::registered;
-        if (lds > 150 * 1024) return hipErrorInvalidValue;      // (launch_gemv keeps such K away from this kernel)
-        hipLaunchKernelGGL(kern, dim3(groups), dim3(nwaves * 64), lds, st, w, reinterpret_cast<const uint16_t*>(x), M, y, ydt,
-                           epi);
-    } else
-        hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS, false, XR>), dim3(groups), dim3(nwaves * 64), lds, st, w,
-                           reinterpret_cast<const uint16_t*>(x), M, y, ydt, epi);
+    if constexpr (MB == 1) {
+        if (epi.gamma) {
+            lds += (size_t)w.K * sizeof(float);            // gamma as fp32
+            auto kern = gemv_rows_kernel<BITS, XMODE, TS, NS, true, XR>;
+            (void)LdsRequest<&gemv_rows_kernel<BITS, XMODE, TS, NS, true, XR>, 150 * 1024>::registered;
+            if (lds > 150 * 1024) return hipErrorInvalidValue;      // (launch_gemv keeps such K away from this kernel)
+            hipLaunchKernelGGL(kern, dim3(groups), dim3(nwaves * 64), lds, st, w.base, reinterpret_cast<const uint16_t*>(x), w.KT, w.K,
+                               w.NT, M, nwaves, y, w.N, ydt, epi);
+            return hipGetLastError();
+        }
+    }
+    // (the exchange area alone passes 64 KB with eight strips, or four strips and two row blocks)
+    if constexpr (NS * MB * 8 * 1024 + 512 > 64 * 1024)
+        (void)LdsRequest<&gemv_rows_kernel<BITS, XMODE, TS, NS, false, XR, MB>, 150 * 1024>::registered;
+    hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS, false, XR, MB>), dim3(groups), dim3(nwaves * 64), lds, st, w.base,
+                       reinterpret_cast<const uint16_t*>(x), w.KT, w.K, w.NT, M, nwaves, y, w.N, ydt, epi);
     return hipGetLastError();
 }
 
@@ -803,22 +848,30 @@ hipError_t launch_rows_t(const WeightView& w, const void* x, int M, void* y, int
     return launch_rows_x<BITS, XMODE, TS, NS, 16>(w, x, M, y, ydt, nwaves, epi, st);
 }
 
+// strips per workgroup: as many as keeps about one workgroup per CU, at most 4
+int strips_per_group(const WeightView& w, int num_cus, const Epilogue& epi)
+{
+    int ns = (w.NT + num_cus / 2) / num_cus;
+    ns = ns >= 3 ? 4 : (ns >= 2 ? 2 : 1);
+    if (epi.kind == kEpiSwiglu && ns < 2) ns = 2;          // a gate strip and its up strip share a workgroup
+    return ns;
+}
+
 template <int BITS, int XMODE>
 hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int ydt, int tuned_waves, int num_cus,
                        const Epilogue& epi, hipStream_t st)
 {
-    // strips per workgroup: as many as keeps about one workgroup per CU, at most 4;
     // 8 waves split K (fewer when the strip has fewer tiles), 4 tiles of x per wave and slab
-    int ns = (w.NT + num_cus / 2) / num_cus;
-    ns = ns >= 3 ? 4 : (ns >= 2 ? 2 : 1);
-    if (epi.kind == kEpiSwiglu && ns < 2) ns = 2;          // a gate strip and its up strip share a workgroup
+    const int ns = strips_per_group(w, num_cus, epi);
     // seven strips per workgroup when that is exactly one workgroup per CU (N = 28672 on 256 CUs:
-    // with four strips the 448 workgroups need a second, mostly empty round); SwiGLU pairs need an even count
-    const bool seven = w.NT == 7 * num_cus && epi.kind != kEpiSwiglu;
+    // with four strips the 448 workgroups need a second, mostly empty round); SwiGLU pairs need an
+    // even count: eight strips there, 224 workgroups in one round
+    const bool seven = w.NT == 7 * num_cus;
     int nwaves = tuned_waves > 0 ? min(tuned_waves, 8) : 8;
     while (nwaves > 1 && nwaves * 2 > w.KT) nwaves >>= 1;
     if constexpr (BITS == 4) {
-        if (seven) return launch_rows_t<BITS, XMODE, 4, 7>(w, x, M, y, ydt, nwaves, epi, st);
+        if (seven && epi.kind == kEpiSwiglu && !epi.gamma) return launch_rows_t<BITS, XMODE, 4, 8>(w, x, M, y, ydt, nwaves, epi, st);
+        if (seven && epi.kind != kEpiSwiglu) return launch_rows_t<BITS, XMODE, 4, 7>(w, x, M, y, ydt, nwaves, epi, st);
         if (ns == 4) return launch_rows_t<BITS, XMODE, 4, 4>(w, x, M, y, ydt, nwaves, epi, st);
     } else if constexpr (XMODE == XF16) {
         // Q8 tiles are twice the registers: four strips x four tiles of f16 operands would spill.  Two
@@ -840,6 +893,25 @@ hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int y
         }
     }
     return launch_rows_t<BITS, XMODE, 4, 1>(w, x, M, y, ydt, nwaves, epi, st);
+}
+
+// 17 .. 32 rows: two activation operands per weight operand.  Two tiles of x per wave and slab
+// (a wave holds 2 x 2 x 4 operand fragments) when a workgroup has several strips, four with one.
+template <int BITS, int XMODE>
+hipError_t launch_rows2(const WeightView& w, const void* x, int M, void* y, int ydt, int tuned_waves, int num_cus,
+                        const Epilogue& epi, hipStream_t st)
+{
+    const int ns = strips_per_group(w, num_cus, epi);
+    int nwaves = tuned_waves > 0 ? min(tuned_waves, 8) : 8;
+    while (nwaves > 1 && nwaves * 2 > w.KT) nwaves >>= 1;
+    if constexpr (BITS == 4) {
+        if (w.NT == 7 * num_cus && epi.kind != kEpiSwiglu)
+            return launch_rows_x<BITS, XMODE, 2, 7, 16, 2>(w, x, M, y, ydt, nwaves, epi, st);
+        if (ns == 4) return launch_rows_x<BITS, XMODE, 2, 4, 16, 2>(w, x, M, y, ydt, nwaves, epi, st);
+    }
+    if (ns >= 2) return launch_rows_x<BITS, XMODE, 2, 2, 16, 2>(w, x, M, y, ydt, nwaves, epi, st);
+    if constexpr (BITS == 4) return launch_rows_x<BITS, XMODE, 4, 1, 16, 2>(w, x, M, y, ydt, nwaves, epi, st);
+    return launch_rows_x<BITS, XMODE, 2, 1, 16, 2>(w, x, M, y, ydt, nwaves, epi, st);
 }
 
 int g_tune_waves = 0, g_tune_unroll = 0, g_tune_rows = 0;
@@ -874,8 +946,8 @@ hipError_t launch_p(const WeightView& w, const void* x, int M, void* y, int ydt,
     // and the norm's row sums - the largest request there is, 146 KB.
     (void)LdsRequest<&gemv_kernel<BITS, XMODE, RMAX, U, ONESHOT, PAIR, NORM>, kLdsCap>::registered;
     if (lds > (size_t)kLdsCap) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(kern, dim3(w.NT / PAIR), dim3(nwaves * PAIR * 64), lds, st, w, x, M, y, ydt, slab_tiles, ldx, (int)xbytes,
-                       epi);
+    hipLaunchKernelGGL(kern, dim3(w.NT / PAIR), dim3(nwaves * PAIR * 64), lds, st, w.base, x, w.KT, w.K, M, nwaves * PAIR * 64, slab_tiles, ldx,
+                       (int)xbytes, y, w.N, ydt, w.NT, epi);
     return hipGetLastError();
 }
 
@@ -923,6 +995,12 @@ void set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll)
     g_tune_unroll = unroll;
 }
 
+// 17 .. 32 rows in one pass (weights streamed once): 16-bit activations, no folded norm
+bool gemv_serves_32(int xdt, int M, const Epilogue& epi)
+{
+    return M > 16 && M <= 32 && xdt != kF32 && !epi.gamma && g_tune_rows != 2;
+}
+
 hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
                        int num_cus, bool exact_operands, const Epilogue& epi, hipStream_t st)
 {
@@ -964,6 +1042,15 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
     // (a folded norm keeps gamma as fp32 in LDS next to the exchange areas: beyond K = 23552 that no
     // longer fits and the LDS kernel, which stages x in slabs, takes the call)
     const bool gamma_fits = !epi.gamma || w.K <= 23552;
+    if (M > 16) {
+        if (!gemv_serves_32(xdt, M, epi)) return hipErrorInvalidValue;
+        if (w.bits == 4) {
+            if (xdt == kF16) return launch_rows2<4, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
+            return launch_rows2<4, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
+        }
+        if (xdt == kF16) return launch_rows2<8, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
+        return launch_rows2<8, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
+    }
     if (rows_kernel && xdt != kF32 && gamma_fits) {
         if (w.bits == 4) {
             if (xdt == kF16) return launch_rows<4, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);

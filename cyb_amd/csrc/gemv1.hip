@@ -65,22 +65,46 @@ __device__ __forceinline__ Frag16 sub_operand(const u32x4_t (&q)[BITS == 4 ? 1 :
 
 // SETS: sets a wave owns (set index wv + nwaves * h).  NS: strips per workgroup (2 = a gate strip
 // and its up strip, SwiGLU epilogue).  EVEN: K is a multiple of 512 and every wave has SETS
-// whole sets, so nothing needs clamping.  NW: waves per workgroup when known at compile time (0 = any).
-template <int BITS, int SETS, int NS, bool EVEN, int NW>
-__global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float16* __restrict__ x, void* __restrict__ y, int ydt,
-                                                     Epilogue epi)
+// whole sets, so nothing needs clamping.  NW: waves that split K when known at compile time (0 = any).
+// SPLIT (NS = 2, NW > 0): the workgroup has 2 * NW waves, waves [0, NW) take the gate strip and
+// [NW, 2 NW) the up strip - per wave the same work as with one strip per workgroup (a wave that
+// holds both strips' tiles has twice the requests in flight and half the waves to hide them).
+// RES: the residual-add epilogue; the residual is requested first of all, so that it is there long
+// before the sums are (asked for at the end it would cost the kernel one more trip to memory).
+template <int BITS, int SETS, int NS, bool EVEN, int NW, bool SPLIT = false, bool RES = false>
+// The arguments are scalars in the order the kernel needs them: the compiler is asked to have
+// them delivered in registers at wave start (kernel argument preload), so the first requests do
+// not wait for a load of the argument block.
+// (14 dwords; the launch's wave count travels with them, the launch geometry is not among what is preloaded.)
+__global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__ wbase, const _Float16* __restrict__ x,
+                                                     const void* __restrict__ residual, void* __restrict__ y, int KT, int K,
+                                                     int launch_waves, int n_rows, int out_dt, int epi_kind)
 {
     constexpr int QV = BITS == 4 ? 1 : 2;
     __shared__ float red[NS * 16 * 16];
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nwaves = NW ? NW : (int)blockDim.x >> 6;          // NW = 0: whatever the launch says
+    static_assert(!SPLIT || (NS == 2 && NW > 0), "split workgroups are gate / up pairs with a known wave count");
+    constexpr int NL = SPLIT ? 1 : NS;            // strips a wave works on
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int wv = wave, half = 0;                      // my place among the waves that split K; SPLIT: my strip of the pair
+    if constexpr (SPLIT) {
+        wv = wave % NW;
+        half = wave / NW;
+    }
+    const int nwaves = NW ? NW : launch_waves;          // NW = 0: whatever the launch says
     const int row = lane & 15, blk = lane >> 4;
-    const int KT = w.KT;
 
+    uint32_t res_word = 0;            // the aligned 32-bit word that holds this lane's residual element
+    uint32_t res_addr = 0;
+    if constexpr (RES) {
+        const int n = min((int)blockIdx.x * 16 + row, n_rows - 1);
+        const uintptr_t p = reinterpret_cast<uintptr_t>(residual) + (uintptr_t)n * (out_dt == kF32 ? 4u : 2u);
+        res_addr = (uint32_t)p;
+        res_word = *reinterpret_cast<const uint32_t*>(p & ~(uintptr_t)3);
+    }
     Frag16 a[SETS];
-    u32x2_t sc[NS][SETS];
-    u32x4_t q[NS][SETS][4][QV];
+    u32x2_t sc[NL][SETS];
+    u32x4_t q[NL][SETS][4][QV];
     bool tile_ok[SETS];               // this lane block's tile of the set exists (!EVEN)
 #pragma unroll
     for (int h = 0; h < SETS; h++) {
@@ -89,7 +113,7 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float1
         if (EVEN) {
             a[h].u = *reinterpret_cast<const u32x4_t*>(x + k);
         } else {
-            a[h].u = *reinterpret_cast<const u32x4_t*>(x + min(k, w.K - 8));
+            a[h].u = *reinterpret_cast<const u32x4_t*>(x + min(k, K - 8));
             tile_ok[h] = 4 * set + blk < KT;
         }
     }
@@ -99,13 +123,13 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float1
     const uint32_t lane_q = (uint32_t)lane * 16u;
     const uint32_t lane_s = (uint32_t)QB + (uint32_t)row * 8u;
 #pragma unroll
-    for (int st = 0; st < NS; st++) {
-        const int strip_tile = ((int)blockIdx.x * NS + st) * KT;           // tile indices fit 32 bits
+    for (int st = 0; st < NL; st++) {
+        const int strip_tile = ((int)blockIdx.x * NS + st + half) * KT;    // tile indices fit 32 bits
 #pragma unroll
         for (int h = 0; h < SETS; h++) {
             const int t0 = 4 * (wv + nwaves * h);
             if (EVEN) {
-                const uint8_t* sb = w.base + (int64_t)(strip_tile + t0) * TB;
+                const uint8_t* sb = wbase + (int64_t)(strip_tile + t0) * TB;
                 sc[st][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(sb + ((uint32_t)blk * TB + lane_s)));
 #pragma unroll
                 for (int b = 0; b < 4; b++)
@@ -113,7 +137,7 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float1
                     for (int v = 0; v < QV; v++)
                         q[st][h][b][v] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(sb + (b * TB + v * 1024) + lane_q));
             } else {
-                const uint8_t* strip = w.base + (int64_t)strip_tile * TB;
+                const uint8_t* strip = wbase + (int64_t)strip_tile * TB;
                 sc[st][h] = __builtin_nontemporal_load(
                     reinterpret_cast<const u32x2_t*>(strip + ((uint32_t)min(t0 + blk, KT - 1) * TB + lane_s)));
 #pragma unroll
@@ -129,8 +153,6 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float1
     // Everything the tail needs from the kernel arguments is fetched now, next to the requests:
     // left to itself the compiler loads each argument where it is first used, i.e. after the
     // final barrier, and the kernel would end with two more round trips to memory.
-    const int n_rows = w.N, out_dt = ydt, epi_kind = epi.kind;
-    const void* const residual = epi.residual;
     asm volatile("" ::"s"(n_rows), "s"(out_dt), "s"(epi_kind), "s"(residual), "s"(y));
     if (!NW) asm volatile("" ::"s"(nwaves));
     __builtin_amdgcn_sched_barrier(0);       // every request is out before any arithmetic
@@ -140,11 +162,11 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float1
         for (int h = 0; h < SETS; h++) {
             // activations past K (the padded tail of the last tile) count as zero; a tile past
             // the end of the strip was clamped to the last one and gets scale zero
-            const bool x_ok = (wv + nwaves * h) * 512 + row * 32 + blk * 8 < w.K;
+            const bool x_ok = (wv + nwaves * h) * 512 + row * 32 + blk * 8 < K;
 #pragma unroll
             for (int p = 0; p < 4; p++) a[h].u[p] = x_ok ? a[h].u[p] : 0u;
 #pragma unroll
-            for (int st = 0; st < NS; st++) {
+            for (int st = 0; st < NL; st++) {
                 sc[st][h][0] = tile_ok[h] ? sc[st][h][0] : 0u;
                 sc[st][h][1] = tile_ok[h] ? sc[st][h][1] : 0u;
             }
@@ -168,12 +190,12 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float1
     // accumulated with the lane's own scales (the other three sums are finite and unused) and the
     // meaningful one is picked once at the end.  Even groups (low nibbles) and odd groups
     // (high nibbles, 16 times too large) are kept apart until the final scaling.
-    float accL[NS][4], accH[NS][4];
+    float accL[NL][4], accH[NL][4];
 #pragma unroll
-    for (int st = 0; st < NS; st++)
+    for (int st = 0; st < NL; st++)
 #pragma unroll
         for (int b = 0; b < 4; b++) accL[st][b] = accH[st][b] = 0.f;
-    constexpr int T = NS * SETS * 4;
+    constexpr int T = NL * SETS * 4;
     float4_t dprev[4];
 #pragma unroll
     for (int i = 0; i <= T; i++) {
@@ -208,13 +230,13 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float1
     // block j adds the partial sums of waves 4i + j in order of i, the MFMA adds the four blocks.
     const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int st = 0; st < NS; st++) {
+    for (int st = 0; st < NL; st++) {
         float tb[4];
 #pragma unroll
         for (int b = 0; b < 4; b++) tb[b] = BITS == 4 ? accL[st][b] + accH[st][b] * 0.0625f : accL[st][b];
         const float t = blk == 0 ? tb[0] : (blk == 1 ? tb[1] : (blk == 2 ? tb[2] : tb[3]));
         const float4_t sum = __builtin_amdgcn_mfma_f32_16x16x4f32(1.0f, t, zero4, 0, 0, 0);
-        if (lane < 16) red[(st * 16 + wv) * 16 + lane] = sum[0];
+        if (lane < 16) red[((st + half) * 16 + wv) * 16 + lane] = sum[0];
     }
     __syncthreads();
     if (tid >= 64) return;
@@ -238,7 +260,11 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(WeightView w, const _Float1
     }
     if (n < n_rows) {
         float v = outv[0];
-        if (epi_kind == kEpiAdd) v += load_out1(residual, out_dt, n);
+        if constexpr (RES) {
+            const uint32_t h = (res_addr & 2u) ? res_word >> 16 : res_word & 0xffffu;
+            v += out_dt == kF32 ? __builtin_bit_cast(float, res_word)
+                                : (out_dt == kF16 ? f16_bits_to_f32(h) : __builtin_bit_cast(float, h << 16));
+        }
         store_out1(y, out_dt, n, v);
     }
 }
@@ -248,15 +274,30 @@ hipError_t launch1_e(const WeightView& w, const void* x, void* y, int ydt, int n
                      hipStream_t st)
 {
     const dim3 grid((unsigned)(w.NT / NS)), block((unsigned)nwaves * 64);
-    if (even && nwaves == 8 && SETS == 1)          // K = 4096: the shape most decode launches have
-        hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, true, SETS == 1 ? 8 : 0>), grid, block, 0, st, w,
-                           reinterpret_cast<const _Float16*>(x), y, ydt, epi);
-    else if (even)
-        hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, true, 0>), grid, block, 0, st, w, reinterpret_cast<const _Float16*>(x), y, ydt,
-                           epi);
-    else
-        hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, false, 0>), grid, block, 0, st, w, reinterpret_cast<const _Float16*>(x), y, ydt,
-                           epi);
+    const _Float16* xh = reinterpret_cast<const _Float16*>(x);
+#define CYBQ_GEMV1_LAUNCH(EVEN_, NW_, SPLIT_, RES_, BLOCK_)                                                                             \
+    hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, EVEN_, NW_, SPLIT_, RES_>), grid, BLOCK_, 0, st, w.base, xh, epi.residual, y, w.KT, w.K, nwaves, \
+                       w.N, ydt, epi.kind)
+    const bool k8 = even && nwaves == 8 && SETS == 1;          // K = 4096: the shape most decode launches have
+    if constexpr (NS == 2) {
+        if constexpr (SETS == 1) {
+            if (k8) CYBQ_GEMV1_LAUNCH(true, 8, true, false, dim3(1024));
+            else if (even) CYBQ_GEMV1_LAUNCH(true, 0, false, false, block);
+            else CYBQ_GEMV1_LAUNCH(false, 0, false, false, block);
+        } else {
+            if (even) CYBQ_GEMV1_LAUNCH(true, 0, false, false, block);
+            else CYBQ_GEMV1_LAUNCH(false, 0, false, false, block);
+        }
+    } else if (epi.kind == kEpiAdd) {
+        if (k8) CYBQ_GEMV1_LAUNCH(true, (SETS == 1 ? 8 : 0), false, true, block);
+        else if (even) CYBQ_GEMV1_LAUNCH(true, 0, false, true, block);
+        else CYBQ_GEMV1_LAUNCH(false, 0, false, true, block);
+    } else {
+        if (k8) CYBQ_GEMV1_LAUNCH(true, (SETS == 1 ? 8 : 0), false, false, block);
+        else if (even) CYBQ_GEMV1_LAUNCH(true, 0, false, false, block);
+        else CYBQ_GEMV1_LAUNCH(false, 0, false, false, block);
+    }
+#undef CYBQ_GEMV1_LAUNCH
     return hipGetLastError();
 }
 

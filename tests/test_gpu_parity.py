@@ -128,6 +128,16 @@ def test_decode_seven_strips_per_workgroup(backend, oracle):
     backend.matmul_ex(qw, x, y2, "add", r)
     torch.cuda.synchronize()
     assert torch.equal(y2, torch.from_numpy(y).cuda() + r)
+    # gate / up pairs of that width: eight strips (four pairs) per workgroup
+    h = N // 2
+    pair = backend.fuse_pairs(backend.upload_quantized(q[:h], s[:h], 4), backend.upload_quantized(q[h:], s[h:], 4))
+    for M in (3, 8, 16):
+        y3 = torch.empty((M, h), dtype=torch.float32, device="cuda")
+        backend.matmul_ex(pair, x[:M].contiguous(), y3, "swiglu")
+        torch.cuda.synchronize()
+        yd = torch.from_numpy(y[:M]).cuda().double()
+        ref = torch.nn.functional.silu(yd[:, :h]) * yd[:, h:]
+        assert ((y3.double() - ref).norm() / ref.norm()).item() < TIGHT, M
 
 
 @pytest.mark.parametrize("bits,xdt", [(4, "f16"), (4, "bf16"), (8, "f16"), (8, "bf16")])
@@ -159,6 +169,50 @@ def test_decode_batched_rows_wide_shapes(backend, oracle, bits, xdt, N):
                 assert torch.equal(y, y1[:M]), M
     finally:
         backend.set_gemv_tuning(0, 0, 0)
+
+
+@pytest.mark.parametrize("bits,xdt", [(4, "f16"), (4, "bf16"), (8, "f16"), (8, "bf16")])
+@pytest.mark.parametrize("shape", [(14336, 384), (28672, 384), (8192, 384), (512, 4096 + 128), (80, 14336), (33, 160)])
+def test_decode_17_to_32_rows_in_one_pass(backend, oracle, bits, xdt, shape):
+    """17 .. 32 rows of 16-bit activations run the batched-rows kernel with two row blocks: the
+    weights stream once.  A row's bits are those of the same kernel at 16 rows or fewer."""
+    N, K = shape
+    q, s = _quant(oracle, bits, N, K, cfg=27)
+    qw = backend.upload_quantized(q, s, bits)
+    wd = torch.from_numpy(oracle.dequant(q, s)).cuda().double()
+    x = _x(32, K, xdt, cfg=28)
+    try:
+        backend.set_gemv_tuning(0, 1, 0)                 # the batched-rows kernel for the 16-row halves too
+        lo, hi = _run(backend, qw, x[:16].contiguous()), _run(backend, qw, x[16:].contiguous())
+        backend.set_gemv_tuning(0, 0, 0)
+        for M in (32, 17, 24):
+            y = _run(backend, qw, x[:M].contiguous())
+            ref = x[:M].double() @ wd.T
+            err = ((y.double() - ref).norm() / ref.norm()).item()
+            assert err < TIGHT, (M, err)
+            assert torch.equal(y[:16], lo), M
+            assert torch.equal(y[16:], hi[:M - 16]), M
+    finally:
+        backend.set_gemv_tuning(0, 0, 0)
+    if N % 32 == 0 and K == 384:
+        # epilogues in the same kernel: residual add, and SwiGLU over a gate / up pair
+        M = 21
+        r = torch.from_numpy(synth.activations(35, M, N)).cuda()
+        y = _run(backend, qw, x[:M].contiguous())
+        y2 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        backend.matmul_ex(qw, x[:M].contiguous(), y2, "add", r)
+        torch.cuda.synchronize()
+        assert torch.equal(y2, y + r)
+        h = N // 2
+        g = backend.upload_quantized(q[:h], s[:h], bits)
+        u = backend.upload_quantized(q[h:], s[h:], bits)
+        pair = backend.fuse_pairs(g, u)
+        y3 = torch.empty((M, h), dtype=torch.float32, device="cuda")
+        backend.matmul_ex(pair, x[:M].contiguous(), y3, "swiglu")
+        torch.cuda.synchronize()
+        yd = y.double()
+        ref = torch.nn.functional.silu(yd[:, :h]) * yd[:, h:]
+        assert ((y3.double() - ref).norm() / ref.norm()).item() < TIGHT
 
 
 def test_decode_long_k_uses_several_slabs(backend, oracle):
