@@ -201,9 +201,10 @@ def main():
         run(plans[key])
         cursor[0] = (cursor[0] + n) % copies
 
-    def prepare(n):
-        """Builds the plans the next walks of n steps will need (a walk's start only depends on n mod copies)."""
-        c = cursor[0]
+    def prepare(n, after=0):
+        """Builds the plans the next walks of n steps will need (a walk's start only depends on n mod
+        copies); after: steps that will be walked before them."""
+        c = (cursor[0] + after) % copies
         for _ in range(copies):
             if (n, c) not in plans:
                 plans[(n, c)] = plan_of(n, c)
@@ -214,9 +215,12 @@ def main():
     flush.fill_(1)
     torch.cuda.synchronize()
     del flush
+    # (every plan is built before the warm-up: the timed passes follow it without the device idling
+    # through host work in between)
+    prepare(args.steps, after=args.warmup)
     if args.warmup > 0:
+        plans[(args.warmup, cursor[0])] = plan_of(args.warmup, cursor[0])
         walk(args.warmup, lambda p: be.matmul_many(p, M, stream))
-    prepare(args.steps)
     mean_pass, passes = timer.until(lambda i: walk(args.steps, lambda p: be.matmul_many(p, M, stream)))
     us = mean_pass / args.steps * 1e6
     gbs = alg_bytes / (mean_pass / args.steps) / 1e9

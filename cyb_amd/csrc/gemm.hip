@@ -193,15 +193,18 @@ __device__ __forceinline__ float4_t mma(const Frag16& a, const Frag16& b, float4
 // XBF = 1: X is bf16, 0: X is f16.  EXACT: see the header comment.
 // Wave wv of WAVES owns MF row blocks of 16 against all NF column blocks.
 template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kernel(WeightView w, const u32x4_t* __restrict__ x, int x_row_blocks, int M,
-                                                   void* __restrict__ y, int ydt, int n_tiles, int m_tiles, float out_scale,
-                                                   float* __restrict__ part, int splits, int kt_per_split, Epilogue epi, NormStats ns)
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kernel(const uint8_t* __restrict__ wbase, const u32x4_t* __restrict__ x, int KT_, int NT_, int x_row_blocks, int M,
+                                                   int n_tiles, int m_tiles, int splits, int kt_per_split, int groups, int N_,
+                                                   void* __restrict__ y, int ydt, int K_, float out_scale,
+                                                   float* __restrict__ part, Epilogue epi, NormStats ns)
 {
+    // (leading scalar arguments in the order of their first use: they arrive in registers at wave start)
+    const WeightView w = {wbase, N_, K_, NT_, KT_, BITS};
     // Workgroups are handed to the 8 XCDs round-robin (id % 8) and every XCD has
     // its own L2.  Give each XCD a contiguous run of tiles in row-block-major
     // order, so the workgroups sharing an L2 read the same rows of X and X is
     // fetched into every L2 once instead of once per column tile.
-    const int per_xcd = (int)gridDim.x >> 3;
+    const int per_xcd = groups >> 3;
     const int item = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
     if (item >= n_tiles * m_tiles * splits) return;
     // split-major: workgroups that run side by side share a K range of X
@@ -497,8 +500,8 @@ hipError_t launch_m(const WeightView& w, const void* x, int M, void* y, int ydt,
     const int kt_per_split = (w.KT + splits - 1) / splits;
     splits = (w.KT + kt_per_split - 1) / kt_per_split;          // no empty split
     const unsigned groups = (unsigned)((tiles * splits + 7) / 8 * 8);
-    hipLaunchKernelGGL(kern, dim3(groups), dim3(WAVES * 64), lds, st, w, reinterpret_cast<const u32x4_t*>(x), (M + 15) / 16, M,
-                       y, ydt, n_tiles, m_tiles, out_scale, part, splits, kt_per_split, epi, ns);
+    hipLaunchKernelGGL(kern, dim3(groups), dim3(WAVES * 64), lds, st, w.base, reinterpret_cast<const u32x4_t*>(x), w.KT, w.NT,
+                       (M + 15) / 16, M, n_tiles, m_tiles, splits, kt_per_split, (int)groups, w.N, y, ydt, w.K, out_scale, part, epi, ns);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || splits == 1) return e;
     const int64_t total = (int64_t)M * w.N;
