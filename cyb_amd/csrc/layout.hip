@@ -27,11 +27,36 @@ __device__ __forceinline__ int staged_weight(const uint8_t* row, int gl, int i)
     return (int)((i < 16) ? (b & 15) : (b >> 4)) - 8;
 }
 
+// A lane's share of one scale group (the 8 weights k = 8 * oct + s of row `row`) as eight
+// offset-8 nibbles in native order within a word pair: weight s sits in byte {0, 2, 1, 3}[s & 3]
+// of word s >> 2, low nibble (the caller shifts odd groups into the high nibbles).
+template <int LAYOUT>
+__device__ __forceinline__ void staged_q4_octet(const uint8_t* row, int gl, int oct, uint32_t& lo, uint32_t& hi)
+{
+    if (LAYOUT == 0) {
+        // PLANAR: weight i is nibble i of the group's 16 bytes (two's complement): one aligned word
+        const uint32_t src = *reinterpret_cast<const uint32_t*>(row + gl * 16 + oct * 4) ^ 0x88888888u;
+        const uint32_t a = src & 0xffffu, b = src >> 16;
+        lo = (a & 0x0f0fu) | (((a >> 4) & 0x0f0fu) << 16);
+        hi = (b & 0x0f0fu) | (((b >> 4) & 0x0f0fu) << 16);
+    } else {
+        // BLOCK_AOS: weights 0..15 are the low nibbles of the 16 bytes behind the f16 scale, 16..31
+        // the high nibbles (already offset-8); the bytes are only 2-byte aligned
+        const uint16_t* p = reinterpret_cast<const uint16_t*>(row + gl * 18 + 2 + (oct & 1) * 8);
+        const uint32_t w0 = (uint32_t)p[0] | ((uint32_t)p[1] << 16), w1 = (uint32_t)p[2] | ((uint32_t)p[3] << 16);
+        const int sh = (oct >> 1) * 4;
+        const uint32_t t0 = (w0 >> sh) & 0x0f0f0f0fu, t1 = (w1 >> sh) & 0x0f0f0f0fu;
+        lo = __builtin_amdgcn_perm(t0, t0, 0x03010200u);       // bytes 1 and 2 change places
+        hi = __builtin_amdgcn_perm(t1, t1, 0x03010200u);
+    }
+}
+
 // One workgroup repacks CT consecutive K tiles of one 16-row strip.  The source rows of
 // that piece are first copied into LDS with coalesced loads (a row's piece is one
 // contiguous run in either interchange layout), then every thread assembles one lane's
-// share of a native tile from LDS and stores it with 128-bit stores: global memory only
-// sees whole runs, the byte-granular gathering stays inside the CU.
+// share of a native tile from LDS - a few aligned words and a handful of bit operations -
+// and stores it with 128-bit stores: global memory only sees whole runs, the gathering
+// stays inside the CU.
 constexpr int kRepackTiles = 4;
 
 template <int BITS, int LAYOUT>
@@ -41,9 +66,10 @@ __global__ __launch_bounds__(256) void repack_kernel(const uint8_t* __restrict__
     constexpr int CT = kRepackTiles;
     constexpr int GB = kSrcGroupBytes<BITS, LAYOUT>;
     constexpr int ROWB = CT * kGroupsPerTile * GB;                  // bytes of one row's piece
-    constexpr int UNIT = LAYOUT == 0 ? 4 : 2;                       // load width the source alignment allows
+    constexpr int UNIT = LAYOUT == 0 ? 16 : 2;                      // load width the source alignment allows
     constexpr int UPR = ROWB / UNIT;                                // units per row
-    __shared__ __attribute__((aligned(16))) uint8_t rows[kTileN][ROWB];
+    constexpr int PITCH = ROWB + (LAYOUT == 0 ? 16 : 4);            // (rows land in different LDS banks)
+    __shared__ __attribute__((aligned(16))) uint8_t rows[kTileN][PITCH];
 
     const int t = threadIdx.x;
     const int chunks = (KT + CT - 1) / CT;
@@ -56,7 +82,7 @@ __global__ __launch_bounds__(256) void repack_kernel(const uint8_t* __restrict__
         const int64_t n = (int64_t)nt * kTileN + r;
         if (n < N && u * UNIT < ng * GB) {
             const uint8_t* src = q + (n * G + g0) * GB + u * UNIT;
-            if (UNIT == 4) *reinterpret_cast<uint32_t*>(&rows[r][u * 4]) = *reinterpret_cast<const uint32_t*>(src);
+            if (UNIT == 16) *reinterpret_cast<u32x4_t*>(&rows[r][u * 16]) = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(src));
             else *reinterpret_cast<uint16_t*>(&rows[r][u * 2]) = *reinterpret_cast<const uint16_t*>(src);
         }
     }
@@ -73,12 +99,10 @@ __global__ __launch_bounds__(256) void repack_kernel(const uint8_t* __restrict__
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int gl = b * 4 + j;
-            const bool ok = row_ok && gl < ng;
-#pragma unroll
-            for (int s = 0; s < 8; s++) {
-                const int v = ok ? staged_weight<4, LAYOUT>(rows[row], gl, oct * 8 + s) : 0;
-                w[q4_word(j, s)] |= (uint32_t)((v + 8) & 15) << q4_shift(j, s);
-            }
+            uint32_t lo = 0x08080808u, hi = 0x08080808u;             // q = 0 where the source has nothing
+            if (row_ok && gl < ng) staged_q4_octet<LAYOUT>(rows[row], gl, oct, lo, hi);
+            w[2 * (j >> 1)] |= lo << (4 * (j & 1));
+            w[2 * (j >> 1) + 1] |= hi << (4 * (j & 1));
         }
         reinterpret_cast<u32x4_t*>(tile)[lane] = (u32x4_t){w[0], w[1], w[2], w[3]};
     } else {
