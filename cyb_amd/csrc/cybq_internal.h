@@ -21,14 +21,14 @@ hipError_t launch_dequant(const WeightView& w, float* out, hipStream_t st);
 // decode path, 1 <= M <= 16 per call, and 17 .. 32 rows where gemv_serves_32 says so (api.hip
 // walks the other 17..32-row calls 16 rows at a time)
 bool gemv_serves_32(int xdt, int M, const Epilogue& epi);
-// exact_operands: keep the weight operands exact integers for one f16 row too (the LDS kernel)
-// instead of the subnormal-operand kernel of gemv1.hip
+// exact_operands: keep the weight operands exact integers for one and two f16 rows too (the LDS
+// kernel) instead of the subnormal-operand kernel of gemv1.hip
 hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
                        int num_cus, bool exact_operands, const Epilogue& epi, hipStream_t st);
-// one-row decode kernel (f16 activations, no folded norm): weight operands are f16 subnormals,
+// decode kernel for one and two rows (f16 activations, no folded norm): weight operands are f16 subnormals,
 // the +8 / +128 bias comes off inside the MFMA accumulation (gemv1.hip)
 bool gemv1_serves(const WeightView& w, int xdt, int M, const Epilogue& epi);
-hipError_t launch_gemv1(const WeightView& w, const void* x, void* y, int ydt, const Epilogue& epi, hipStream_t st);
+hipError_t launch_gemv1(const WeightView& w, const void* x, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st);
 // prefill path (api.hip sends 16-bit activations with M > 32 here)
 // exact: two MFMAs per group with losslessly split weights; otherwise one f16 MFMA
 // per group with weights rounded once to f16

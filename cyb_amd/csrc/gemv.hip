@@ -1010,10 +1010,10 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
     // more if that is what it takes to bring a wave's share down to 8 tiles, all requested
     // up front.  (K = 4096 is 4 waves x 8 tiles for every N: with few strips 8 waves x 4 tiles
     // measured 2 - 4 % slower.)
-    // one f16 row: the kernel of gemv1.hip (unless the caller asked for exact integer weight
+    // one or two f16 rows: the kernel of gemv1.hip (unless the caller asked for exact integer weight
     // operands, or a test forces one of the kernels below)
     if (!exact_operands && g_tune_waves == 0 && g_tune_rows == 0 && g_tune_unroll == 0 && gemv1_serves(w, xdt, M, epi))
-        return launch_gemv1(w, x, y, ydt, epi, st);
+        return launch_gemv1(w, x, M, y, ydt, epi, st);
     int nwaves = g_tune_waves;
     if (nwaves <= 0) {
         nwaves = 2;

@@ -1,4 +1,5 @@
-// gemv1.hip - decode kernel for ONE activation row: y[1,N] = x[1,K] * W^T, f16 activations.
+// gemv1.hip - decode kernel for one or two activation rows: y[M,N] = x[M,K] * W^T, f16 activations.
+// (Described for one row; the two-row form is at the kernel's template parameters.)
 //
 // HBM-bound: a workgroup owns one 16-row strip of W (one contiguous run of memory) and
 // requests all of it up front; everything else is arranged so that nothing stands between
@@ -69,19 +70,29 @@ __device__ __forceinline__ Frag16 sub_operand(const u32x4_t (&q)[BITS == 4 ? 1 :
 // SPLIT (NS = 2, NW > 0): the workgroup has 2 * NW waves, waves [0, NW) take the gate strip and
 // [NW, 2 NW) the up strip - per wave the same work as with one strip per workgroup (a wave that
 // holds both strips' tiles has twice the requests in flight and half the waves to hide them).
-// RES: the residual-add epilogue; the residual is requested first of all, so that it is there long
-// before the sums are (asked for at the end it would cost the kernel one more trip to memory).
-template <int BITS, int SETS, int NS, bool EVEN, int NW, bool SPLIT = false, bool RES = false>
+// RES (MR = 1): the residual-add epilogue; the residual is requested first of all, so that it is there
+// long before the sums are (asked for at the end it would cost the kernel one more trip to memory).
+// MR: batch rows, 1 or 2.  The 16 rows of an A operand are MR batch rows x 16 / MR scale groups:
+// an operand covers 4 / MR tiles of a set, a set takes MR operand loads and MR scale loads per lane,
+// and lane block b ends up with batch row b / (4 / MR) and the tiles t = b mod (4 / MR), + 4 / MR, ...
+// of the set.  (The scheme works for four rows as well - 12 load instructions per set instead of 6 -
+// and was measured slower there than the batched-rows kernel: 8.8 against 8.6 us at 4096 -> 14336.)
+template <int BITS, int SETS, int NS, bool EVEN, int NW, bool SPLIT = false, bool RES = false, int MR = 1>
 // The arguments are scalars in the order the kernel needs them: the compiler is asked to have
 // them delivered in registers at wave start (kernel argument preload), so the first requests do
-// not wait for a load of the argument block.
-// (14 dwords; the launch's wave count travels with them, the launch geometry is not among what is preloaded.)
+// not wait for a load of the argument block.  (13 dwords; the launch's wave count travels with
+// them, the launch geometry is not among what is preloaded.  flags = output type | epilogue << 4 | M << 8.)
 __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__ wbase, const _Float16* __restrict__ x,
                                                      const void* __restrict__ residual, void* __restrict__ y, int KT, int K,
-                                                     int launch_waves, int n_rows, int out_dt, int epi_kind)
+                                                     int launch_waves, int n_rows, int flags)
 {
+    static_assert(MR == 1 || MR == 2, "batch rows per operand");
+    static_assert(!RES || MR == 1, "the residual prefetch is the one-row form");
     constexpr int QV = BITS == 4 ? 1 : 2;
-    __shared__ float red[NS * 16 * 16];
+    constexpr int GPA = 16 / MR;                  // scale groups per A operand
+    constexpr int TPA = 4 / MR;                   // tiles per A operand
+    __shared__ float red[NS * MR * 16 * 16];
+    const int out_dt = flags & 15, epi_kind = (flags >> 4) & 15, M = flags >> 8;
     const int tid = threadIdx.x, lane = tid & 63;
     static_assert(!SPLIT || (NS == 2 && NW > 0), "split workgroups are gate / up pairs with a known wave count");
     constexpr int NL = SPLIT ? 1 : NS;            // strips a wave works on
@@ -93,6 +104,7 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
     }
     const int nwaves = NW ? NW : launch_waves;          // NW = 0: whatever the launch says
     const int row = lane & 15, blk = lane >> 4;
+    const int my_tile = blk % TPA;                // the tiles of a set this lane block ends up with: my_tile + TPA * c
 
     uint32_t res_word = 0;            // the aligned 32-bit word that holds this lane's residual element
     uint32_t res_addr = 0;
@@ -102,19 +114,27 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
         res_addr = (uint32_t)p;
         res_word = *reinterpret_cast<const uint32_t*>(p & ~(uintptr_t)3);
     }
-    Frag16 a[SETS];
-    u32x2_t sc[NL][SETS];
+    // A row i of an operand: batch row i / GPA (rows past M repeat the last one, their sums are not stored),
+    // scale group i % GPA of the operand's tiles
+    const _Float16* xrow = x;
+    if constexpr (MR > 1) xrow += min(row / GPA, M - 1) * K;
+    const int xk = (row % GPA) * 32 + blk * 8;
+    Frag16 a[SETS][MR];
+    u32x2_t sc[NL][SETS][MR];
     u32x4_t q[NL][SETS][4][QV];
-    bool tile_ok[SETS];               // this lane block's tile of the set exists (!EVEN)
+    bool tile_ok[SETS][MR];           // this lane block's tiles of the set exist (!EVEN)
 #pragma unroll
     for (int h = 0; h < SETS; h++) {
         const int set = wv + nwaves * h;
-        const int k = set * 512 + row * 32 + blk * 8;
-        if (EVEN) {
-            a[h].u = *reinterpret_cast<const u32x4_t*>(x + k);
-        } else {
-            a[h].u = *reinterpret_cast<const u32x4_t*>(x + min(k, K - 8));
-            tile_ok[h] = 4 * set + blk < KT;
+#pragma unroll
+        for (int p = 0; p < MR; p++) {
+            const int k = set * 512 + p * (TPA * 128) + xk;
+            if (EVEN) {
+                a[h][p].u = *reinterpret_cast<const u32x4_t*>(xrow + k);
+            } else {
+                a[h][p].u = *reinterpret_cast<const u32x4_t*>(xrow + min(k, K - 8));
+                tile_ok[h][p] = 4 * set + my_tile + TPA * p < KT;
+            }
         }
     }
     // Addresses: one wave-uniform 64-bit base per (strip, set) plus a 32-bit lane offset, so the
@@ -130,7 +150,10 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
             const int t0 = 4 * (wv + nwaves * h);
             if (EVEN) {
                 const uint8_t* sb = wbase + (int64_t)(strip_tile + t0) * TB;
-                sc[st][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(sb + ((uint32_t)blk * TB + lane_s)));
+#pragma unroll
+                for (int c = 0; c < MR; c++)
+                    sc[st][h][c] = __builtin_nontemporal_load(
+                        reinterpret_cast<const u32x2_t*>(sb + ((uint32_t)(my_tile + TPA * c) * TB + lane_s)));
 #pragma unroll
                 for (int b = 0; b < 4; b++)
 #pragma unroll
@@ -138,8 +161,10 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
                         q[st][h][b][v] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(sb + (b * TB + v * 1024) + lane_q));
             } else {
                 const uint8_t* strip = wbase + (int64_t)strip_tile * TB;
-                sc[st][h] = __builtin_nontemporal_load(
-                    reinterpret_cast<const u32x2_t*>(strip + ((uint32_t)min(t0 + blk, KT - 1) * TB + lane_s)));
+#pragma unroll
+                for (int c = 0; c < MR; c++)
+                    sc[st][h][c] = __builtin_nontemporal_load(
+                        reinterpret_cast<const u32x2_t*>(strip + ((uint32_t)min(t0 + my_tile + TPA * c, KT - 1) * TB + lane_s)));
 #pragma unroll
                 for (int b = 0; b < 4; b++) {
                     const uint8_t* tp = strip + (int64_t)min(t0 + b, KT - 1) * TB;
@@ -150,25 +175,27 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
             }
         }
     }
-    // Everything the tail needs from the kernel arguments is fetched now, next to the requests:
-    // left to itself the compiler loads each argument where it is first used, i.e. after the
-    // final barrier, and the kernel would end with two more round trips to memory.
-    asm volatile("" ::"s"(n_rows), "s"(out_dt), "s"(epi_kind), "s"(residual), "s"(y));
+    // Everything the tail needs from the kernel arguments is kept live from here on: left to
+    // itself the compiler fetches an argument where it is first used, i.e. after the final barrier.
+    asm volatile("" ::"s"(n_rows), "s"(out_dt), "s"(epi_kind), "s"(residual), "s"(y), "s"(M));
     if (!NW) asm volatile("" ::"s"(nwaves));
     __builtin_amdgcn_sched_barrier(0);       // every request is out before any arithmetic
 
     if (!EVEN) {
 #pragma unroll
         for (int h = 0; h < SETS; h++) {
-            // activations past K (the padded tail of the last tile) count as zero; a tile past
-            // the end of the strip was clamped to the last one and gets scale zero
-            const bool x_ok = (wv + nwaves * h) * 512 + row * 32 + blk * 8 < K;
 #pragma unroll
-            for (int p = 0; p < 4; p++) a[h].u[p] = x_ok ? a[h].u[p] : 0u;
+            for (int p = 0; p < MR; p++) {
+                // activations past K (the padded tail of the last tile) count as zero; a tile past
+                // the end of the strip was clamped to the last one and gets scale zero
+                const bool x_ok = (wv + nwaves * h) * 512 + p * (TPA * 128) + xk < K;
 #pragma unroll
-            for (int st = 0; st < NL; st++) {
-                sc[st][h][0] = tile_ok[h] ? sc[st][h][0] : 0u;
-                sc[st][h][1] = tile_ok[h] ? sc[st][h][1] : 0u;
+                for (int e = 0; e < 4; e++) a[h][p].u[e] = x_ok ? a[h][p].u[e] : 0u;
+#pragma unroll
+                for (int st = 0; st < NL; st++) {
+                    sc[st][h][p][0] = tile_ok[h][p] ? sc[st][h][p][0] : 0u;
+                    sc[st][h][p][1] = tile_ok[h][p] ? sc[st][h][p][1] : 0u;
+                }
             }
         }
     }
@@ -179,22 +206,24 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
     kL.u = (u32x4_t){kSubBiasL, kSubBiasL, kSubBiasL, kSubBiasL};
     kH.u = (u32x4_t){cH, cH, cH, cH};
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
-    float4_t biasL[SETS], biasH[SETS];
+    float4_t biasL[SETS][MR], biasH[SETS][MR];
 #pragma unroll
-    for (int h = 0; h < SETS; h++) {
-        if (BITS == 4) biasL[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[h].h, kL.h, zero, 0, 0, 0);
-        biasH[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[h].h, kH.h, zero, 0, 0, 0);
-    }
+    for (int h = 0; h < SETS; h++)
+#pragma unroll
+        for (int p = 0; p < MR; p++) {
+            if (BITS == 4) biasL[h][p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[h][p].h, kL.h, zero, 0, 0, 0);
+            biasH[h][p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[h][p].h, kH.h, zero, 0, 0, 0);
+        }
 
-    // Lane block b holds meaningful sums only for tile b of every set.  All four tiles are
-    // accumulated with the lane's own scales (the other three sums are finite and unused) and the
-    // meaningful one is picked once at the end.  Even groups (low nibbles) and odd groups
-    // (high nibbles, 16 times too large) are kept apart until the final scaling.
-    float accL[NL][4], accH[NL][4];
+    // A lane block holds meaningful sums only for its own tiles of every set (one in TPA).  All
+    // tiles are accumulated with the lane's own scales, TPA sums side by side (the others are
+    // finite and unused), and the meaningful one is picked once at the end.  Even groups (low
+    // nibbles) and odd groups (high nibbles, 16 times too large) are kept apart until the final scaling.
+    float accL[NL][TPA], accH[NL][TPA];
 #pragma unroll
     for (int st = 0; st < NL; st++)
 #pragma unroll
-        for (int b = 0; b < 4; b++) accL[st][b] = accH[st][b] = 0.f;
+        for (int b = 0; b < TPA; b++) accL[st][b] = accH[st][b] = 0.f;
     constexpr int T = NL * SETS * 4;
     float4_t dprev[4];
 #pragma unroll
@@ -202,21 +231,21 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
         // MFMAs of tile i first, then the scaling of tile i - 1 whose results have landed meanwhile
         float4_t d[4];
         if (i < T) {
-            const int st = i / (SETS * 4), h = (i / 4) % SETS, b = i % 4;
+            const int st = i / (SETS * 4), h = (i / 4) % SETS, b = i % 4, p = b / TPA;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const Frag16 B = sub_operand<BITS>(q[st][h][b], r);
-                d[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[h].h, B.h, (BITS == 8 || (r & 1)) ? biasH[h] : biasL[h], 0, 0, 0);
+                d[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[h][p].h, B.h, (BITS == 8 || (r & 1)) ? biasH[h][p] : biasL[h][p], 0, 0, 0);
             }
         }
         if (i > 0) {
-            const int st = (i - 1) / (SETS * 4), h = ((i - 1) / 4) % SETS, b = (i - 1) % 4;
+            const int st = (i - 1) / (SETS * 4), h = ((i - 1) / 4) % SETS, b = (i - 1) % 4, p = b / TPA, slot = b % TPA;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const uint32_t sb = (r & 1) ? (sc[st][h][r >> 1] >> 16) : (sc[st][h][r >> 1] & 0xffffu);
+                const uint32_t sb = (r & 1) ? (sc[st][h][p][r >> 1] >> 16) : (sc[st][h][p][r >> 1] & 0xffffu);
                 const float sf = f16_bits_to_f32(sb);
-                if (BITS == 4 && (r & 1)) accH[st][b] = __builtin_fmaf(sf, dprev[r][r], accH[st][b]);
-                else accL[st][b] = __builtin_fmaf(sf, dprev[r][r], accL[st][b]);
+                if (BITS == 4 && (r & 1)) accH[st][slot] = __builtin_fmaf(sf, dprev[r][r], accH[st][slot]);
+                else accL[st][slot] = __builtin_fmaf(sf, dprev[r][r], accL[st][slot]);
             }
         }
 #pragma unroll
@@ -224,123 +253,172 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
         __builtin_amdgcn_sched_barrier(0);
     }
 
-    // Blocks meet inside the matrix pipe: with B[k = block][n] = the block's sum and A = ones, a
-    // 16x16x4 fp32 MFMA leaves sum_k B[k][n] in every row - one instruction instead of two
-    // cross-lane round trips.  Waves meet through LDS; the last sum is the same trick again: lane
-    // block j adds the partial sums of waves 4i + j in order of i, the MFMA adds the four blocks.
+    // Blocks meet inside the matrix pipe: with B[k = block][n] = the block's sum and A[m][k] = 1 where
+    // block k belongs to batch row m, a 16x16x4 fp32 MFMA leaves sum_k B[k][n] in row m - one
+    // instruction instead of two cross-lane round trips.  Waves meet through LDS; the last sum is the
+    // same trick again: lane block j adds the partial sums of waves 4i + j in order of i, the MFMA
+    // adds the four blocks.
     const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+    const float mine = (MR == 1 || blk / TPA == row) ? 1.0f : 0.0f;
 #pragma unroll
     for (int st = 0; st < NL; st++) {
-        float tb[4];
+        float tb[TPA];
 #pragma unroll
-        for (int b = 0; b < 4; b++) tb[b] = BITS == 4 ? accL[st][b] + accH[st][b] * 0.0625f : accL[st][b];
-        const float t = blk == 0 ? tb[0] : (blk == 1 ? tb[1] : (blk == 2 ? tb[2] : tb[3]));
-        const float4_t sum = __builtin_amdgcn_mfma_f32_16x16x4f32(1.0f, t, zero4, 0, 0, 0);
-        if (lane < 16) red[((st + half) * 16 + wv) * 16 + lane] = sum[0];
+        for (int b = 0; b < TPA; b++) tb[b] = BITS == 4 ? accL[st][b] + accH[st][b] * 0.0625f : accL[st][b];
+        float t = tb[0];
+#pragma unroll
+        for (int b = 1; b < TPA; b++) t = my_tile == b ? tb[b] : t;
+        const float4_t sum = __builtin_amdgcn_mfma_f32_16x16x4f32(mine, t, zero4, 0, 0, 0);
+        if (lane < 16) {
+#pragma unroll
+            for (int m = 0; m < MR; m++) red[(((st + half) * MR + m) * 16 + wv) * 16 + lane] = sum[m];
+        }
     }
     __syncthreads();
     if (tid >= 64) return;
     constexpr int SLOTS = NW ? (NW + 3) / 4 : 4;
-    float outv[NS];
+    float outv[NS][MR];
 #pragma unroll
-    for (int st = 0; st < NS; st++) {
-        float t[SLOTS];
+    for (int st = 0; st < NS; st++)
 #pragma unroll
-        for (int i = 0; i < SLOTS; i++) t[i] = red[(st * 16 + min(4 * i + blk, 15)) * 16 + row];
-        float v = 0.f;
+        for (int m = 0; m < MR; m++) {
+            float t[SLOTS];
 #pragma unroll
-        for (int i = 0; i < SLOTS; i++) v += 4 * i + blk < nwaves ? t[i] : 0.f;
-        outv[st] = __builtin_amdgcn_mfma_f32_16x16x4f32(1.0f, v, zero4, 0, 0, 0)[0] * unscale;
-    }
+            for (int i = 0; i < SLOTS; i++) t[i] = red[((st * MR + m) * 16 + min(4 * i + blk, 15)) * 16 + row];
+            float v = 0.f;
+#pragma unroll
+            for (int i = 0; i < SLOTS; i++) v += 4 * i + blk < nwaves ? t[i] : 0.f;
+            outv[st][m] = __builtin_amdgcn_mfma_f32_16x16x4f32(1.0f, v, zero4, 0, 0, 0)[0] * unscale;
+        }
     if (lane >= 16) return;
     const int n = blockIdx.x * 16 + lane;
     if (NS == 2) {               // SwiGLU: strips 2i / 2i+1 are gate / up of output strip i
-        if (n < (n_rows >> 1)) store_out1(y, out_dt, n, silu_mul(outv[0], outv[NS - 1]));
+        const int n_out = n_rows >> 1;
+#pragma unroll
+        for (int m = 0; m < MR; m++)
+            if (m < M && n < n_out) store_out1(y, out_dt, (int64_t)m * n_out + n, silu_mul(outv[0][m], outv[NS - 1][m]));
         return;
     }
     if (n < n_rows) {
-        float v = outv[0];
-        if constexpr (RES) {
-            const uint32_t h = (res_addr & 2u) ? res_word >> 16 : res_word & 0xffffu;
-            v += out_dt == kF32 ? __builtin_bit_cast(float, res_word)
-                                : (out_dt == kF16 ? f16_bits_to_f32(h) : __builtin_bit_cast(float, h << 16));
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+            float v = outv[0][m];
+            if constexpr (RES) {
+                const uint32_t h = (res_addr & 2u) ? res_word >> 16 : res_word & 0xffffu;
+                v += out_dt == kF32 ? __builtin_bit_cast(float, res_word)
+                                    : (out_dt == kF16 ? f16_bits_to_f32(h) : __builtin_bit_cast(float, h << 16));
+            } else if (MR > 1 && epi_kind == kEpiAdd) {
+                if (m < M) v += load_out1(residual, out_dt, (int64_t)m * n_rows + n);
+            }
+            if (m < M) store_out1(y, out_dt, (int64_t)m * n_rows + n, v);
         }
-        store_out1(y, out_dt, n, v);
     }
 }
 
-template <int BITS, int SETS, int NS>
-hipError_t launch1_e(const WeightView& w, const void* x, void* y, int ydt, int nwaves, bool even, const Epilogue& epi,
+// sets of four K tiles a wave may own (all of them in registers, 16 waves per workgroup at
+// most: 128 registers per lane): two, three for Q4 with one strip per workgroup, one for
+// Q8 gate / up pairs; with two batch rows per operand two (Q4, one strip) or one
+constexpr int max_sets_per_wave(int bits, int ns, int mr)
+{
+    if (mr == 1) return bits == 4 ? (ns == 1 ? 3 : 2) : (ns == 1 ? 2 : 1);
+    return bits == 4 && ns == 1 ? 2 : 1;
+}
+
+struct Shape1 {        // how a strip's K is split over waves
+    int per_wave, nwaves;
+    bool even, k8;
+};
+
+Shape1 shape_of(const WeightView& w)
+{
+    const int nsets = (w.KT + 3) / 4;
+    Shape1 s;
+    s.per_wave = (nsets + 15) / 16;
+    s.nwaves = (nsets + s.per_wave - 1) / s.per_wave;
+    s.even = w.K % 512 == 0 && nsets % s.nwaves == 0;
+    s.k8 = s.even && s.nwaves == 8 && s.per_wave == 1;          // K = 4096: the shape most decode launches have
+    return s;
+}
+
+template <int BITS, int SETS, int NS, int MR>
+hipError_t launch1_e(const WeightView& w, const void* x, int M, void* y, int ydt, const Shape1& sh, const Epilogue& epi,
                      hipStream_t st)
 {
+    const int nwaves = sh.nwaves;
     const dim3 grid((unsigned)(w.NT / NS)), block((unsigned)nwaves * 64);
     const _Float16* xh = reinterpret_cast<const _Float16*>(x);
-#define CYBQ_GEMV1_LAUNCH(EVEN_, NW_, SPLIT_, RES_, BLOCK_)                                                                             \
-    hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, EVEN_, NW_, SPLIT_, RES_>), grid, BLOCK_, 0, st, w.base, xh, epi.residual, y, w.KT, w.K, nwaves, \
-                       w.N, ydt, epi.kind)
-    const bool k8 = even && nwaves == 8 && SETS == 1;          // K = 4096: the shape most decode launches have
+    const int flags = ydt | (epi.kind << 4) | (M << 8);
+#define CYBQ_GEMV1_LAUNCH(EVEN_, NW_, SPLIT_, RES_, BLOCK_)                                                                          \
+    hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, EVEN_, NW_, SPLIT_, RES_, MR>), grid, BLOCK_, 0, st, w.base, xh, epi.residual, y, \
+                       w.KT, w.K, nwaves, w.N, flags)
+    const bool k8 = sh.k8 && SETS == 1;
     if constexpr (NS == 2) {
         if constexpr (SETS == 1) {
             if (k8) CYBQ_GEMV1_LAUNCH(true, 8, true, false, dim3(1024));
-            else if (even) CYBQ_GEMV1_LAUNCH(true, 0, false, false, block);
+            else if constexpr (MR > 1) return hipErrorInvalidValue;        // gemv1_serves() said no
+            else if (sh.even) CYBQ_GEMV1_LAUNCH(true, 0, false, false, block);
             else CYBQ_GEMV1_LAUNCH(false, 0, false, false, block);
-        } else {
-            if (even) CYBQ_GEMV1_LAUNCH(true, 0, false, false, block);
+        } else if constexpr (MR == 1) {
+            if (sh.even) CYBQ_GEMV1_LAUNCH(true, 0, false, false, block);
             else CYBQ_GEMV1_LAUNCH(false, 0, false, false, block);
+        } else return hipErrorInvalidValue;
+    } else if (MR == 1 && epi.kind == kEpiAdd) {
+        if constexpr (MR == 1) {
+            if (k8) CYBQ_GEMV1_LAUNCH(true, (SETS == 1 ? 8 : 0), false, true, block);
+            else if (sh.even) CYBQ_GEMV1_LAUNCH(true, 0, false, true, block);
+            else CYBQ_GEMV1_LAUNCH(false, 0, false, true, block);
         }
-    } else if (epi.kind == kEpiAdd) {
-        if (k8) CYBQ_GEMV1_LAUNCH(true, (SETS == 1 ? 8 : 0), false, true, block);
-        else if (even) CYBQ_GEMV1_LAUNCH(true, 0, false, true, block);
-        else CYBQ_GEMV1_LAUNCH(false, 0, false, true, block);
     } else {
         if (k8) CYBQ_GEMV1_LAUNCH(true, (SETS == 1 ? 8 : 0), false, false, block);
-        else if (even) CYBQ_GEMV1_LAUNCH(true, 0, false, false, block);
+        else if (sh.even) CYBQ_GEMV1_LAUNCH(true, 0, false, false, block);
         else CYBQ_GEMV1_LAUNCH(false, 0, false, false, block);
     }
 #undef CYBQ_GEMV1_LAUNCH
     return hipGetLastError();
 }
 
-// sets of four K tiles a wave may own (all of them in registers, 16 waves per workgroup at
-// most: 128 registers per lane): two, three for Q4 with one strip per workgroup, one for
-// Q8 gate / up pairs
-constexpr int max_sets_per_wave(int bits, int ns) { return bits == 4 ? (ns == 1 ? 3 : 2) : (ns == 1 ? 2 : 1); }
-
-template <int BITS, int NS>
-hipError_t launch1_s(const WeightView& w, const void* x, void* y, int ydt, const Epilogue& epi, hipStream_t st)
+template <int BITS, int NS, int MR>
+hipError_t launch1_s(const WeightView& w, const void* x, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st)
 {
-    const int nsets = (w.KT + 3) / 4;
-    const int per_wave = (nsets + 15) / 16;
-    const int nwaves = (nsets + per_wave - 1) / per_wave;
-    const bool even = w.K % 512 == 0 && nsets % nwaves == 0;
-    constexpr int MAXS = max_sets_per_wave(BITS, NS);
-    if (per_wave == 1) return launch1_e<BITS, 1, NS>(w, x, y, ydt, nwaves, even, epi, st);
+    const Shape1 sh = shape_of(w);
+    constexpr int MAXS = max_sets_per_wave(BITS, NS, MR);
+    if (sh.per_wave == 1) return launch1_e<BITS, 1, NS, MR>(w, x, M, y, ydt, sh, epi, st);
     if constexpr (MAXS >= 2) {
-        if (per_wave == 2) return launch1_e<BITS, 2, NS>(w, x, y, ydt, nwaves, even, epi, st);
+        if (sh.per_wave == 2) return launch1_e<BITS, 2, NS, MR>(w, x, M, y, ydt, sh, epi, st);
     }
     if constexpr (MAXS >= 3) {
-        if (per_wave == 3) return launch1_e<BITS, 3, NS>(w, x, y, ydt, nwaves, even, epi, st);
+        if (sh.per_wave == 3) return launch1_e<BITS, 3, NS, MR>(w, x, M, y, ydt, sh, epi, st);
     }
     return hipErrorInvalidValue;         // gemv1_serves() said no
+}
+
+template <int BITS, int NS>
+hipError_t launch1_m(const WeightView& w, const void* x, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st)
+{
+    if (M == 1) return launch1_s<BITS, NS, 1>(w, x, M, y, ydt, epi, st);
+    return launch1_s<BITS, NS, 2>(w, x, M, y, ydt, epi, st);
 }
 
 }  // namespace
 
 bool gemv1_serves(const WeightView& w, int xdt, int M, const Epilogue& epi)
 {
-    if (M != 1 || xdt != kF16 || epi.gamma) return false;
-    const int nsets = (w.KT + 3) / 4;
-    return (nsets + 15) / 16 <= max_sets_per_wave(w.bits, epi.kind == kEpiSwiglu ? 2 : 1);
+    if (M < 1 || M > 2 || xdt != kF16 || epi.gamma) return false;
+    const int mr = M;
+    const int ns = epi.kind == kEpiSwiglu ? 2 : 1;
+    const Shape1 sh = shape_of(w);
+    if (mr > 1 && ns == 2 && !sh.k8) return false;          // pairs with several rows: split workgroups only
+    return sh.per_wave <= max_sets_per_wave(w.bits, ns, mr);
 }
 
-hipError_t launch_gemv1(const WeightView& w, const void* x, void* y, int ydt, const Epilogue& epi, hipStream_t st)
+hipError_t launch_gemv1(const WeightView& w, const void* x, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st)
 {
     if (epi.kind == kEpiSwiglu) {
-        if (w.bits == 4) return launch1_s<4, 2>(w, x, y, ydt, epi, st);
-        return launch1_s<8, 2>(w, x, y, ydt, epi, st);
+        if (w.bits == 4) return launch1_m<4, 2>(w, x, M, y, ydt, epi, st);
+        return launch1_m<8, 2>(w, x, M, y, ydt, epi, st);
     }
-    if (w.bits == 4) return launch1_s<4, 1>(w, x, y, ydt, epi, st);
-    return launch1_s<8, 1>(w, x, y, ydt, epi, st);
+    if (w.bits == 4) return launch1_m<4, 1>(w, x, M, y, ydt, epi, st);
+    return launch1_m<8, 1>(w, x, M, y, ydt, epi, st);
 }
 
 }  // namespace cybq

@@ -276,17 +276,38 @@ def test_decode_batched_rows_equal_single_rows_bitwise(backend, oracle):
 @pytest.mark.parametrize("shape", [(64, 128), (48, 160), (100, 4096 + 96), (4096, 4096), (256, 14336), (64, 11008),
                                    (32, 16384), (16, 24576), (16, 32768)])
 def test_one_row_kernel_shapes(backend, oracle, bits, shape):
-    """One f16 row (subnormal weight operands, bias removed inside the accumulation): whole and
-    ragged sets of K tiles, one to three sets per wave, and K beyond what it serves."""
+    """One and two f16 rows (subnormal weight operands, bias removed inside the accumulation; the 16
+    rows of an activation operand are 1 / 2 batch rows x 16 / 8 scale groups): whole and ragged
+    sets of K tiles, one to three sets per wave, and K beyond what the kernel serves (3 and 4 rows
+    take the batched-rows kernel)."""
     N, K = shape
     q, s = _quant(oracle, bits, N, K)
     qw = backend.upload_quantized(q, s, bits, formats.BLOCK_AOS if N % 32 else formats.PLANAR)
-    x = _x(1, K, "f16", outliers=0.001)
-    y = _run(backend, qw, x)
-    assert oracle.rel_l2(y.cpu().numpy(), oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT
-    assert torch.equal(_run(backend, qw, x), y)                 # reproducible
-    for ydt in ("f16", "bf16"):
-        assert torch.equal(_run(backend, qw, x, ydt), y.to(TDT[ydt]))
+    x4 = _x(4, K, "f16", outliers=0.001)
+    ref = oracle.matmul_f64(q, s, x4.float().cpu().numpy())
+    for M in (1, 2, 3, 4):
+        x = x4[:M].contiguous()
+        y = _run(backend, qw, x)
+        assert oracle.rel_l2(y.cpu().numpy(), ref[:M]) < TIGHT, M
+        assert torch.equal(_run(backend, qw, x), y)                 # reproducible
+        for ydt in ("f16", "bf16"):
+            assert torch.equal(_run(backend, qw, x, ydt), y.to(TDT[ydt]))
+        # fused epilogues of the same kernel: residual add, and SwiGLU where the rows pair up
+        r = torch.from_numpy(synth.activations(36, M, N)).cuda()
+        y2 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        backend.matmul_ex(qw, x, y2, "add", r)
+        torch.cuda.synchronize()
+        assert torch.equal(y2, y + r), M
+    if N % 32 == 0 and N >= 64:
+        h = N // 2
+        pair = backend.fuse_pairs(backend.upload_quantized(q[:h], s[:h], bits), backend.upload_quantized(q[h:], s[h:], bits))
+        for M in (1, 2, 4):
+            y3 = torch.empty((M, h), dtype=torch.float32, device="cuda")
+            backend.matmul_ex(pair, x4[:M].contiguous(), y3, "swiglu")
+            torch.cuda.synchronize()
+            rd = torch.from_numpy(ref[:M]).cuda()
+            want = torch.nn.functional.silu(rd[:, :h]) * rd[:, h:]
+            assert ((y3.double() - want).norm() / want.norm()).item() < TIGHT, M
 
 
 @pytest.mark.parametrize("bits", [4, 8])
