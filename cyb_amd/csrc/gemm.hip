@@ -345,12 +345,12 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
         // barrier keeps the two waves of a SIMD in the same phase, so they do not cover for each
         // other.  (With one wave per SIMD, the 128-row shape, the same order measured slower.)
         if constexpr (WAVES == 8 && !EXACT) {
-            constexpr int PAIRS = 4 * NF * OPS * MF / 2;
+            constexpr int READS = 4 * NF * OPS;
             __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);          // LDS reads run two ahead of their MFMAs
 #pragma unroll
-            for (int i = 0; i < PAIRS; i++) {
+            for (int i = 0; i < READS; i++) {
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // one LDS read
-                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);      // two MFMAs
+                __builtin_amdgcn_sched_group_barrier(0x008, MF, 0);     // its MFMAs, one per row block
                 __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);      // two vector ALU instructions
             }
         }
@@ -526,6 +526,14 @@ hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt,
 {
     const int64_t tiles256 = (int64_t)((w.NT + NF - 1) / NF) * ((M + 255) / 256);
     const bool few_rows = M < 256 || (M == 256 && w.KT < 64);
+    // 512-row workgroups (four row blocks per wave: half the LDS operand reads per MFMA) once they
+    // fill the chip by themselves
+    if constexpr (!EXACT && NF == 7) {           // (eight column blocks x four row blocks spill)
+        const int64_t tiles512 = (int64_t)((w.NT + NF - 1) / NF) * ((M + 511) / 512);
+        const int rem = M % 512;                       // (a last tile at most half full: 256-row tiles waste less)
+        if (tiles512 >= num_cus && (rem == 0 || rem > 256))
+            return launch_m<BITS, XBF, NF, EXACT, 4, 8>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
+    }
     if (tiles256 < num_cus && few_rows) return launch_m<BITS, XBF, NF, EXACT, 2, 4>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
     return launch_m<BITS, XBF, NF, EXACT, 2, 8>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
 }

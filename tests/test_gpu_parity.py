@@ -596,6 +596,42 @@ def test_config4_full_size(backend, oracle, prefill_mode, M, shape):
         assert torch.equal(y2, y * 2)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("xdt", ["f16", "bf16"])
+def test_prefill_512_row_workgroups(backend, oracle, bits, xdt):
+    """FAST mode, N a multiple of 112 and enough rows for 512-row workgroups to fill the chip: a wave
+    multiplies four row blocks per weight operand.  Row counts that are whole tiles, leave a last
+    tile more than half full, or fall back to 256-row tiles; residual add and folded RMSNorm ride along."""
+    N, K = 14336, 384
+    q, s = _quant(oracle, bits, N, K, cfg=41)
+    qw = backend.upload_quantized(q, s, bits)
+    wd = torch.from_numpy(oracle.dequant(q, s)).cuda().double()
+    for M in (1024, 1300, 1100):
+        x = _x(M, K, xdt, cfg=42)
+        y = _run(backend, qw, x)
+        ref = x.double() @ wd.T
+        assert ((y.double() - ref).norm() / ref.norm()).item() < FAST, M
+        assert torch.equal(_run(backend, qw, x), y)                 # reproducible
+        # a row's bits depend neither on its place in a workgroup's tile nor on the tile shape
+        # (600 rows run as 256-row tiles)
+        assert torch.equal(_run(backend, qw, x[M - 600:].contiguous()), y[M - 600:]), M
+    M = 1024
+    x = _x(M, K, xdt, cfg=42)
+    r = torch.from_numpy(synth.activations(43, M, N)).cuda()
+    y2 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    backend.matmul_ex(qw, x, y2, "add", r)
+    torch.cuda.synchronize()
+    assert torch.equal(y2, _run(backend, qw, x) + r)
+    gamma = (1.0 + 0.1 * torch.from_numpy(synth.activations(44, 1, K))[0]).cuda()
+    y3 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    backend.matmul_norm(qw, x, gamma, 1e-5, y3)
+    torch.cuda.synchronize()
+    xd = x.double()
+    xn = xd * torch.rsqrt((xd * xd).mean(dim=1, keepdim=True) + 1e-5) * gamma.double()
+    ref = xn @ wd.T
+    assert ((y3.double() - ref).norm() / ref.norm()).item() < 2 * FAST
+
+
 # ------------------------------------------------------- fused epilogues
 # The reference's definitions of the ops around a linear are not in its tree (parity
 # unpinned); the checks below pin the library's stated formulas: y = r + x W^T, and
