@@ -408,6 +408,41 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
             }
         return;
     }
+    // fp32 output whose rows are 16-byte aligned: the accumulators (lane = column, four rows per
+    // lane) go through LDS - the operand buffers are free after the last K tile's barrier, a
+    // wave's share of them holds one of its row blocks - and leave as 128-bit stores, 64 lanes
+    // writing whole runs of a row instead of 64-byte pieces of four rows.
+    const bool rows_aligned = (w.N & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & 15u) == 0 &&
+                              (epi.kind != kEpiAdd || (reinterpret_cast<uintptr_t>(epi.residual) & 15u) == 0);
+    if (ydt == kF32 && rows_aligned) {
+        constexpr int ROWF = NF * 16;               // floats of a tile row
+        constexpr int V4 = ROWF / 4;                // 128-bit pieces of a tile row
+        float* stg = reinterpret_cast<float*>(smem) + wv * (16 * ROWF);
+        const float4_t* stg4 = reinterpret_cast<const float4_t*>(stg);
+#pragma unroll
+        for (int i = 0; i < MF; i++) {
+#pragma unroll
+            for (int f = 0; f < NF; f++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) stg[(oct * 4 + r) * ROWF + f * 16 + row16] = acc[i][f][r] * out_scale;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int p = lane; p < 16 * V4; p += 64) {
+                const int row = p / V4, c4 = p - row * V4;
+                const int m = m0 + i * 16 + row, n = nt0 * 16 + c4 * 4;
+                if (m < M && n < w.N) {
+                    float4_t v = stg4[p];
+                    const int64_t at = (int64_t)m * w.N + n;
+                    if (epi.kind == kEpiAdd) v += *reinterpret_cast<const float4_t*>(reinterpret_cast<const float*>(epi.residual) + at);
+                    *reinterpret_cast<float4_t*>(reinterpret_cast<float*>(y) + at) = v;
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < MF; i++)
 #pragma unroll
