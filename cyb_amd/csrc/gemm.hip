@@ -408,15 +408,16 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
             }
         return;
     }
-    // fp32 output whose rows are 16-byte aligned: the accumulators (lane = column, four rows per
-    // lane) go through LDS - the operand buffers are free after the last K tile's barrier, a
-    // wave's share of them holds one of its row blocks - and leave as 128-bit stores, 64 lanes
-    // writing whole runs of a row instead of 64-byte pieces of four rows.
-    const bool rows_aligned = (w.N & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & 15u) == 0 &&
-                              (epi.kind != kEpiAdd || (reinterpret_cast<uintptr_t>(epi.residual) & 15u) == 0);
-    if (ydt == kF32 && rows_aligned) {
+    // Output rows that start on a 16-byte boundary (8 for 16-bit outputs): the accumulators (lane =
+    // column, four rows per lane) go through LDS - the operand buffers are free after the last K
+    // tile's barrier, a wave's share of them holds one of its row blocks - and leave four
+    // elements per lane, 64 lanes writing whole runs of a row instead of 64-byte pieces of four rows.
+    const uintptr_t amask = ydt == kF32 ? 15u : 7u;
+    const bool rows_aligned = (w.N & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & amask) == 0 &&
+                              (epi.kind != kEpiAdd || (reinterpret_cast<uintptr_t>(epi.residual) & amask) == 0);
+    if (rows_aligned) {
         constexpr int ROWF = NF * 16;               // floats of a tile row
-        constexpr int V4 = ROWF / 4;                // 128-bit pieces of a tile row
+        constexpr int V4 = ROWF / 4;                // four-element pieces of a tile row
         float* stg = reinterpret_cast<float*>(smem) + wv * (16 * ROWF);
         const float4_t* stg4 = reinterpret_cast<const float4_t*>(stg);
 #pragma unroll
@@ -434,8 +435,28 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
                 if (m < M && n < w.N) {
                     float4_t v = stg4[p];
                     const int64_t at = (int64_t)m * w.N + n;
-                    if (epi.kind == kEpiAdd) v += *reinterpret_cast<const float4_t*>(reinterpret_cast<const float*>(epi.residual) + at);
-                    *reinterpret_cast<float4_t*>(reinterpret_cast<float*>(y) + at) = v;
+                    if (ydt == kF32) {
+                        if (epi.kind == kEpiAdd) v += *reinterpret_cast<const float4_t*>(reinterpret_cast<const float*>(epi.residual) + at);
+                        *reinterpret_cast<float4_t*>(reinterpret_cast<float*>(y) + at) = v;
+                    } else {
+                        if (epi.kind == kEpiAdd) {
+                            const u32x2_t rr = *reinterpret_cast<const u32x2_t*>(reinterpret_cast<const uint16_t*>(epi.residual) + at);
+#pragma unroll
+                            for (int e = 0; e < 4; e++) {
+                                const uint32_t h = (e & 1) ? rr[e >> 1] >> 16 : rr[e >> 1] & 0xffffu;
+                                v[e] += ydt == kF16 ? f16_bits_to_f32(h) : __builtin_bit_cast(float, h << 16);
+                            }
+                        }
+                        u32x2_t o;
+                        if (ydt == kF16) {
+                            const half2_t a = {(_Float16)v[0], (_Float16)v[1]}, b = {(_Float16)v[2], (_Float16)v[3]};
+                            o = (u32x2_t){as_u32(a), as_u32(b)};
+                        } else {
+                            o = (u32x2_t){(uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16),
+                                          (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16)};
+                        }
+                        *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(y) + at) = o;
+                    }
                 }
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
