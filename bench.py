@@ -35,8 +35,8 @@ MIN_TIMED_S = 0.050
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the
 # same counter reads for a plain 256 MiB copy; profiles/decode_gemv_q4_4096x14336_m1.md and
 # profiles/prefill_gemm_q4_4096x14336_m512.md
-TRAFFIC_DECODE_BYTES = 33_194_100
-TRAFFIC_PREFILL_M512_BYTES = 121_870_000      # multiply 113.4 MB + activation staging pass 8.5 MB
+TRAFFIC_DECODE_BYTES = 33_191_700
+TRAFFIC_PREFILL_M512_BYTES = 121_100_000      # multiply 113.4 MB + activation staging pass 8.5 MB
 
 
 def log(*a):
@@ -119,7 +119,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=2000)      # (about 14 ms: the clocks settle within the first 10 ms of load)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the prefill / sweep / stack extras")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -255,6 +255,7 @@ def main():
     lat = sorted(timer.once(lambda: walk(1, lambda p: be.matmul_many(p, M, stream))) * 1e6 for _ in range(20))
     per = sorted(t / args.steps * 1e6 for t in passes)
     spread = {"min": round(per[0], 3), "median": round(per[len(per) // 2], 3), "max": round(per[-1], 3),
+              "in_order": [round(t / args.steps * 1e6, 3) for t in passes],
               "of": f"{len(per)} timed passes of {args.steps} back-to-back launches, us per launch"}
 
     result = {
