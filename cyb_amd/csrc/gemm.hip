@@ -190,6 +190,86 @@ __device__ __forceinline__ float4_t mma(const Frag16& a, const Frag16& b, float4
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, c, 0, 0, 0);
 }
 
+// The finished sums of one wave (MF row blocks x NF column blocks, lane = column, four rows per lane;
+// first row m0, first column block nt0) -> y, with the residual-add epilogue.  `stg`: 16 x NF*16
+// floats of LDS that belong to this wave.
+template <int MF, int NF>
+__device__ __forceinline__ void write_rows(const float4_t (&acc)[MF][NF], float* stg, int m0, int nt0, int M, int N, void* y, int ydt,
+                                           float out_scale, const Epilogue& epi, int lane)
+{
+    const int row16 = lane & 15, oct = lane >> 4;
+    // Output rows that start on a 16-byte boundary (8 for 16-bit outputs): the accumulators (lane =
+    // column, four rows per lane) go through LDS - the operand buffers are free after the last K
+    // tile's barrier, a wave's share of them holds one of its row blocks - and leave four
+    // elements per lane, 64 lanes writing whole runs of a row instead of 64-byte pieces of four rows.
+    const uintptr_t amask = ydt == kF32 ? 15u : 7u;
+    const bool rows_aligned = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & amask) == 0 &&
+                              (epi.kind != kEpiAdd || (reinterpret_cast<uintptr_t>(epi.residual) & amask) == 0);
+    if (rows_aligned) {
+        constexpr int ROWF = NF * 16;               // floats of a tile row
+        constexpr int V4 = ROWF / 4;                // four-element pieces of a tile row
+        const float4_t* stg4 = reinterpret_cast<const float4_t*>(stg);
+#pragma unroll
+        for (int i = 0; i < MF; i++) {
+#pragma unroll
+            for (int f = 0; f < NF; f++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) stg[(oct * 4 + r) * ROWF + f * 16 + row16] = acc[i][f][r] * out_scale;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int p = lane; p < 16 * V4; p += 64) {
+                const int row = p / V4, c4 = p - row * V4;
+                const int m = m0 + i * 16 + row, n = nt0 * 16 + c4 * 4;
+                if (m < M && n < N) {
+                    float4_t v = stg4[p];
+                    const int64_t at = (int64_t)m * N + n;
+                    if (ydt == kF32) {
+                        if (epi.kind == kEpiAdd) v += *reinterpret_cast<const float4_t*>(reinterpret_cast<const float*>(epi.residual) + at);
+                        *reinterpret_cast<float4_t*>(reinterpret_cast<float*>(y) + at) = v;
+                    } else {
+                        if (epi.kind == kEpiAdd) {
+                            const u32x2_t rr = *reinterpret_cast<const u32x2_t*>(reinterpret_cast<const uint16_t*>(epi.residual) + at);
+#pragma unroll
+                            for (int e = 0; e < 4; e++) {
+                                const uint32_t h = (e & 1) ? rr[e >> 1] >> 16 : rr[e >> 1] & 0xffffu;
+                                v[e] += ydt == kF16 ? f16_bits_to_f32(h) : __builtin_bit_cast(float, h << 16);
+                            }
+                        }
+                        u32x2_t o;
+                        if (ydt == kF16) {
+                            const half2_t a = {(_Float16)v[0], (_Float16)v[1]}, b = {(_Float16)v[2], (_Float16)v[3]};
+                            o = (u32x2_t){as_u32(a), as_u32(b)};
+                        } else {
+                            o = (u32x2_t){(uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16),
+                                          (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16)};
+                        }
+                        *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(y) + at) = o;
+                    }
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < MF; i++)
+#pragma unroll
+        for (int f = 0; f < NF; f++) {
+            const int n = (nt0 + f) * 16 + row16;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int m = m0 + i * 16 + oct * 4 + r;
+                if (m < M && n < N) {
+                    float v = acc[i][f][r] * out_scale;
+                    if (epi.kind == kEpiAdd) v += load_out_g(epi.residual, ydt, (int64_t)m * N + n);
+                    store_out_g(y, ydt, (int64_t)m * N + n, v);
+                }
+            }
+        }
+}
+
 // XBF = 1: X is bf16, 0: X is f16.  EXACT: see the header comment.
 // Wave wv of WAVES owns MF row blocks of 16 against all NF column blocks.
 template <int BITS, int XBF, int NF, bool EXACT, int MF, int WAVES>
@@ -408,77 +488,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
             }
         return;
     }
-    // Output rows that start on a 16-byte boundary (8 for 16-bit outputs): the accumulators (lane =
-    // column, four rows per lane) go through LDS - the operand buffers are free after the last K
-    // tile's barrier, a wave's share of them holds one of its row blocks - and leave four
-    // elements per lane, 64 lanes writing whole runs of a row instead of 64-byte pieces of four rows.
-    const uintptr_t amask = ydt == kF32 ? 15u : 7u;
-    const bool rows_aligned = (w.N & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & amask) == 0 &&
-                              (epi.kind != kEpiAdd || (reinterpret_cast<uintptr_t>(epi.residual) & amask) == 0);
-    if (rows_aligned) {
-        constexpr int ROWF = NF * 16;               // floats of a tile row
-        constexpr int V4 = ROWF / 4;                // four-element pieces of a tile row
-        float* stg = reinterpret_cast<float*>(smem) + wv * (16 * ROWF);
-        const float4_t* stg4 = reinterpret_cast<const float4_t*>(stg);
-#pragma unroll
-        for (int i = 0; i < MF; i++) {
-#pragma unroll
-            for (int f = 0; f < NF; f++)
-#pragma unroll
-                for (int r = 0; r < 4; r++) stg[(oct * 4 + r) * ROWF + f * 16 + row16] = acc[i][f][r] * out_scale;
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-#pragma unroll
-            for (int p = lane; p < 16 * V4; p += 64) {
-                const int row = p / V4, c4 = p - row * V4;
-                const int m = m0 + i * 16 + row, n = nt0 * 16 + c4 * 4;
-                if (m < M && n < w.N) {
-                    float4_t v = stg4[p];
-                    const int64_t at = (int64_t)m * w.N + n;
-                    if (ydt == kF32) {
-                        if (epi.kind == kEpiAdd) v += *reinterpret_cast<const float4_t*>(reinterpret_cast<const float*>(epi.residual) + at);
-                        *reinterpret_cast<float4_t*>(reinterpret_cast<float*>(y) + at) = v;
-                    } else {
-                        if (epi.kind == kEpiAdd) {
-                            const u32x2_t rr = *reinterpret_cast<const u32x2_t*>(reinterpret_cast<const uint16_t*>(epi.residual) + at);
-#pragma unroll
-                            for (int e = 0; e < 4; e++) {
-                                const uint32_t h = (e & 1) ? rr[e >> 1] >> 16 : rr[e >> 1] & 0xffffu;
-                                v[e] += ydt == kF16 ? f16_bits_to_f32(h) : __builtin_bit_cast(float, h << 16);
-                            }
-                        }
-                        u32x2_t o;
-                        if (ydt == kF16) {
-                            const half2_t a = {(_Float16)v[0], (_Float16)v[1]}, b = {(_Float16)v[2], (_Float16)v[3]};
-                            o = (u32x2_t){as_u32(a), as_u32(b)};
-                        } else {
-                            o = (u32x2_t){(uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16),
-                                          (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16)};
-                        }
-                        *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(y) + at) = o;
-                    }
-                }
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-        }
-        return;
-    }
-#pragma unroll
-    for (int i = 0; i < MF; i++)
-#pragma unroll
-        for (int f = 0; f < NF; f++) {
-            const int n = (nt0 + f) * 16 + row16;
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int m = m0 + i * 16 + oct * 4 + r;
-                if (m < M && n < w.N) {
-                    float v = acc[i][f][r] * out_scale;
-                    if (epi.kind == kEpiAdd) v += load_out_g(epi.residual, ydt, (int64_t)m * w.N + n);
-                    store_out_g(y, ydt, (int64_t)m * w.N + n, v);
-                }
-            }
-        }
+    write_rows<MF, NF>(acc, reinterpret_cast<float*>(smem) + wv * (16 * NF * 16), m0, nt0, M, w.N, y, ydt, out_scale, epi, lane);
 }
 
 // y = epilogue(out_scale * (part[0] + part[1] + ... + part[splits-1])), slabs added in that order.
