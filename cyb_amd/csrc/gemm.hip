@@ -491,6 +491,167 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
     write_rows<MF, NF>(acc, reinterpret_cast<float*>(smem) + wv * (16 * NF * 16), m0, nt0, M, w.N, y, ydt, out_scale, epi, lane);
 }
 
+// The same multiply (FAST mode, f16 operands) with the work of a workgroup split by role:
+// MW waves only multiply - each owns MF row blocks against all NF column blocks, streams its X
+// from global memory XD K tiles ahead and reads the weight operands from LDS - and four waves
+// only fetch packed weight tiles and dequantise them into LDS, several K tiles ahead.  Loads
+// retire in order within a wave: in gemm_kernel the wait for the next rows of X is also a wait
+// for every weight tile requested before them, and a first touch in HBM holds the matrix pipe
+// up; here the multiplying waves never wait for HBM.  Waves are dealt to the four SIMDs in turn,
+// so every SIMD carries one staging wave: the dequantisation runs in the issue slots the MFMAs
+// leave free.  MW*MF*16 x NF*16 outputs per workgroup, one barrier per K tile, no K split.
+template <int BITS, int NF, int MF, int MW, int XD>
+__global__ __launch_bounds__((MW + 4) * 64) __attribute__((amdgpu_waves_per_eu((MW + 4) / 4, (MW + 4) / 4))) void gemm_roles_kernel(
+    const uint8_t* __restrict__ wbase, const u32x4_t* __restrict__ x, int KT_, int NT_, int x_row_blocks, int M, int n_tiles,
+    int m_tiles, int groups, int N_, void* __restrict__ y, int ydt, int K_, float out_scale, Epilogue epi, NormStats ns)
+{
+    const WeightView w = {wbase, N_, K_, NT_, KT_, BITS};
+    constexpr int SW = 4;                             // staging waves
+    constexpr int WT = (NF + SW - 1) / SW;            // weight tiles a staging wave handles per K tile
+    constexpr int TILE16 = 4 * 64;                    // u32x4 per column block per K tile
+    constexpr int BUF16 = NF * TILE16;
+    constexpr int DEPTH = 4;                          // K tiles of packed weights in flight per staging wave
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    u32x4_t* ws = reinterpret_cast<u32x4_t*>(smem);   // [2][NF][4][64]
+
+    const int per_xcd = groups >> 3;                  // (same tile order as gemm_kernel)
+    const int item = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+    if (item >= n_tiles * m_tiles) return;
+    const int tile_m = item / n_tiles, tile_n = item - tile_m * n_tiles;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nt0 = tile_n * NF;
+    const int KT = w.KT, K = w.K;
+    const int kt0 = tile_n % KT;
+    auto rot = [&](int kt) {
+        const int r = min(kt, KT - 1) + kt0;
+        return r >= KT ? r - KT : r;
+    };
+
+    if (wave >= MW) {
+        // ---- staging waves ----------------------------------------------------------------
+        const int pw = wave - MW;
+        const uint32_t magic = q4_magic_vgpr();
+        int64_t wtile[WT];
+        int wdst[WT];
+#pragma unroll
+        for (int t = 0; t < WT; t++) {
+            const int f = min(pw + SW * t, NF - 1);     // (past the end: a neighbour's block again, same values)
+            wdst[t] = f * TILE16;
+            wtile[t] = (int64_t)min(nt0 + f, w.NT - 1) * w.KT;
+        }
+        WRegs<BITS> wreg[DEPTH][WT];
+        auto fetch = [&](WRegs<BITS> (&dst)[WT], int kt) {
+#pragma unroll
+            for (int t = 0; t < WT; t++) load_wtile<BITS>(dst[t], w, wtile[t] + rot(kt), lane);
+        };
+        auto stage = [&](WRegs<BITS> (&src)[WT], u32x4_t* buf) {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int t = 0; t < WT; t++) dequant_group_to_lds<BITS, 0, false>(src[t], j, magic, buf + wdst[t], lane);
+        };
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) fetch(wreg[d], d);
+        stage(wreg[0], ws);
+        fetch(wreg[0], DEPTH);
+        __syncthreads();
+        // during K tile kt: tile kt + 1 (register set (kt + 1) % DEPTH) -> the other LDS buffer, then that
+        // set is refilled with tile kt + 1 + DEPTH
+        auto k_tile = [&](int kt, auto residue) {
+            constexpr int R = decltype(residue)::value;            // = (kt + 1) % DEPTH
+            stage(wreg[R], ws + ((R & 1) ? BUF16 : 0));
+            fetch(wreg[R], kt + 1 + DEPTH);
+            __syncthreads();
+        };
+        for (int kt = 0; kt < KT; kt += DEPTH) {
+            k_tile(kt, std::integral_constant<int, 1>{});
+            if (kt + 1 < KT) k_tile(kt + 1, std::integral_constant<int, 2>{});
+            if (kt + 2 < KT) k_tile(kt + 2, std::integral_constant<int, 3>{});
+            if (kt + 3 < KT) k_tile(kt + 3, std::integral_constant<int, 0>{});
+        }
+        return;
+    }
+
+    // ---- multiplying waves --------------------------------------------------------------------
+    const int m0 = tile_m * (MW * MF * 16) + wave * (MF * 16);
+    const int G = K / kGroup;
+    const u32x4_t* xb[MF];
+#pragma unroll
+    for (int i = 0; i < MF; i++) xb[i] = x + ((int64_t)min(m0 / 16 + i, x_row_blocks - 1) * G) * 64 + lane;
+    auto load_x = [&](Frag16 (&dst)[MF], int kt, int j) {
+        const int g = min(rot(kt) * 4 + j, G - 1);
+#pragma unroll
+        for (int i = 0; i < MF; i++) dst[i].u = xb[i][g * 64];
+    };
+    float4_t acc[MF][NF];
+#pragma unroll
+    for (int i = 0; i < MF; i++)
+#pragma unroll
+        for (int f = 0; f < NF; f++) acc[i][f] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    Frag16 xa[XD][4][MF];          // XD K tiles of X in flight
+#pragma unroll
+    for (int d = 0; d < XD; d++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) load_x(xa[d][j], d, j);
+    __syncthreads();
+    auto k_tile = [&](int kt, auto residue) {
+        constexpr int D = decltype(residue)::value;                 // = kt % XD
+        const u32x4_t* wcur = ws + ((kt & 1) ? BUF16 : 0);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+#pragma unroll
+            for (int f = 0; f < NF; f++) {
+                Frag16 b;
+                b.u = wcur[f * TILE16 + j * 64 + lane];
+#pragma unroll
+                for (int i = 0; i < MF; i++) acc[i][f] = mma<0>(xa[D][j][i], b, acc[i][f]);
+            }
+            load_x(xa[D][j], kt + XD, j);      // this group's operands are free: those of K tile kt + XD take their place
+        }
+        constexpr int READS = 4 * NF;
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);          // LDS reads run two ahead of their MFMAs
+#pragma unroll
+        for (int i = 0; i < READS; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, MF, 0);
+        }
+        __syncthreads();
+    };
+    for (int kt = 0; kt < KT; kt += XD) {
+        k_tile(kt, std::integral_constant<int, 0>{});
+        if constexpr (XD > 1) {
+            if (kt + 1 < KT) k_tile(kt + 1, std::integral_constant<int, 1>{});
+        }
+    }
+    if (epi.gamma || ns.unscale) {
+#pragma unroll
+        for (int i = 0; i < MF; i++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float rs = row_factor(ns, epi.gamma != nullptr, min(m0 + i * 16 + (lane >> 4) * 4 + r, M - 1), K, epi.eps);
+#pragma unroll
+                for (int f = 0; f < NF; f++) acc[i][f][r] *= rs;
+            }
+    }
+    write_rows<MF, NF>(acc, reinterpret_cast<float*>(smem) + wave * (16 * NF * 16), m0, nt0, M, w.N, y, ydt, out_scale, epi, lane);
+}
+
+template <int BITS, int NF, int MF, int MW, int XD>
+hipError_t launch_roles(const WeightView& w, const void* x, int M, void* y, int ydt, float out_scale, const Epilogue& epi,
+                        const NormStats& ns, hipStream_t st)
+{
+    constexpr int lds = 2 * NF * (4 * 64) * 16;
+    constexpr int BM = MW * MF * 16;
+    (void)LdsRequest<&gemm_roles_kernel<BITS, NF, MF, MW, XD>, lds>::registered;
+    const int n_tiles = (w.NT + NF - 1) / NF, m_tiles = (M + BM - 1) / BM;
+    const unsigned groups = (unsigned)(((int64_t)n_tiles * m_tiles + 7) / 8 * 8);
+    hipLaunchKernelGGL((gemm_roles_kernel<BITS, NF, MF, MW, XD>), dim3(groups), dim3((MW + 4) * 64), lds, st, w.base,
+                       reinterpret_cast<const u32x4_t*>(x), w.KT, w.NT, (M + 15) / 16, M, n_tiles, m_tiles, (int)groups, w.N, y, ydt, w.K,
+                       out_scale, epi, ns);
+    return hipGetLastError();
+}
+
 // y = epilogue(out_scale * (part[0] + part[1] + ... + part[splits-1])), slabs added in that order.
 // One thread per output element; N = columns of a slab (for SwiGLU y has N / 2).
 __global__ void splitk_reduce_kernel(const float* __restrict__ part, int splits, int M, int N, void* __restrict__ y, int ydt,
@@ -599,6 +760,14 @@ hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt,
         const int rem = M % 512;                       // (a last tile at most half full: 256-row tiles waste less)
         if (tiles512 >= num_cus && (rem == 0 || rem > 256))
             return launch_m<BITS, XBF, NF, EXACT, 4, 8>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
+    }
+    if constexpr (!EXACT && NF == 7 && BITS == 4) {
+        static const int roles = getenv("CYBQ_ROLES") ? atoi(getenv("CYBQ_ROLES")) : 0;      // EXPERIMENT
+        if (roles && tiles256 >= num_cus && epi.kind != kEpiSwiglu) {
+            if (roles == 1) return launch_roles<BITS, NF, 4, 4, 1>(w, x, M, y, ydt, out_scale, epi, ns, st);
+            if (roles == 2) return launch_roles<BITS, NF, 2, 8, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
+            if (roles == 3) return launch_roles<BITS, NF, 2, 8, 1>(w, x, M, y, ydt, out_scale, epi, ns, st);
+        }
     }
     if (tiles256 < num_cus && few_rows) return launch_m<BITS, XBF, NF, EXACT, 2, 4>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
     return launch_m<BITS, XBF, NF, EXACT, 2, 8>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
