@@ -761,13 +761,10 @@ hipError_t launch_t(const WeightView& w, const void* x, int M, void* y, int ydt,
         if (tiles512 >= num_cus && (rem == 0 || rem > 256))
             return launch_m<BITS, XBF, NF, EXACT, 4, 8>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
     }
-    if constexpr (!EXACT && NF == 7 && BITS == 4) {
-        static const int roles = getenv("CYBQ_ROLES") ? atoi(getenv("CYBQ_ROLES")) : 0;      // EXPERIMENT
-        if (roles && tiles256 >= num_cus && epi.kind != kEpiSwiglu) {
-            if (roles == 1) return launch_roles<BITS, NF, 4, 4, 1>(w, x, M, y, ydt, out_scale, epi, ns, st);
-            if (roles == 2) return launch_roles<BITS, NF, 2, 8, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
-            if (roles == 3) return launch_roles<BITS, NF, 2, 8, 1>(w, x, M, y, ydt, out_scale, epi, ns, st);
-        }
+    // enough 256-row tiles to fill the chip without a K split: the role-split kernel (the SwiGLU
+    // epilogue is not among what it writes)
+    if constexpr (!EXACT) {
+        if (tiles256 >= num_cus && epi.kind != kEpiSwiglu) return launch_roles<BITS, NF, 2, 8, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
     }
     if (tiles256 < num_cus && few_rows) return launch_m<BITS, XBF, NF, EXACT, 2, 4>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
     return launch_m<BITS, XBF, NF, EXACT, 2, 8>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);

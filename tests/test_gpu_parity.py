@@ -632,6 +632,39 @@ def test_prefill_512_row_workgroups(backend, oracle, bits, xdt):
     assert ((y3.double() - ref).norm() / ref.norm()).item() < 2 * FAST
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("shape", [(14336, 384, 512), (4096, 384, 2048), (6144, 160, 1100)])
+def test_prefill_role_split_kernel(backend, oracle, bits, shape):
+    """FAST mode with enough 256-row tiles to fill the chip: some waves of a workgroup only multiply,
+    the others only fetch and dequantise weights.  Seven and eight column blocks per tile, a ragged
+    last row tile, every activation and output type, residual add and folded RMSNorm."""
+    N, K, M = shape
+    q, s = _quant(oracle, bits, N, K, cfg=45)
+    qw = backend.upload_quantized(q, s, bits)
+    wd = torch.from_numpy(oracle.dequant(q, s)).cuda().double()
+    r = torch.from_numpy(synth.activations(47, M, N)).cuda()
+    for xdt, ydt in (("bf16", "f32"), ("f16", "bf16"), ("f32", "f16")):
+        x = _x(M, K, xdt, cfg=46)
+        ref = x.double() @ wd.T
+        y = _run(backend, qw, x, ydt)
+        bar = FAST if ydt == "f32" else 4e-3            # (a 16-bit output rounds every element once more)
+        assert ((y.double() - ref).norm() / ref.norm()).item() < bar, (xdt, ydt)
+        assert torch.equal(_run(backend, qw, x, ydt), y)             # reproducible
+        y2 = torch.empty((M, N), dtype=TDT[ydt], device="cuda")
+        backend.matmul_ex(qw, x, y2, "add", r.to(TDT[ydt]))
+        torch.cuda.synchronize()
+        want = ref + r.to(TDT[ydt]).double()
+        assert ((y2.double() - want).norm() / want.norm()).item() < bar, (xdt, ydt)
+    x = _x(M, K, "bf16", cfg=46)
+    gamma = (1.0 + 0.1 * torch.from_numpy(synth.activations(48, 1, K))[0]).cuda()
+    y3 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    backend.matmul_norm(qw, x, gamma, 1e-5, y3)
+    torch.cuda.synchronize()
+    xd = x.double()
+    ref = (xd * torch.rsqrt((xd * xd).mean(dim=1, keepdim=True) + 1e-5) * gamma.double()) @ wd.T
+    assert ((y3.double() - ref).norm() / ref.norm()).item() < 2 * FAST
+
+
 # ------------------------------------------------------- fused epilogues
 # The reference's definitions of the ops around a linear are not in its tree (parity
 # unpinned); the checks below pin the library's stated formulas: y = r + x W^T, and
