@@ -36,7 +36,7 @@ MIN_TIMED_S = 0.050
 # same counter reads for a plain 256 MiB copy; profiles/decode_gemv_q4_4096x14336_m1.md and
 # profiles/prefill_gemm_q4_4096x14336_m512.md
 TRAFFIC_DECODE_BYTES = 33_191_700
-TRAFFIC_PREFILL_M512_BYTES = 121_100_000      # multiply 112.6 MB + activation staging pass 8.5 MB
+TRAFFIC_PREFILL_M512_BYTES = 121_400_000      # multiply 112.9 MB + activation staging pass 8.5 MB
 
 
 def log(*a):
