@@ -623,6 +623,12 @@ __global__ __launch_bounds__((MW + 4) * 64) __attribute__((amdgpu_waves_per_eu((
         if constexpr (XD > 1) {
             if (kt + 1 < KT) k_tile(kt + 1, std::integral_constant<int, 1>{});
         }
+        if constexpr (XD > 2) {
+            if (kt + 2 < KT) k_tile(kt + 2, std::integral_constant<int, 2>{});
+        }
+        if constexpr (XD > 3) {
+            if (kt + 3 < KT) k_tile(kt + 3, std::integral_constant<int, 3>{});
+        }
     }
     if (epi.gamma || ns.unscale) {
 #pragma unroll
@@ -782,6 +788,15 @@ hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt
         return launch_t<BITS, XBF, 8, true>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
     }
     if constexpr (XBF == 0) {       // FAST multiplies in f16: bf16 activations were widened by the staging pass
+        // up to 128 rows on a wide output: 128 x 64 tiles fill most of the chip without a K split and
+        // its second pass over the partial sums
+        if (M <= 128 && epi.kind != kEpiSwiglu) {
+            const int64_t tiles64 = (w.NT + 3) / 4;                  // 64-column tiles
+            if (tiles64 * 2 >= 3 * num_cus)          // more than one round of them: the plain kernel (48 against 58 us at N = 28672)
+                return launch_m<BITS, 0, 4, false, 2, 4>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
+            if (tiles64 * 4 >= 3 * num_cus)          // one round: the role-split kernel (30 against 34.5 us at N = 14336)
+                return launch_roles<BITS, 4, 2, 4, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
+        }
         if (nf7) return launch_t<BITS, 0, 7, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
         return launch_t<BITS, 0, 8, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
     }
