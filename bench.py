@@ -124,7 +124,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the prefill / sweep / stack extras")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="no timing: a plain 256 MiB device copy (calibration), then the decode and prefill "
-                         "kernels, for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
+                         "kernels and the 16-row decode kernel on both sweep shapes, for rocprofv3 --pmc runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the op would shard by rows of W "
@@ -185,6 +185,17 @@ def main():
         yp = torch.empty((512, N), dtype=torch.float32, device=dev)
         for i in range(10):
             be.matmul(ws[i % copies], xp, yp, stream=stream)
+        torch.cuda.synchronize()
+        # the batched-rows decode kernel at 16 rows on both sweep shapes (the down projection is the
+        # kernel furthest below its roofline: counters say what it waits for)
+        qd, sd = formats.quantize(synth.weights(6, K, N), bits)
+        wd = [be.upload_quantized(qd, sd, bits)]
+        wd += [wd[0].clone() for _ in range(copies - 1)]
+        for (wl, Kx, Nx) in ((ws, K, N), (wd, N, K)):
+            xb = torch.from_numpy(synth.activations(3, 16, Kx)).to(dev).to(torch.float16)
+            yb = torch.empty((16, Nx), dtype=torch.float32, device=dev)
+            for i in range(50):
+                be.matmul(wl[i % copies], xb, yb, stream=stream)
         torch.cuda.synchronize()
         log("traffic probe done")
         return
