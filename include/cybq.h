@@ -139,8 +139,9 @@ int cybq_weight_info(const cybq_weight* w, int* quant, int64_t* N, int64_t* K,
  * with fp32 accumulation.
  *   x  [M,K] row-major, xdt in {F16,BF16,F32}, 16-byte aligned
  *   y  [M,N] row-major, ydt in {F32,F16,BF16} (fp32 accumulator rounded once)
- *   M >= 1.  M <= 16 runs the HBM-streaming decode kernels (17..32 rows: two
- *   passes of them), larger M the LDS-tiled MFMA prefill kernel (fp32
+ *   M >= 1.  M <= 32 runs the HBM-streaming decode kernels (17..32 rows of 16-bit
+ *   activations: one pass with two row blocks; with a folded norm two passes of 16
+ *   rows), larger M the LDS-tiled MFMA prefill kernel (fp32
  *   activations in CYBQ_PREFILL_EXACT mode: the decode kernel, 16 rows at a
  *   time; in FAST mode they are rounded once to f16 on the way in and take
  *   the prefill kernel from 17 rows on); there is no other path. */
