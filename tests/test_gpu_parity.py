@@ -669,6 +669,40 @@ def test_prefill_role_split_kernel(backend, oracle, bits, shape):
     assert ((y3.double() - ref).norm() / ref.norm()).item() < 2 * FAST
 
 
+def test_lm_head_shape(backend, oracle):
+    """The LM head of a Llama-3-sized vocabulary (decide/pipeline.md:51): 128256 rows, K = 4096, Q4 -
+    8016 strips, several rounds of workgroups per CU.  Weights are made and quantised on the device;
+    every output is checked against a float64 product over the exactly dequantised tensor (chunks of
+    rows), a sample of rows against the oracle from the packed bytes."""
+    N, K, bits = 128256, 4096, 4
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1234)
+    w = torch.empty((N, K), dtype=torch.float32, device="cuda").normal_(0.0, 0.02, generator=gen)
+    qd = torch.empty(N * K // 2, dtype=torch.uint8, device="cuda")
+    sd = torch.empty(N * (K // 32), dtype=torch.int16, device="cuda")
+    backend.quantize(bits, w, N, K, qd, sd)
+    qw = backend.weight_from_device(bits, N, K, qd, sd)
+    torch.cuda.synchronize()
+    backend.dequant(qw, w)                       # w now holds scale * q, bit-exact (tested elsewhere)
+    torch.cuda.synchronize()
+    rows = torch.arange(0, N, 997, device="cuda")
+    qrows = formats.unpack_planar(qd.view(N, K // 2)[rows].cpu().numpy().reshape(-1), bits, len(rows), K)
+    srows = sd.view(N, K // 32)[rows].cpu().numpy().view(np.uint16)
+    assert np.array_equal(oracle.dequant(qrows, srows), w[rows].cpu().numpy())
+    for M, xdt in ((1, "f16"), (2, "f16"), (8, "f16"), (8, "bf16"), (20, "f16")):
+        x = _x(M, K, xdt, cfg=51)
+        y = _run(backend, qw, x)
+        xd = x.double()
+        num = den = 0.0
+        for r0 in range(0, N, 16032):
+            ref = xd @ w[r0:r0 + 16032].double().T
+            num += ((y[:, r0:r0 + 16032].double() - ref) ** 2).sum().item()
+            den += (ref ** 2).sum().item()
+        assert (num / den) ** 0.5 < TIGHT, (M, xdt)
+        ref = oracle.matmul_f64(qrows, srows, x.float().cpu().numpy())
+        assert oracle.rel_l2(y[:, rows].cpu().numpy(), ref) < TIGHT, (M, xdt)
+
+
 # ------------------------------------------------------- fused epilogues
 # The reference's definitions of the ops around a linear are not in its tree (parity
 # unpinned); the checks below pin the library's stated formulas: y = r + x W^T, and
