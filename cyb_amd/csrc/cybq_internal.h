@@ -25,10 +25,11 @@ bool gemv_serves_32(int xdt, int M, const Epilogue& epi);
 // kernel) instead of the subnormal-operand kernel of gemv1.hip
 hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
                        int num_cus, bool exact_operands, const Epilogue& epi, hipStream_t st);
-// decode kernel for one and two rows (f16 activations, no folded norm): weight operands are f16 subnormals,
+// decode kernel for one and two rows (f16 / bf16 activations, no folded norm): weight operands are f16 subnormals
+// (bf16: 128 + u),
 // the +8 / +128 bias comes off inside the MFMA accumulation (gemv1.hip)
 bool gemv1_serves(const WeightView& w, int xdt, int M, const Epilogue& epi);
-hipError_t launch_gemv1(const WeightView& w, const void* x, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st);
+hipError_t launch_gemv1(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st);
 // prefill path (api.hip sends 16-bit activations with M > 32 here)
 // exact: two MFMAs per group with losslessly split weights; otherwise one f16 MFMA
 // per group with weights rounded once to f16

@@ -1018,7 +1018,7 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
     // one or two f16 rows: the kernel of gemv1.hip (unless the caller asked for exact integer weight
     // operands, or a test forces one of the kernels below)
     if (!exact_operands && g_tune_waves == 0 && g_tune_rows == 0 && g_tune_unroll == 0 && gemv1_serves(w, xdt, M, epi))
-        return launch_gemv1(w, x, M, y, ydt, epi, st);
+        return launch_gemv1(w, x, xdt, M, y, ydt, epi, st);
     int nwaves = g_tune_waves;
     if (nwaves <= 0) {
         nwaves = 2;

@@ -47,11 +47,18 @@ __device__ __forceinline__ float load_out1(const void* p, int dt, int64_t idx)
 }
 
 // B operand of scale group r of one tile as loaded by a lane
-template <int BITS>
-__device__ __forceinline__ Frag16 sub_operand(const u32x4_t (&q)[BITS == 4 ? 1 : 2], int r)
+// (XBF: bf16 activations - the operand is the bf16 number 128 + u, there are no bf16 subnormals to use:
+// their products with x would leave the fp32 range)
+template <int BITS, bool XBF>
+__device__ __forceinline__ Frag16 sub_operand(const u32x4_t (&q)[BITS == 4 ? 1 : 2], int r, uint32_t magic)
 {
     Frag16 b;
-    if (BITS == 4) {
+    if (XBF) {
+        uint32_t o[4];
+        if (BITS == 4) unpack_q4_bf16_biased(q[0][2 * (r >> 1)], q[0][2 * (r >> 1) + 1], r & 1, magic, o);
+        else unpack_q8_bf16_biased(q[BITS == 4 ? 0 : (r >> 1)][(r & 1) * 2], q[BITS == 4 ? 0 : (r >> 1)][(r & 1) * 2 + 1], o);
+        b.u = (u32x4_t){o[0], o[1], o[2], o[3]};
+    } else if (BITS == 4) {
         uint32_t o[4];
         unpack_q4_sub(q[0][2 * (r >> 1)], q[0][2 * (r >> 1) + 1], r & 1, o);
         b.u = (u32x4_t){o[0], o[1], o[2], o[3]};
@@ -77,7 +84,9 @@ __device__ __forceinline__ Frag16 sub_operand(const u32x4_t (&q)[BITS == 4 ? 1 :
 // and lane block b ends up with batch row b / (4 / MR) and the tiles t = b mod (4 / MR), + 4 / MR, ...
 // of the set.  (The scheme works for four rows as well - 12 load instructions per set instead of 6 -
 // and was measured slower there than the batched-rows kernel: 8.8 against 8.6 us at 4096 -> 14336.)
-template <int BITS, int SETS, int NS, bool EVEN, int NW, bool SPLIT = false, bool RES = false, int MR = 1>
+// XBF: bf16 activations (bf16 MFMA, biased weight operands 128 + u, the constant operand is -136 / -128 for
+// every group and nothing is left to fold into the final scaling).
+template <int BITS, int SETS, int NS, bool EVEN, int NW, bool SPLIT = false, bool RES = false, int MR = 1, bool XBF = false>
 // The arguments are scalars in the order the kernel needs them: the compiler is asked to have
 // them delivered in registers at wave start (kernel argument preload), so the first requests do
 // not wait for a load of the argument block.  (13 dwords; the launch's wave count travels with
@@ -201,8 +210,15 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
     }
 
     Frag16 kL, kH;
-    constexpr uint32_t cH = BITS == 4 ? kSubBiasH : kSubBiasQ8;
-    constexpr float unscale = BITS == 4 ? kSubUnscale : kSubUnscaleQ8;
+    constexpr bool TWO = BITS == 4 && !XBF;           // even and odd groups carry different factors
+    constexpr uint32_t cH = XBF ? (BITS == 4 ? kBf16Neg136x2 : kBf16Neg128x2) : (BITS == 4 ? kSubBiasH : kSubBiasQ8);
+    constexpr float unscale = XBF ? 1.0f : (BITS == 4 ? kSubUnscale : kSubUnscaleQ8);
+    uint32_t magic = 0;
+    if constexpr (XBF && BITS == 4) magic = q4_magic_vgpr_bf16();
+    auto mma = [](const Frag16& a, const Frag16& b, float4_t c) {
+        if constexpr (XBF) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, c, 0, 0, 0);
+        else return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, c, 0, 0, 0);
+    };
     kL.u = (u32x4_t){kSubBiasL, kSubBiasL, kSubBiasL, kSubBiasL};
     kH.u = (u32x4_t){cH, cH, cH, cH};
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
@@ -211,8 +227,8 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
     for (int h = 0; h < SETS; h++)
 #pragma unroll
         for (int p = 0; p < MR; p++) {
-            if (BITS == 4) biasL[h][p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[h][p].h, kL.h, zero, 0, 0, 0);
-            biasH[h][p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[h][p].h, kH.h, zero, 0, 0, 0);
+            if (TWO) biasL[h][p] = mma(a[h][p], kL, zero);
+            biasH[h][p] = mma(a[h][p], kH, zero);
         }
 
     // A lane block holds meaningful sums only for its own tiles of every set (one in TPA).  All
@@ -234,8 +250,8 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
             const int st = i / (SETS * 4), h = (i / 4) % SETS, b = i % 4, p = b / TPA;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const Frag16 B = sub_operand<BITS>(q[st][h][b], r);
-                d[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[h][p].h, B.h, (BITS == 8 || (r & 1)) ? biasH[h][p] : biasL[h][p], 0, 0, 0);
+                const Frag16 B = sub_operand<BITS, XBF>(q[st][h][b], r, magic);
+                d[r] = mma(a[h][p], B, (!TWO || (r & 1)) ? biasH[h][p] : biasL[h][p]);
             }
         }
         if (i > 0) {
@@ -244,7 +260,7 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
             for (int r = 0; r < 4; r++) {
                 const uint32_t sb = (r & 1) ? (sc[st][h][p][r >> 1] >> 16) : (sc[st][h][p][r >> 1] & 0xffffu);
                 const float sf = f16_bits_to_f32(sb);
-                if (BITS == 4 && (r & 1)) accH[st][slot] = __builtin_fmaf(sf, dprev[r][r], accH[st][slot]);
+                if (TWO && (r & 1)) accH[st][slot] = __builtin_fmaf(sf, dprev[r][r], accH[st][slot]);
                 else accL[st][slot] = __builtin_fmaf(sf, dprev[r][r], accL[st][slot]);
             }
         }
@@ -264,7 +280,7 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
     for (int st = 0; st < NL; st++) {
         float tb[TPA];
 #pragma unroll
-        for (int b = 0; b < TPA; b++) tb[b] = BITS == 4 ? accL[st][b] + accH[st][b] * 0.0625f : accL[st][b];
+        for (int b = 0; b < TPA; b++) tb[b] = TWO ? accL[st][b] + accH[st][b] * 0.0625f : accL[st][b];
         float t = tb[0];
 #pragma unroll
         for (int b = 1; b < TPA; b++) t = my_tile == b ? tb[b] : t;
@@ -340,7 +356,7 @@ Shape1 shape_of(const WeightView& w)
     return s;
 }
 
-template <int BITS, int SETS, int NS, int MR>
+template <int BITS, int SETS, int NS, int MR, bool XBF>
 hipError_t launch1_e(const WeightView& w, const void* x, int M, void* y, int ydt, const Shape1& sh, const Epilogue& epi,
                      hipStream_t st)
 {
@@ -349,7 +365,7 @@ hipError_t launch1_e(const WeightView& w, const void* x, int M, void* y, int ydt
     const _Float16* xh = reinterpret_cast<const _Float16*>(x);
     const int flags = ydt | (epi.kind << 4) | (M << 8);
 #define CYBQ_GEMV1_LAUNCH(EVEN_, NW_, SPLIT_, RES_, BLOCK_)                                                                          \
-    hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, EVEN_, NW_, SPLIT_, RES_, MR>), grid, BLOCK_, 0, st, w.base, xh, epi.residual, y, \
+    hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, EVEN_, NW_, SPLIT_, RES_, MR, XBF>), grid, BLOCK_, 0, st, w.base, xh, epi.residual, y, \
                        w.KT, w.K, nwaves, w.N, flags)
     const bool k8 = sh.k8 && SETS == 1;
     if constexpr (NS == 2) {
@@ -377,33 +393,37 @@ hipError_t launch1_e(const WeightView& w, const void* x, int M, void* y, int ydt
     return hipGetLastError();
 }
 
-template <int BITS, int NS, int MR>
+template <int BITS, int NS, int MR, bool XBF>
 hipError_t launch1_s(const WeightView& w, const void* x, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st)
 {
     const Shape1 sh = shape_of(w);
     constexpr int MAXS = max_sets_per_wave(BITS, NS, MR);
-    if (sh.per_wave == 1) return launch1_e<BITS, 1, NS, MR>(w, x, M, y, ydt, sh, epi, st);
+    if (sh.per_wave == 1) return launch1_e<BITS, 1, NS, MR, XBF>(w, x, M, y, ydt, sh, epi, st);
     if constexpr (MAXS >= 2) {
-        if (sh.per_wave == 2) return launch1_e<BITS, 2, NS, MR>(w, x, M, y, ydt, sh, epi, st);
+        if (sh.per_wave == 2) return launch1_e<BITS, 2, NS, MR, XBF>(w, x, M, y, ydt, sh, epi, st);
     }
     if constexpr (MAXS >= 3) {
-        if (sh.per_wave == 3) return launch1_e<BITS, 3, NS, MR>(w, x, M, y, ydt, sh, epi, st);
+        if (sh.per_wave == 3) return launch1_e<BITS, 3, NS, MR, XBF>(w, x, M, y, ydt, sh, epi, st);
     }
     return hipErrorInvalidValue;         // gemv1_serves() said no
 }
 
 template <int BITS, int NS>
-hipError_t launch1_m(const WeightView& w, const void* x, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st)
+hipError_t launch1_m(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st)
 {
-    if (M == 1) return launch1_s<BITS, NS, 1>(w, x, M, y, ydt, epi, st);
-    return launch1_s<BITS, NS, 2>(w, x, M, y, ydt, epi, st);
+    if (xdt == kBF16) {
+        if (M == 1) return launch1_s<BITS, NS, 1, true>(w, x, M, y, ydt, epi, st);
+        return launch1_s<BITS, NS, 2, true>(w, x, M, y, ydt, epi, st);
+    }
+    if (M == 1) return launch1_s<BITS, NS, 1, false>(w, x, M, y, ydt, epi, st);
+    return launch1_s<BITS, NS, 2, false>(w, x, M, y, ydt, epi, st);
 }
 
 }  // namespace
 
 bool gemv1_serves(const WeightView& w, int xdt, int M, const Epilogue& epi)
 {
-    if (M < 1 || M > 2 || xdt != kF16 || epi.gamma) return false;
+    if (M < 1 || M > 2 || xdt == kF32 || epi.gamma) return false;
     const int mr = M;
     const int ns = epi.kind == kEpiSwiglu ? 2 : 1;
     const Shape1 sh = shape_of(w);
@@ -411,14 +431,14 @@ bool gemv1_serves(const WeightView& w, int xdt, int M, const Epilogue& epi)
     return sh.per_wave <= max_sets_per_wave(w.bits, ns, mr);
 }
 
-hipError_t launch_gemv1(const WeightView& w, const void* x, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st)
+hipError_t launch_gemv1(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st)
 {
     if (epi.kind == kEpiSwiglu) {
-        if (w.bits == 4) return launch1_m<4, 2>(w, x, M, y, ydt, epi, st);
-        return launch1_m<8, 2>(w, x, M, y, ydt, epi, st);
+        if (w.bits == 4) return launch1_m<4, 2>(w, x, xdt, M, y, ydt, epi, st);
+        return launch1_m<8, 2>(w, x, xdt, M, y, ydt, epi, st);
     }
-    if (w.bits == 4) return launch1_m<4, 1>(w, x, M, y, ydt, epi, st);
-    return launch1_m<8, 1>(w, x, M, y, ydt, epi, st);
+    if (w.bits == 4) return launch1_m<4, 1>(w, x, xdt, M, y, ydt, epi, st);
+    return launch1_m<8, 1>(w, x, xdt, M, y, ydt, epi, st);
 }
 
 }  // namespace cybq

@@ -87,11 +87,12 @@ typedef enum cybq_dtype { CYBQ_F32 = 0, CYBQ_F16 = 1, CYBQ_BF16 = 2 } cybq_dtype
  *          the fp32 CPU path only by accumulation order.  Half the throughput. */
 typedef enum cybq_prefill_mode { CYBQ_PREFILL_FAST = 0, CYBQ_PREFILL_EXACT = 1 } cybq_prefill_mode;
 
-/* How the decode kernel for one and two rows of f16 activations forms its weight operands.  Both
+/* How the decode kernel for one and two rows of 16-bit activations forms its weight operands.  Both
  * accumulate in fp32 and stay far inside the 1e-3 tolerance.
- *   STREAM (default) the packed nibbles / bytes are used as f16 subnormals (q + bias) * 2^-22
- *          straight from memory and the bias is removed inside the same fp32 accumulation;
- *          about 4e-7 relative L2 (the sums carry the bias until it cancels: a tensor of zeros
+ *   STREAM (default) the packed nibbles / bytes are used straight from memory - as f16 subnormals
+ *          (q + bias) * 2^-22 with f16 activations, as the bf16 numbers 128 + (q + bias) with bf16
+ *          activations - and the bias is removed inside the same fp32 accumulation; about 4e-7
+ *          (bf16: 1e-6) relative L2 (the sums carry the bias until it cancels: a tensor of zeros
  *          gives values around 1e-7 of the activations' scale, not exact zeros), the quickest form.
  *   EXACT  the weight operand is the exact integer q (more unpack arithmetic per byte);
  *          about 3e-7 relative L2, and a tensor of zeros gives exact zeros. */

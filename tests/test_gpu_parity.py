@@ -275,15 +275,16 @@ def test_decode_batched_rows_equal_single_rows_bitwise(backend, oracle):
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("shape", [(64, 128), (48, 160), (100, 4096 + 96), (4096, 4096), (256, 14336), (64, 11008),
                                    (32, 16384), (16, 24576), (16, 32768)])
-def test_one_row_kernel_shapes(backend, oracle, bits, shape):
-    """One and two f16 rows (subnormal weight operands, bias removed inside the accumulation; the 16
+@pytest.mark.parametrize("xdt", ["f16", "bf16"])
+def test_one_row_kernel_shapes(backend, oracle, bits, shape, xdt):
+    """One and two f16 / bf16 rows (subnormal weight operands - bf16: 128 + u -, bias removed inside the accumulation; the 16
     rows of an activation operand are 1 / 2 batch rows x 16 / 8 scale groups): whole and ragged
     sets of K tiles, one to three sets per wave, and K beyond what the kernel serves (3 and 4 rows
     take the batched-rows kernel)."""
     N, K = shape
     q, s = _quant(oracle, bits, N, K)
     qw = backend.upload_quantized(q, s, bits, formats.BLOCK_AOS if N % 32 else formats.PLANAR)
-    x4 = _x(4, K, "f16", outliers=0.001)
+    x4 = _x(4, K, xdt, outliers=0.001)
     ref = oracle.matmul_f64(q, s, x4.float().cpu().numpy())
     for M in (1, 2, 3, 4):
         x = x4[:M].contiguous()
