@@ -86,22 +86,31 @@ __device__ __forceinline__ Frag16 sub_operand(const u32x4_t (&q)[BITS == 4 ? 1 :
 // and was measured slower there than the batched-rows kernel: 8.8 against 8.6 us at 4096 -> 14336.)
 // XBF: bf16 activations (bf16 MFMA, biased weight operands 128 + u, the constant operand is -136 / -128 for
 // every group and nothing is left to fold into the final scaling).
-template <int BITS, int SETS, int NS, bool EVEN, int NW, bool SPLIT = false, bool RES = false, int MR = 1, bool XBF = false>
+// NORM: RMSNorm folded in (y = epilogue(rstd[m] * sum_k round(x * gamma) * W), rstd = 1 / sqrt(mean x^2 + eps)):
+// gamma is requested next to x, the operand becomes x * gamma (fp32, rounded once to the operand type) in
+// registers, the squares of x are summed per wave on the way and meet across waves with the partial sums.
+template <int BITS, int SETS, int NS, bool EVEN, int NW, bool SPLIT = false, bool RES = false, int MR = 1, bool XBF = false,
+          bool NORM = false>
 // The arguments are scalars in the order the kernel needs them: the compiler is asked to have
 // them delivered in registers at wave start (kernel argument preload), so the first requests do
-// not wait for a load of the argument block.  (13 dwords; the launch's wave count travels with
-// them, the launch geometry is not among what is preloaded.  flags = output type | epilogue << 4 | M << 8.)
+// not wait for a load of the argument block.  (14 dwords are preloaded; the launch's wave count travels
+// with them, the launch geometry is not among what is preloaded.  flags = output type | epilogue << 4 |
+// M << 8 | gamma type << 16.  aux0: the residual, or gamma with a folded norm - then the residual is aux1.)
 __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__ wbase, const _Float16* __restrict__ x,
-                                                     const void* __restrict__ residual, void* __restrict__ y, int KT, int K,
-                                                     int launch_waves, int n_rows, int flags)
+                                                     const void* __restrict__ aux0, void* __restrict__ y, int KT, int K,
+                                                     int launch_waves, int n_rows, int flags, float eps,
+                                                     const void* __restrict__ aux1)
 {
+    static_assert(!(NORM && RES), "the residual prefetch has no folded-norm form");
+    const void* const residual = NORM ? aux1 : aux0;
     static_assert(MR == 1 || MR == 2, "batch rows per operand");
     static_assert(!RES || MR == 1, "the residual prefetch is the one-row form");
     constexpr int QV = BITS == 4 ? 1 : 2;
     constexpr int GPA = 16 / MR;                  // scale groups per A operand
     constexpr int TPA = 4 / MR;                   // tiles per A operand
     __shared__ float red[NS * MR * 16 * 16];
-    const int out_dt = flags & 15, epi_kind = (flags >> 4) & 15, M = flags >> 8;
+    __shared__ float ssq_red[NORM ? MR * 16 : 1];       // [batch row][wave]
+    const int out_dt = flags & 15, epi_kind = (flags >> 4) & 15, M = (flags >> 8) & 255, gdt = (flags >> 16) & 15;
     const int tid = threadIdx.x, lane = tid & 63;
     static_assert(!SPLIT || (NS == 2 && NW > 0), "split workgroups are gate / up pairs with a known wave count");
     constexpr int NL = SPLIT ? 1 : NS;            // strips a wave works on
@@ -129,6 +138,7 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
     if constexpr (MR > 1) xrow += min(row / GPA, M - 1) * K;
     const int xk = (row % GPA) * 32 + blk * 8;
     Frag16 a[SETS][MR];
+    u32x4_t gam[NORM ? SETS : 1][MR][2];      // NORM: gamma at the operand's k (fp32: 32 bytes, else 16 and a repeat)
     u32x2_t sc[NL][SETS][MR];
     u32x4_t q[NL][SETS][4][QV];
     bool tile_ok[SETS][MR];           // this lane block's tiles of the set exist (!EVEN)
@@ -138,11 +148,14 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
 #pragma unroll
         for (int p = 0; p < MR; p++) {
             const int k = set * 512 + p * (TPA * 128) + xk;
-            if (EVEN) {
-                a[h][p].u = *reinterpret_cast<const u32x4_t*>(xrow + k);
-            } else {
-                a[h][p].u = *reinterpret_cast<const u32x4_t*>(xrow + min(k, K - 8));
-                tile_ok[h][p] = 4 * set + my_tile + TPA * p < KT;
+            const int kc = EVEN ? k : min(k, K - 8);
+            a[h][p].u = *reinterpret_cast<const u32x4_t*>(xrow + kc);
+            if (!EVEN) tile_ok[h][p] = 4 * set + my_tile + TPA * p < KT;
+            if constexpr (NORM) {
+                const int esz = gdt == kF32 ? 4 : 2;
+                const char* gp = static_cast<const char*>(aux0) + (int64_t)kc * esz;
+                gam[h][p][0] = *reinterpret_cast<const u32x4_t*>(gp);
+                gam[h][p][1] = *reinterpret_cast<const u32x4_t*>(gp + (esz == 4 ? 16 : 0));
             }
         }
     }
@@ -209,6 +222,51 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
         }
     }
 
+    float ssq = 0.f;                  // NORM: squares of the activations this lane holds (batch row (lane & 15) / GPA)
+    if constexpr (NORM) {
+#pragma unroll
+        for (int h = 0; h < SETS; h++)
+#pragma unroll
+            for (int p = 0; p < MR; p++) {
+                float g[8];
+                if (gdt == kF32) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const uint32_t lo = gam[h][p][0][e], hi = gam[h][p][1][e];       // (values first: a bit cast
+                        g[e] = __builtin_bit_cast(float, lo);                             // straight from a vector
+                        g[4 + e] = __builtin_bit_cast(float, hi);                         // element read element 0)
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const uint32_t v = gam[h][p][0][e];
+                        g[2 * e] = gdt == kF16 ? f16_bits_to_f32(v & 0xffffu) : __builtin_bit_cast(float, v << 16);
+                        g[2 * e + 1] = gdt == kF16 ? f16_bits_to_f32(v >> 16) : __builtin_bit_cast(float, v & 0xffff0000u);
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const uint32_t v = a[h][p].u[e];
+                    float x0, x1;
+                    if (XBF) {
+                        x0 = __builtin_bit_cast(float, v << 16);
+                        x1 = __builtin_bit_cast(float, v & 0xffff0000u);
+                    } else {
+                        x0 = f16_bits_to_f32(v & 0xffffu);
+                        x1 = f16_bits_to_f32(v >> 16);
+                    }
+                    ssq = __builtin_fmaf(x1, x1, __builtin_fmaf(x0, x0, ssq));
+                    x0 *= g[2 * e];
+                    x1 *= g[2 * e + 1];
+                    if (XBF) {
+                        a[h][p].u[e] = pack_bf16x2(x0, x1);
+                    } else {
+                        const half2_t hh = {(_Float16)x0, (_Float16)x1};
+                        a[h][p].u[e] = as_u32(hh);
+                    }
+                }
+            }
+    }
     Frag16 kL, kH;
     constexpr bool TWO = BITS == 4 && !XBF;           // even and odd groups carry different factors
     constexpr uint32_t cH = XBF ? (BITS == 4 ? kBf16Neg136x2 : kBf16Neg128x2) : (BITS == 4 ? kSubBiasH : kSubBiasQ8);
@@ -290,6 +348,17 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
             for (int m = 0; m < MR; m++) red[(((st + half) * MR + m) * 16 + wv) * 16 + lane] = sum[m];
         }
     }
+    if constexpr (NORM) {
+        // rows of the operand first (the four lane blocks of a row meet in an fp32 MFMA against ones), then the
+        // rows that belong to a batch row: the same 0/1 matrix that joins the lane blocks' sums
+        const float4_t r1 = __builtin_amdgcn_mfma_f32_16x16x4f32(ssq, 1.0f, zero4, 0, 0, 0);
+        const float t = (r1[0] + r1[1]) + (r1[2] + r1[3]);
+        const float4_t r2 = __builtin_amdgcn_mfma_f32_16x16x4f32(mine, t, zero4, 0, 0, 0);
+        if (lane == 0 && half == 0) {
+#pragma unroll
+            for (int m = 0; m < MR; m++) ssq_red[m * 16 + wv] = r2[m];
+        }
+    }
     __syncthreads();
     if (tid >= 64) return;
     constexpr int SLOTS = NW ? (NW + 3) / 4 : 4;
@@ -306,6 +375,16 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
             for (int i = 0; i < SLOTS; i++) v += 4 * i + blk < nwaves ? t[i] : 0.f;
             outv[st][m] = __builtin_amdgcn_mfma_f32_16x16x4f32(1.0f, v, zero4, 0, 0, 0)[0] * unscale;
         }
+    if constexpr (NORM) {
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+            float t = 0.f;
+            for (int k = 0; k < nwaves; k++) t += ssq_red[m * 16 + k];
+            const float rstd = 1.0f / sqrtf(t / (float)K + eps);
+#pragma unroll
+            for (int st = 0; st < NS; st++) outv[st][m] *= rstd;
+        }
+    }
     if (lane >= 16) return;
     const int n = blockIdx.x * 16 + lane;
     if (NS == 2) {               // SwiGLU: strips 2i / 2i+1 are gate / up of output strip i
@@ -323,7 +402,7 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
                 const uint32_t h = (res_addr & 2u) ? res_word >> 16 : res_word & 0xffffu;
                 v += out_dt == kF32 ? __builtin_bit_cast(float, res_word)
                                     : (out_dt == kF16 ? f16_bits_to_f32(h) : __builtin_bit_cast(float, h << 16));
-            } else if (MR > 1 && epi_kind == kEpiAdd) {
+            } else if ((MR > 1 || NORM) && epi_kind == kEpiAdd) {
                 if (m < M) v += load_out1(residual, out_dt, (int64_t)m * n_rows + n);
             }
             if (m < M) store_out1(y, out_dt, (int64_t)m * n_rows + n, v);
@@ -333,9 +412,11 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
 
 // sets of four K tiles a wave may own (all of them in registers, 16 waves per workgroup at
 // most: 128 registers per lane): two, three for Q4 with one strip per workgroup, one for
-// Q8 gate / up pairs; with two batch rows per operand two (Q4, one strip) or one
-constexpr int max_sets_per_wave(int bits, int ns, int mr)
+// Q8 gate / up pairs; with two batch rows per operand two (Q4, one strip) or one; with a folded norm
+// (gamma travels in registers next to x) two for one row and one strip, else one
+constexpr int max_sets_per_wave(int bits, int ns, int mr, bool norm)
 {
+    if (norm) return ns == 1 && mr == 1 ? 2 : 1;
     if (mr == 1) return bits == 4 ? (ns == 1 ? 3 : 2) : (ns == 1 ? 2 : 1);
     return bits == 4 && ns == 1 ? 2 : 1;
 }
@@ -356,17 +437,18 @@ Shape1 shape_of(const WeightView& w)
     return s;
 }
 
-template <int BITS, int SETS, int NS, int MR, bool XBF>
+template <int BITS, int SETS, int NS, int MR, bool XBF, bool NORM>
 hipError_t launch1_e(const WeightView& w, const void* x, int M, void* y, int ydt, const Shape1& sh, const Epilogue& epi,
                      hipStream_t st)
 {
     const int nwaves = sh.nwaves;
     const dim3 grid((unsigned)(w.NT / NS)), block((unsigned)nwaves * 64);
     const _Float16* xh = reinterpret_cast<const _Float16*>(x);
-    const int flags = ydt | (epi.kind << 4) | (M << 8);
+    const int flags = ydt | (epi.kind << 4) | (M << 8) | (epi.gamma_dt << 16);
+    const void* aux0 = NORM ? epi.gamma : epi.residual;
 #define CYBQ_GEMV1_LAUNCH(EVEN_, NW_, SPLIT_, RES_, BLOCK_)                                                                          \
-    hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, EVEN_, NW_, SPLIT_, RES_, MR, XBF>), grid, BLOCK_, 0, st, w.base, xh, epi.residual, y, \
-                       w.KT, w.K, nwaves, w.N, flags)
+    hipLaunchKernelGGL((gemv1_kernel<BITS, SETS, NS, EVEN_, NW_, SPLIT_, (RES_) && !NORM, MR, XBF, NORM>), grid, BLOCK_, 0, st, w.base, xh, \
+                       aux0, y, w.KT, w.K, nwaves, w.N, flags, epi.eps, epi.residual)
     const bool k8 = sh.k8 && SETS == 1;
     if constexpr (NS == 2) {
         if constexpr (SETS == 1) {
@@ -378,8 +460,8 @@ hipError_t launch1_e(const WeightView& w, const void* x, int M, void* y, int ydt
             if (sh.even) CYBQ_GEMV1_LAUNCH(true, 0, false, false, block);
             else CYBQ_GEMV1_LAUNCH(false, 0, false, false, block);
         } else return hipErrorInvalidValue;
-    } else if (MR == 1 && epi.kind == kEpiAdd) {
-        if constexpr (MR == 1) {
+    } else if (MR == 1 && !NORM && epi.kind == kEpiAdd) {
+        if constexpr (MR == 1 && !NORM) {
             if (k8) CYBQ_GEMV1_LAUNCH(true, (SETS == 1 ? 8 : 0), false, true, block);
             else if (sh.even) CYBQ_GEMV1_LAUNCH(true, 0, false, true, block);
             else CYBQ_GEMV1_LAUNCH(false, 0, false, true, block);
@@ -393,42 +475,49 @@ hipError_t launch1_e(const WeightView& w, const void* x, int M, void* y, int ydt
     return hipGetLastError();
 }
 
-template <int BITS, int NS, int MR, bool XBF>
+template <int BITS, int NS, int MR, bool XBF, bool NORM>
 hipError_t launch1_s(const WeightView& w, const void* x, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st)
 {
     const Shape1 sh = shape_of(w);
-    constexpr int MAXS = max_sets_per_wave(BITS, NS, MR);
-    if (sh.per_wave == 1) return launch1_e<BITS, 1, NS, MR, XBF>(w, x, M, y, ydt, sh, epi, st);
+    constexpr int MAXS = max_sets_per_wave(BITS, NS, MR, NORM);
+    if (sh.per_wave == 1) return launch1_e<BITS, 1, NS, MR, XBF, NORM>(w, x, M, y, ydt, sh, epi, st);
     if constexpr (MAXS >= 2) {
-        if (sh.per_wave == 2) return launch1_e<BITS, 2, NS, MR, XBF>(w, x, M, y, ydt, sh, epi, st);
+        if (sh.per_wave == 2) return launch1_e<BITS, 2, NS, MR, XBF, NORM>(w, x, M, y, ydt, sh, epi, st);
     }
     if constexpr (MAXS >= 3) {
-        if (sh.per_wave == 3) return launch1_e<BITS, 3, NS, MR, XBF>(w, x, M, y, ydt, sh, epi, st);
+        if (sh.per_wave == 3) return launch1_e<BITS, 3, NS, MR, XBF, NORM>(w, x, M, y, ydt, sh, epi, st);
     }
     return hipErrorInvalidValue;         // gemv1_serves() said no
+}
+
+template <int BITS, int NS, bool NORM>
+hipError_t launch1_x(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st)
+{
+    if (xdt == kBF16) {
+        if (M == 1) return launch1_s<BITS, NS, 1, true, NORM>(w, x, M, y, ydt, epi, st);
+        return launch1_s<BITS, NS, 2, true, NORM>(w, x, M, y, ydt, epi, st);
+    }
+    if (M == 1) return launch1_s<BITS, NS, 1, false, NORM>(w, x, M, y, ydt, epi, st);
+    return launch1_s<BITS, NS, 2, false, NORM>(w, x, M, y, ydt, epi, st);
 }
 
 template <int BITS, int NS>
 hipError_t launch1_m(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st)
 {
-    if (xdt == kBF16) {
-        if (M == 1) return launch1_s<BITS, NS, 1, true>(w, x, M, y, ydt, epi, st);
-        return launch1_s<BITS, NS, 2, true>(w, x, M, y, ydt, epi, st);
-    }
-    if (M == 1) return launch1_s<BITS, NS, 1, false>(w, x, M, y, ydt, epi, st);
-    return launch1_s<BITS, NS, 2, false>(w, x, M, y, ydt, epi, st);
+    if (epi.gamma) return launch1_x<BITS, NS, true>(w, x, xdt, M, y, ydt, epi, st);
+    return launch1_x<BITS, NS, false>(w, x, xdt, M, y, ydt, epi, st);
 }
 
 }  // namespace
 
 bool gemv1_serves(const WeightView& w, int xdt, int M, const Epilogue& epi)
 {
-    if (M < 1 || M > 2 || xdt == kF32 || epi.gamma) return false;
+    if (M < 1 || M > 2 || xdt == kF32) return false;
     const int mr = M;
     const int ns = epi.kind == kEpiSwiglu ? 2 : 1;
     const Shape1 sh = shape_of(w);
     if (mr > 1 && ns == 2 && !sh.k8) return false;          // pairs with several rows: split workgroups only
-    return sh.per_wave <= max_sets_per_wave(w.bits, ns, mr);
+    return sh.per_wave <= max_sets_per_wave(w.bits, ns, mr, epi.gamma != nullptr);
 }
 
 hipError_t launch_gemv1(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt, const Epilogue& epi, hipStream_t st)
