@@ -458,11 +458,13 @@ def main():
         # one native walk over the linear nodes per step (BASELINE configs[4])
         from cyb_amd import stack as stk
         stack_out = {}
-        for label, shapes, epis in (("per_linear_224_launches", None, False),
-                                    ("qkv_and_gate_up_fused_128_launches", stk.fused_shapes(), False),
-                                    ("fused_128_launches_swiglu_and_residual_epilogues", stk.fused_shapes(), True)):
+        for label, shapes, epis, norms in (("per_linear_224_launches", None, False, False),
+                                           ("qkv_and_gate_up_fused_128_launches", stk.fused_shapes(), False, False),
+                                           ("fused_128_launches_swiglu_and_residual_epilogues", stk.fused_shapes(), True, False),
+                                           ("fused_128_launches_rmsnorm_swiglu_and_residual_folded", stk.fused_shapes(), True, True)):
             t0 = time.time()
-            st = stk.build(be, layers=32, seed=5, shapes=shapes, order=list(shapes) if shapes else None, epilogues=epis)
+            st = stk.build(be, layers=32, seed=5, shapes=shapes, order=list(shapes) if shapes else None, epilogues=epis,
+                           norms=norms)
             log(f"stack {label} built in {time.time() - t0:.1f}s: {st.weight_bytes} weight bytes")
             res = {"weight_bytes": int(st.weight_bytes), "launches_per_step": len(st.nodes)}
             for Ms in (1, 8):

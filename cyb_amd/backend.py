@@ -83,6 +83,7 @@ def load_library() -> ctypes.CDLL:
     lib.cybq_matmul_norm.argtypes = [vp, vp, vp, ci, i64, vp, ci, ctypes.c_float, vp, ci, ci, vp, vp]
     lib.cybq_weight_fuse_pairs.argtypes = [vp, vp, vp, ctypes.POINTER(vp)]
     lib.cybq_matmul_many_ex.argtypes = [vp, i64, vp, vp, vp, vp, vp, ci, i64, ci, vp]
+    lib.cybq_matmul_many_norm.argtypes = [vp, i64, vp, vp, vp, ci, ctypes.c_float, vp, vp, vp, ci, i64, ci, vp]
     lib.cybq_set_prefill_mode.argtypes = [vp, ci]
     lib.cybq_set_decode_mode.argtypes = [vp, ci]
     lib.cybq_matmul_many.argtypes = [vp, i64, vp, vp, vp, ci, i64, ci, vp]
@@ -172,7 +173,7 @@ class QWeight:
 class MatmulPlan:
     """Pointer arrays of a fixed node list (one decode step's linears)."""
 
-    def __init__(self, backend: "Backend", weights, xs, ys, epilogues=None, residuals=None):
+    def __init__(self, backend: "Backend", weights, xs, ys, epilogues=None, residuals=None, gammas=None, eps: float = 1e-5):
         n = len(weights)
         if not (n == len(xs) == len(ys)):
             raise CybqError(-1, "invalid argument", "weights / xs / ys differ in length")
@@ -191,6 +192,20 @@ class MatmulPlan:
                 raise CybqError(-1, "invalid argument", "epilogues / residuals differ in length from the node list")
             self.epi = (ctypes.c_int * n)(*[EPILOGUES[e] for e in epilogues])
             self.res = arr(*[_ptr(r) for r in (residuals or [None] * n)])
+        # folded RMSNorm per node (None = no norm in front of that node): cybq_matmul_many_norm
+        self.gamma = None
+        self.eps = float(eps)
+        self.gdt = F32
+        if gammas is not None:
+            if len(gammas) != n:
+                raise CybqError(-1, "invalid argument", "gammas differ in length from the node list")
+            given = [g for g in gammas if g is not None]
+            if given:
+                self.gdt = _dtype_code(given[0], None)
+                if any(_dtype_code(g, None) != self.gdt for g in given):
+                    raise CybqError(-1, "invalid argument", "all gammas of a plan share one type")
+                self.gamma = arr(*[_ptr(g) for g in gammas])
+                self.keep = self.keep + (list(gammas),)
 
 
 class Backend:
@@ -342,19 +357,25 @@ class Backend:
             self.weights[name] = w
         return w
 
-    def plan_many(self, weights, xs, ys, epilogues=None, residuals=None) -> "MatmulPlan":
-        """Freezes a list of (weight, x, y[, epilogue, residual]) nodes into pointer arrays for matmul_many."""
-        return MatmulPlan(self, weights, xs, ys, epilogues, residuals)
+    def plan_many(self, weights, xs, ys, epilogues=None, residuals=None, gammas=None, eps: float = 1e-5) -> "MatmulPlan":
+        """Freezes a list of (weight, x, y[, epilogue, residual, gamma]) nodes into pointer arrays for matmul_many."""
+        return MatmulPlan(self, weights, xs, ys, epilogues, residuals, gammas, eps)
 
     def matmul_many(self, plan: "MatmulPlan", M: int, stream: int = 0) -> None:
         if M not in plan.checked:                      # once per plan and batch size, not per step
-            ws, xs, ys, rs = plan.keep
+            ws, xs, ys, rs = plan.keep[:4]
+            gs = plan.keep[4] if len(plan.keep) > 4 else None
             for i, w in enumerate(ws):
                 epi = "none"
                 if plan.epi is not None:
                     epi = next(k for k, v in EPILOGUES.items() if v == plan.epi[i])
-                self._check_call(w, xs[i], ys[i], M, epi, rs[i] if rs else None)
+                self._check_call(w, xs[i], ys[i], M, epi, rs[i] if rs else None, gs[i] if gs else None)
             plan.checked.add(M)
+        if plan.gamma is not None:
+            self._check(self._lib.cybq_matmul_many_norm(self._ctx, plan.count, plan.w, plan.x, plan.gamma, plan.gdt,
+                                                        ctypes.c_float(plan.eps), plan.y, plan.epi, plan.res, plan.xdt, M,
+                                                        plan.ydt, stream))
+            return
         if plan.epi is not None:
             self._check(self._lib.cybq_matmul_many_ex(self._ctx, plan.count, plan.w, plan.x, plan.y, plan.epi, plan.res,
                                                       plan.xdt, M, plan.ydt, stream))

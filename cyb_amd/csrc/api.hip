@@ -536,6 +536,21 @@ int cybq_matmul_many_ex(cybq_ctx* ctx, int64_t count, const cybq_weight* const* 
     return CYBQ_OK;
 }
 
+int cybq_matmul_many_norm(cybq_ctx* ctx, int64_t count, const cybq_weight* const* w, const void* const* x,
+                          const void* const* gamma, cybq_dtype gdt, float eps, void* const* y, const int* epilogue,
+                          const void* const* residual, cybq_dtype xdt, int64_t M, cybq_dtype ydt, void* stream)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (count < 0 || (count > 0 && (!w || !x || !y))) return fail(ctx, CYBQ_ERR_INVALID, "bad node list");
+    for (int64_t i = 0; i < count; i++) {
+        const cybq_epilogue e = epilogue ? static_cast<cybq_epilogue>(epilogue[i]) : CYBQ_EPI_NONE;
+        int rc = matmul_fused(ctx, w[i], x[i], xdt, M, gamma ? gamma[i] : nullptr, gdt, eps, y[i], ydt, e,
+                              residual ? residual[i] : nullptr, stream, ctx->workspace, ctx->workspace_bytes);
+        if (rc) return rc;
+    }
+    return CYBQ_OK;
+}
+
 int cybq_dequant(cybq_ctx* ctx, const cybq_weight* w, float* out, void* stream)
 {
     if (!ctx) return CYBQ_ERR_INVALID;

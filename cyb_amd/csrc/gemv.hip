@@ -13,6 +13,7 @@
 // an exact small integer and the only rounding is the fp32 accumulation.
 // Split-K partials meet in LDS in a fixed order: results are deterministic and
 // row m of a batch is bit-identical to the same row run alone.
+#include <type_traits>
 #include "cybq_device.h"
 #include "cybq_internal.h"
 
@@ -576,52 +577,83 @@ __device__ __forceinline__ void tile_issue_regs(const TileRegs<BITS>& t, const F
     tile_multiply<BITS, XMODE>(a, b, d);
 }
 
-// NORM: RMSNorm folded into the activation load (epi.gamma / epi.eps): an operand fragment
-// is multiplied by gamma in registers right after it reaches operand order, the lane adds
-// the squares of what it holds; rows meet across lanes and waves in the final exchange.
-template <int XMODE>
-__device__ __forceinline__ void norm_frag(Frag16& a, const float* gamma_lds, int k0, bool counts, float& ssq)
+// NORM: RMSNorm folded into the activation load (epi.gamma / epi.eps).  A lane multiplies the 16 B
+// piece of x it loaded (eight neighbouring k of one row) by gamma and adds up its squares while the
+// piece is still as loaded: every element of the batch is touched once per workgroup, where the
+// operand fragments made from the pieces repeat a batch of four rows four times.  Rows meet
+// across lanes and waves in the final exchange.
+// GH: x and gamma are both f16 - gamma sits in LDS as loaded and the product is one packed f16
+// multiply per pair (the product of two f16 is exact in fp32, so its single rounding to f16 is the
+// rounding the fp32 form makes); otherwise gamma is fp32 in LDS and the pair goes through fp32.
+// v as the lanes named by a DPP control see it (quad permutations, mirrors within a row of 16)
+template <int CTRL>
+__device__ __forceinline__ float lane_cross(float v)
 {
-    float g[8];
-    {
-        const float4_t g0 = reinterpret_cast<const float4_t*>(gamma_lds + k0)[0];
-        const float4_t g1 = reinterpret_cast<const float4_t*>(gamma_lds + k0)[1];
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+// (the LDS reads of a tile's pieces are issued together, ahead of the arithmetic)
+struct GammaPiece {
+    u32x4_t lo, hi;           // 8 x fp32, or (GH) 8 x f16 in lo
+};
+
+template <bool GH>
+__device__ __forceinline__ GammaPiece gamma_piece(const void* gamma_lds, int k)
+{
+    GammaPiece g;
+    if constexpr (GH) {
+        g.lo = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const uint16_t*>(gamma_lds) + k);
+        g.hi = g.lo;
+    } else {
+        g.lo = reinterpret_cast<const u32x4_t*>(reinterpret_cast<const float*>(gamma_lds) + k)[0];
+        g.hi = reinterpret_cast<const u32x4_t*>(reinterpret_cast<const float*>(gamma_lds) + k)[1];
+    }
+    return g;
+}
+
+template <int XMODE, bool GH>
+__device__ __forceinline__ void norm_piece(u32x4_t& v, const GammaPiece& gp, bool counts, float& ssq)
+{
+    float sq = ssq;
+    if constexpr (GH) {
+        const u32x4_t g = gp.lo;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            g[i] = g0[i];
-            g[4 + i] = g1[i];
+        for (int p = 0; p < 4; p++) {
+            const half2_t h = as_h2(v[p]);
+            sq = __builtin_amdgcn_fdot2(h, h, sq, false);
+            v[p] = as_u32(h * as_h2(g[p]));
+        }
+    } else {
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const uint32_t ua = p < 2 ? gp.lo[2 * p] : gp.hi[2 * p - 4], ub = p < 2 ? gp.lo[2 * p + 1] : gp.hi[2 * p - 3];
+            const float ga = __builtin_bit_cast(float, ua), gb = __builtin_bit_cast(float, ub);
+            if (XMODE == XBF16) {
+                const float v0 = __builtin_bit_cast(float, v[p] << 16);
+                const float v1 = __builtin_bit_cast(float, v[p] & 0xffff0000u);
+                sq = fmaf(v1, v1, fmaf(v0, v0, sq));
+                v[p] = pack_bf16x2(v0 * ga, v1 * gb);
+            } else {
+                const half2_t h = as_h2(v[p]);
+                sq = __builtin_amdgcn_fdot2(h, h, sq, false);
+                const half2_t o = {(_Float16)((float)h.x * ga), (_Float16)((float)h.y * gb)};
+                v[p] = as_u32(o);
+            }
         }
     }
-#pragma unroll
-    for (int p = 0; p < 4; p++) {
-        float v0, v1;
-        if (XMODE == XBF16) {
-            v0 = __builtin_bit_cast(float, a.u[p] << 16);
-            v1 = __builtin_bit_cast(float, a.u[p] & 0xffff0000u);
-        } else {
-            const half2_t h = as_h2(a.u[p]);
-            v0 = (float)h.x;
-            v1 = (float)h.y;
-        }
-        if (counts) ssq = fmaf(v1, v1, fmaf(v0, v0, ssq));
-        v0 *= g[2 * p];
-        v1 *= g[2 * p + 1];
-        if (XMODE == XBF16) {
-            a.u[p] = pack_bf16x2(v0, v1);
-        } else {
-            const half2_t h = {(_Float16)v0, (_Float16)v1};
-            a.u[p] = as_u32(h);
-        }
-    }
+    ssq = counts ? sq : ssq;
 }
 
 // MB: blocks of 16 batch rows (2 = 17..32 rows: every unpacked weight operand is multiplied with
 // two activation operands, the weights still stream once).
+// gamma / gamma_dt (NORM) sit ahead of y in the argument list: everything the first loads need is
+// then in the argument registers the hardware fills before the kernel starts.
 template <int BITS, int XMODE, int TS, int NS, bool NORM, int XR, int MB = 1>
 // (waves_per_eu: the scheduler would otherwise trade the up-front loads for occupancy)
-__global__ __launch_bounds__((TS <= 2 && MB == 1) ? 1024 : 512) __attribute__((amdgpu_waves_per_eu(2, (TS <= 2 && MB == 1) ? 4 : 2)))
-void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restrict__ x, int KT_, int K, int NT, int M, int nwaves,
-                      void* __restrict__ y, int N, int ydt, Epilogue epi)
+__global__ __launch_bounds__((TS <= 2 && MB == 1 && !NORM) ? 1024 : 512)
+__attribute__((amdgpu_waves_per_eu(2, (TS <= 2 && MB == 1 && !NORM) ? 4 : 2)))
+void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restrict__ x, const void* __restrict__ gamma, int KT_, int K,
+                      int NT, int M, int nwaves, int gamma_dt, int N, void* __restrict__ y, int ydt, Epilogue epi)
 {
     const WeightView w = {wbase, N, K, NT, KT_, BITS};
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -646,18 +678,14 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
     const int64_t xblock = MB > 1 ? (int64_t)(min(16 + lane / P, M - 1) - min(lane / P, M - 1)) * w.K : 0;     // to my row of the second block
     const int klast = w.K - 8 - (lane % P) * 8;          // last start at which this lane's piece is inside the row
     const int from_lane = ((((lane & 15) & (XR - 1)) * P) | oct) << 2;       // byte address for ds_bpermute (+ 16 per group)
-    // NORM: gamma as fp32 in LDS behind the exchange areas (read per fragment with LDS loads, which
-    // do not queue behind the weight requests the way global loads would)
-    float* gamma_lds = reinterpret_cast<float*>(smem) + NS * MB * nwaves * 4 * 64 + nwaves * 16;
-    if (NORM) {
-        for (int c = tid; c < (w.K >> 3); c += nwaves * 64) {
-            float g[8];
-            load_gamma8(epi.gamma, epi.gamma_dt, c * 8, g);
-            reinterpret_cast<float4_t*>(gamma_lds + c * 8)[0] = (float4_t){g[0], g[1], g[2], g[3]};
-            reinterpret_cast<float4_t*>(gamma_lds + c * 8)[1] = (float4_t){g[4], g[5], g[6], g[7]};
-        }
-        __syncthreads();
-    }
+    // NORM: each wave keeps the gamma of the K tiles it is working on in an LDS area of its own,
+    // behind the exchange areas
+    uint8_t* gamma_lds = smem + ((size_t)NS * MB * nwaves * 4 * 64 + 8 * 16 + (size_t)wv * TS * kTileK) * sizeof(float);
+    const bool gamma_h = NORM && XMODE == XF16 && gamma_dt == kF16;
+    const bool gamma_f32 = NORM && gamma_dt == kF32;
+    const int g_count = gamma_f32 ? 4 : 8;               // values of a tile's gamma a lane loads,
+    const int g_first = (lane & (gamma_f32 ? 31 : 15)) * g_count;       // the first of them,
+    const int g_shift = gamma_f32 ? 2 : 1;               // log2 of their size
 
     float acc[NS][MB][4];
 #pragma unroll
@@ -666,7 +694,7 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
         for (int b = 0; b < MB; b++)
 #pragma unroll
             for (int r = 0; r < 4; r++) acc[s][b][r] = 0.f;
-    float ssq = 0.f;          // NORM: squares of the x values this lane holds (row lane % 16)
+    float ssq = 0.f;          // NORM: squares of the x values this lane loaded (row lane / P)
 
     int64_t sbase[NS];
 #pragma unroll
@@ -677,11 +705,15 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
         int kt[TS];
         bool valid[TS];
         Frag16 a[MB][TS][4];
+        u32x4_t graw[NORM ? TS : 1];        // NORM: gamma of my tiles, 8 values in each of 16 lanes (4 in each of 32: fp32)
 #pragma unroll
         for (int u = 0; u < TS; u++) {
             const int t = slab0 + wv + nwaves * u;
             valid[u] = t < KT;
             kt[u] = min(t, KT - 1);
+            if (NORM)
+                graw[u] = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const uint8_t*>(gamma) +
+                                                            ((size_t)min(kt[u] * kTileK + g_first, w.K - g_count) << g_shift));
 #pragma unroll
             for (int h = 0; h < L; h++) {
                 // (past the end of K: any x inside the row will do, the padded weights are zero)
@@ -704,6 +736,60 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
         for (int s = 0; s < AHEAD; s++)
 #pragma unroll
             for (int u = 0; u < TS; u++) load_tile<BITS>(buf[s][u], w, sbase[s] + kt[u], lane);
+        if (NORM) {
+            // my tiles' gamma -> my LDS area (16 or 32 lanes hold a tile's 128 values; fp32, or as loaded
+            // when x and gamma are both f16), read back below piece by piece: no other wave is involved
+            if (gamma_h) {
+                if (lane < 16) {
+#pragma unroll
+                    for (int u = 0; u < TS; u++) reinterpret_cast<u32x4_t*>(gamma_lds)[u * 16 + lane] = graw[u];
+                }
+            } else if (gamma_f32) {
+                if (lane < 32) {
+#pragma unroll
+                    for (int u = 0; u < TS; u++) reinterpret_cast<u32x4_t*>(gamma_lds)[u * 32 + lane] = graw[u];
+                }
+            } else if (lane < 16) {
+                const bool gh = gamma_dt == kF16;
+#pragma unroll
+                for (int u = 0; u < TS; u++) {
+                    float g[8];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const half2_t h = as_h2(graw[u][i]);
+                        g[2 * i] = gh ? (float)h.x : __builtin_bit_cast(float, graw[u][i] << 16);
+                        g[2 * i + 1] = gh ? (float)h.y : __builtin_bit_cast(float, graw[u][i] & 0xffff0000u);
+                    }
+                    reinterpret_cast<float4_t*>(gamma_lds)[u * 32 + 2 * lane] = (float4_t){g[0], g[1], g[2], g[3]};
+                    reinterpret_cast<float4_t*>(gamma_lds)[u * 32 + 2 * lane + 1] = (float4_t){g[4], g[5], g[6], g[7]};
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            auto norm_all = [&](auto packed) {
+                constexpr bool GH = decltype(packed)::value;
+#pragma unroll
+                for (int u = 0; u < TS; u++) {
+                    GammaPiece g[L];
+                    bool counts[L];
+#pragma unroll
+                    for (int h = 0; h < L; h++) {
+                        const int k0 = kt[u] * kTileK + h * (GPL * 32);
+                        const int kp = k0 + (lane % P) * 8;             // my piece (one past K repeats one inside: not counted)
+                        const int kk = (XR == 16 ? min(k0, w.K - 32) + (lane % P) * 8 : min(kp, w.K - 8)) - kt[u] * kTileK + u * kTileK;
+                        g[h] = gamma_piece<GH>(gamma_lds, kk);
+                        counts[h] = valid[u] && kp < w.K;
+                    }
+#pragma unroll
+                    for (int h = 0; h < L; h++) norm_piece<XMODE, GH>(a[0][u][h].u, g[h], counts[h], ssq);
+                }
+            };
+            if constexpr (XMODE == XF16) {
+                if (gamma_h) norm_all(std::true_type{});
+                else norm_all(std::false_type{});
+            } else norm_all(std::false_type{});
+        }
 #pragma unroll
         for (int b = 0; b < MB; b++)
 #pragma unroll
@@ -718,15 +804,6 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
                         a[b][u][j].u[p] =
                             (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane + (j % GPL) * 16, (int)raw[j / GPL][p]);
             }
-        if (NORM) {
-#pragma unroll
-            for (int u = 0; u < TS; u++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const int kg = kt[u] * kTileK + j * 32;            // (a group past K repeats the last one: not counted)
-                    norm_frag<XMODE>(a[0][u][j], gamma_lds, min(kg, w.K - 32) + oct * 8, valid[u] && kg < w.K, ssq);
-                }
-        }
 #pragma unroll
         for (int s = 0; s < NS; s++) {
             if (NS > 2) __builtin_amdgcn_sched_barrier(0);
@@ -775,19 +852,34 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
             for (int r = 0; r < 4; r++) red[(((s * MB + b) * nwaves + wv) * 4 + r) * 64 + lane] = acc[s][b][r];
     float* ssq_part = red + NS * MB * nwaves * 4 * 64;      // [wave][row]
     if (NORM) {
-        ssq += __shfl_xor(ssq, 16, 64);
-        ssq += __shfl_xor(ssq, 32, 64);
-        if (lane < 16) ssq_part[wv * 16 + lane] = ssq;
+        // lane l holds pieces of row l / P: sum over each run of P lanes with lane-crossing moves
+        // inside the ALU (pairs, quads, then the mirror images within 8 and within 16 lanes)
+        ssq += lane_cross<0xB1>(ssq);
+        ssq += lane_cross<0x4E>(ssq);
+        if (P >= 8) ssq += lane_cross<0x141>(ssq);
+        if (P >= 16) ssq += lane_cross<0x140>(ssq);
+        if (lane % P == 0) {
+            ssq_part[wv * 16 + lane / P] = ssq;
+            if (wv == 0) {                              // the slots of waves this launch does not have
+#pragma unroll
+                for (int k = 1; k < 8; k++)
+                    if (k >= nwaves) ssq_part[k * 16 + lane / P] = 0.f;
+            }
+        }
     }
     __syncthreads();
     float rstd[4] = {1.f, 1.f, 1.f, 1.f};             // of the rows this lane's outputs belong to
     if (NORM) {
+        // (eight slots whatever the wave count, all reads in flight at once; rows past the batch read
+        // slots nobody wrote and are not stored)
+        float4_t t = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            float t = 0.f;
-            for (int k = 0; k < nwaves; k++) t += ssq_part[k * 16 + 4 * oct + r];
-            rstd[r] = 1.0f / sqrtf(t / (float)w.K + epi.eps);
-        }
+        for (int k = 0; k < 8; k++) t += *reinterpret_cast<const float4_t*>(ssq_part + k * 16 + 4 * oct);
+        // (hardware reciprocal and reciprocal square root, 1 ulp each: the correctly rounded divisions
+        // and root are some 140 instructions here, half a microsecond between the barrier and the stores)
+        const float inv_k = __builtin_amdgcn_rcpf((float)w.K);
+#pragma unroll
+        for (int r = 0; r < 4; r++) rstd[r] = __builtin_amdgcn_rsqf(fmaf(t[r], inv_k, epi.eps));
     }
     // wave v finishes (strip, output register) pairs v, v + waves, ...
     if (NS >= 2 && epi.kind == kEpiSwiglu) {       // strips 2j / 2j+1 of the group are gate / up of output strip (strip0 >> 1) + j
@@ -817,16 +909,16 @@ template <int BITS, int XMODE, int TS, int NS, int XR, int MB = 1>
 hipError_t launch_rows_x(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
                          hipStream_t st)
 {
-    size_t lds = (size_t)NS * MB * nwaves * 4 * 64 * sizeof(float) + (size_t)nwaves * 16 * sizeof(float);
+    size_t lds = (size_t)NS * MB * nwaves * 4 * 64 * sizeof(float) + 8 * 16 * sizeof(float);
     const unsigned groups = (unsigned)((w.NT + NS - 1) / NS);
     if constexpr (MB == 1) {
         if (epi.gamma) {
-            lds += (size_t)w.K * sizeof(float);            // gamma as fp32
+            lds += (size_t)nwaves * TS * kTileK * sizeof(float);            // each wave's tiles of gamma as fp32
             auto kern = gemv_rows_kernel<BITS, XMODE, TS, NS, true, XR>;
             (void)LdsRequest<&gemv_rows_kernel<BITS, XMODE, TS, NS, true, XR>, 150 * 1024>::registered;
-            if (lds > 150 * 1024) return hipErrorInvalidValue;      // (launch_gemv keeps such K away from this kernel)
-            hipLaunchKernelGGL(kern, dim3(groups), dim3(nwaves * 64), lds, st, w.base, reinterpret_cast<const uint16_t*>(x), w.KT, w.K,
-                               w.NT, M, nwaves, y, w.N, ydt, epi);
+            if (lds > 150 * 1024) return hipErrorInvalidValue;
+            hipLaunchKernelGGL(kern, dim3(groups), dim3(nwaves * 64), lds, st, w.base, reinterpret_cast<const uint16_t*>(x), epi.gamma,
+                               w.KT, w.K, w.NT, M, nwaves, epi.gamma_dt, w.N, y, ydt, epi);
             return hipGetLastError();
         }
     }
@@ -834,7 +926,7 @@ hipError_t launch_rows_x(const WeightView& w, const void* x, int M, void* y, int
     if constexpr (NS * MB * 8 * 1024 + 512 > 64 * 1024)
         (void)LdsRequest<&gemv_rows_kernel<BITS, XMODE, TS, NS, false, XR, MB>, 150 * 1024>::registered;
     hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS, false, XR, MB>), dim3(groups), dim3(nwaves * 64), lds, st, w.base,
-                       reinterpret_cast<const uint16_t*>(x), w.KT, w.K, w.NT, M, nwaves, y, w.N, ydt, epi);
+                       reinterpret_cast<const uint16_t*>(x), nullptr, w.KT, w.K, w.NT, M, nwaves, 0, w.N, y, ydt, epi);
     return hipGetLastError();
 }
 
@@ -875,7 +967,7 @@ hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int y
         // overlap the other's stream (128256 rows at 8 rows: 70 -> 54 us)
         if (ns == 4 && (int64_t)w.NT >= (int64_t)8 * num_cus && !epi.gamma)
             return launch_rows_t<BITS, XMODE, 2, 4>(w, x, M, y, ydt, nwaves, epi, st);
-        if (seven && epi.kind == kEpiSwiglu && !epi.gamma) return launch_rows_t<BITS, XMODE, 4, 8>(w, x, M, y, ydt, nwaves, epi, st);
+        if (seven && epi.kind == kEpiSwiglu) return launch_rows_t<BITS, XMODE, 4, 8>(w, x, M, y, ydt, nwaves, epi, st);
         if (seven && epi.kind != kEpiSwiglu) return launch_rows_t<BITS, XMODE, 4, 7>(w, x, M, y, ydt, nwaves, epi, st);
         if (ns == 4) return launch_rows_t<BITS, XMODE, 4, 4>(w, x, M, y, ydt, nwaves, epi, st);
     } else if constexpr (XMODE == XF16) {
@@ -893,8 +985,10 @@ hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int y
         // 112 tiles are 2 slabs of 56, seven tiles per wave)
         auto pad = [&](int ts) { return (w.KT + nwaves * ts - 1) / (nwaves * ts) * (nwaves * ts) - w.KT; };
         if (w.KT > nwaves * 4) {
-            if (pad(8) <= pad(7) && pad(8) <= pad(4)) return launch_rows_t<BITS, XMODE, 8, 1>(w, x, M, y, ydt, nwaves, epi, st);
-            if (pad(7) <= pad(4)) return launch_rows_t<BITS, XMODE, 7, 1>(w, x, M, y, ydt, nwaves, epi, st);
+            // (seven or eight tiles of full-width x loads and a folded norm do not fit the registers)
+            const bool fits = !epi.gamma || M <= 8;
+            if (pad(8) <= pad(7) && pad(8) <= pad(4) && fits) return launch_rows_t<BITS, XMODE, 8, 1>(w, x, M, y, ydt, nwaves, epi, st);
+            if (pad(7) <= pad(4) && fits) return launch_rows_t<BITS, XMODE, 7, 1>(w, x, M, y, ydt, nwaves, epi, st);
         }
     }
     return launch_rows_t<BITS, XMODE, 4, 1>(w, x, M, y, ydt, nwaves, epi, st);
@@ -1044,9 +1138,6 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
     // 27.6 us at 4096 -> 28672)
     const bool wide_q8 = w.bits == 8 && (w.NT + num_cus / 2) / num_cus >= 3;
     const bool rows_kernel = g_tune_rows == 1 || (g_tune_rows == 0 && M >= (wide_q8 ? 5 : 3));
-    // (a folded norm keeps gamma as fp32 in LDS next to the exchange areas: beyond K = 23552 that no
-    // longer fits and the LDS kernel, which stages x in slabs, takes the call)
-    const bool gamma_fits = !epi.gamma || w.K <= 23552;
     if (M > 16) {
         if (!gemv_serves_32(xdt, M, epi)) return hipErrorInvalidValue;
         if (w.bits == 4) {
@@ -1056,7 +1147,7 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
         if (xdt == kF16) return launch_rows2<8, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
         return launch_rows2<8, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
     }
-    if (rows_kernel && xdt != kF32 && gamma_fits) {
+    if (rows_kernel && xdt != kF32) {
         if (w.bits == 4) {
             if (xdt == kF16) return launch_rows<4, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
             return launch_rows<4, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);

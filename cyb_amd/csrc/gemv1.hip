@@ -109,7 +109,7 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
     constexpr int GPA = 16 / MR;                  // scale groups per A operand
     constexpr int TPA = 4 / MR;                   // tiles per A operand
     __shared__ float red[NS * MR * 16 * 16];
-    __shared__ float ssq_red[NORM ? MR * 16 : 1];       // [batch row][wave]
+    __shared__ __attribute__((aligned(16))) float ssq_red[NORM ? MR * 16 : 4];       // [batch row][wave]
     const int out_dt = flags & 15, epi_kind = (flags >> 4) & 15, M = (flags >> 8) & 255, gdt = (flags >> 16) & 15;
     const int tid = threadIdx.x, lane = tid & 63;
     static_assert(!SPLIT || (NS == 2 && NW > 0), "split workgroups are gate / up pairs with a known wave count");
@@ -378,9 +378,16 @@ __global__ __launch_bounds__(1024) void gemv1_kernel(const uint8_t* __restrict__
     if constexpr (NORM) {
 #pragma unroll
         for (int m = 0; m < MR; m++) {
+            // (four vector reads in flight rather than a loop of dependent ones; hardware reciprocal
+            // and reciprocal square root, 1 ulp each)
             float t = 0.f;
-            for (int k = 0; k < nwaves; k++) t += ssq_red[m * 16 + k];
-            const float rstd = 1.0f / sqrtf(t / (float)K + eps);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float4_t v = *reinterpret_cast<const float4_t*>(ssq_red + m * 16 + 4 * q);
+#pragma unroll
+                for (int e = 0; e < 4; e++) t += 4 * q + e < nwaves ? v[e] : 0.f;
+            }
+            const float rstd = __builtin_amdgcn_rsqf(fmaf(t, __builtin_amdgcn_rcpf((float)K), eps));
 #pragma unroll
             for (int st = 0; st < NS; st++) outv[st][m] *= rstd;
         }

@@ -38,6 +38,8 @@ class LinearStack:
     weights: List[QWeight] = field(default_factory=list)
     planar: Dict[str, tuple] = field(default_factory=dict)     # name -> (q bytes, scales) kept for checks
     epilogues: List[str] = field(default_factory=list)         # per node: "none" | "add" | "swiglu" (empty = none anywhere)
+    gammas: List[object] = field(default_factory=list)         # per node: RMSNorm weight folded in front of it, or None (empty = no norms)
+    eps: float = 1e-5
 
     @property
     def weight_bytes(self) -> int:
@@ -59,14 +61,19 @@ def fused_shapes(shapes: Dict[str, tuple] = None) -> Dict[str, tuple]:
             "down_proj": shapes["down_proj"]}
 
 
+NORMED = ("q_proj", "k_proj", "v_proj", "qkv_proj", "gate_proj", "up_proj", "gate_up_proj")      # linears that follow an RMSNorm
+
+
 def build(backend: Backend, layers: int = 32, bits: int = formats.Q4, seed: int = 5, keep_planar=0,
-          shapes: Dict[str, tuple] = None, order: List[str] = None, epilogues: bool = False) -> LinearStack:
+          shapes: Dict[str, tuple] = None, order: List[str] = None, epilogues: bool = False, norms: bool = False) -> LinearStack:
     """Random-init stack with N(0, 0.02) weights quantised on the device.
 
     keep_planar: for the first that many layers (or for the layers listed), the PLANAR device
     buffers are kept in `stack.planar` so that a checker can pull them back and recompute outputs.
     epilogues: with the fused shapes, `gate_up_proj` becomes a strip-interleaved pair run with the
-    SwiGLU epilogue (its output has half the columns) and `o_proj` / `down_proj` add a residual."""
+    SwiGLU epilogue (its output has half the columns) and `o_proj` / `down_proj` add a residual.
+    norms: the linears that follow an RMSNorm in the decode loop (q / k / v, gate / up) get a seeded
+    gamma (f16, 1 +- 0.1) per layer and norm, folded into their activation load."""
     import torch
     shapes = shapes or synth.LLAMA3_8B_LINEARS
     st = LinearStack(backend, layers, bits)
@@ -75,6 +82,7 @@ def build(backend: Backend, layers: int = 32, bits: int = formats.Q4, seed: int 
     order = order or [l for l in LINEAR_ORDER if l in shapes] or list(shapes)
     kept = set(range(keep_planar)) if isinstance(keep_planar, int) else set(keep_planar)
     for layer in range(layers):
+        layer_gamma = {}
         for lin in order:
             K, N = shapes[lin]
             w = torch.empty((N, K), dtype=torch.float32, device="cuda").normal_(0.0, 0.02, generator=gen)
@@ -103,6 +111,11 @@ def build(backend: Backend, layers: int = 32, bits: int = formats.Q4, seed: int 
             st.nodes.append(QMatMul(w=name, x=f"in.{K}", y=f"out.{lin}", quant=bits, M=1, N=N, K=K))
             if epilogues:
                 st.epilogues.append(epi)
+            if norms:
+                which = "input" if lin in ("q_proj", "k_proj", "v_proj", "qkv_proj") else "post_attention"
+                if lin in NORMED and which not in layer_gamma:
+                    layer_gamma[which] = (1.0 + 0.1 * torch.empty(K, dtype=torch.float32, device="cuda").normal_(generator=gen)).to(torch.float16)
+                st.gammas.append(layer_gamma[which] if lin in NORMED else None)
             if layer in kept:
                 st.planar[name] = (qd, sd)
             del w
@@ -130,7 +143,8 @@ def edges_for(stack: LinearStack, M: int, seed: int = 5, shapes: Dict[str, tuple
 
 def plan(stack: LinearStack, edges):
     xs, ys = [edges[n.x] for n in stack.nodes], [edges[n.y] for n in stack.nodes]
+    gammas = stack.gammas or None
     if not stack.epilogues:
-        return stack.backend.plan_many(stack.weights, xs, ys)
+        return stack.backend.plan_many(stack.weights, xs, ys, gammas=gammas, eps=stack.eps)
     res = [edges[f"res.{n.N}"] if e == "add" else None for n, e in zip(stack.nodes, stack.epilogues)]
-    return stack.backend.plan_many(stack.weights, xs, ys, stack.epilogues, res)
+    return stack.backend.plan_many(stack.weights, xs, ys, stack.epilogues, res, gammas=gammas, eps=stack.eps)

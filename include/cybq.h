@@ -227,6 +227,15 @@ int cybq_matmul_many_ex(cybq_ctx* ctx, int64_t count, const cybq_weight* const* 
                         const void* const* residual, cybq_dtype xdt, int64_t M, cybq_dtype ydt,
                         void* stream);
 
+/* cybq_matmul_many_ex with a folded RMSNorm per node: gamma[i] is the node's gamma ([K] of type
+ * gdt) or NULL (no norm in front of that node); all norms share gdt and eps.  One native walk then
+ * covers a whole decode layer as the loop runs it (decide/pipeline.md:51): norm + QKV, O + residual,
+ * norm + gate/up with SwiGLU, down + residual.  gamma, epilogue and residual may each be NULL. */
+int cybq_matmul_many_norm(cybq_ctx* ctx, int64_t count, const cybq_weight* const* w,
+                          const void* const* x, const void* const* gamma, cybq_dtype gdt, float eps,
+                          void* const* y, const int* epilogue, const void* const* residual,
+                          cybq_dtype xdt, int64_t M, cybq_dtype ydt, void* stream);
+
 /* Replaces: nothing the runtime calls per token; it is the verification hook
  * ("dequantised weights match bit-exactly"): out[N,K] f32 = f32(scale) * q. */
 int cybq_dequant(cybq_ctx* ctx, const cybq_weight* w, float* out, void* stream);

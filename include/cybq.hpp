@@ -183,9 +183,12 @@ public:
     {
         if (nodes.empty()) return Status{};
         std::vector<const cybq_weight*> ws;
-        std::vector<const void*> xs, rs;
+        std::vector<const void*> xs, rs, gs;
         std::vector<void*> ys;
         std::vector<int> es;
+        bool normed = false;                  // one gamma type and one eps for the whole list
+        cybq_dtype gdt = CYBQ_F32;
+        float eps = 0.f;
         auto x0i = edges.find(nodes[0].x), y0i = edges.find(nodes[0].y);
         if (x0i == edges.end() || y0i == edges.end()) return fail(CYBQ_ERR_INVALID, "unresolved node '" + nodes[0].w + "'");
         const Edge &x0 = x0i->second, &y0 = y0i->second;
@@ -197,7 +200,19 @@ public:
                 return fail(CYBQ_ERR_INVALID, "run_all needs one M and one dtype pair");
             if (xi->second.rows < n.M || yi->second.rows < n.M) return fail(CYBQ_ERR_SHAPE, "edge has too few rows");
             if (Status s = check_cols(*w, n, xi->second, yi->second); !s) return s;
-            if (!n.norm_gamma.empty()) return fail(CYBQ_ERR_INVALID, "run_all does not take folded norms: use run()");
+            const void* gam = nullptr;
+            if (!n.norm_gamma.empty()) {
+                auto gi = edges.find(n.norm_gamma);
+                if (gi == edges.end()) return fail(CYBQ_ERR_INVALID, "gamma edge of '" + n.w + "' not bound");
+                if (gi->second.rows * gi->second.cols != w->cols()) return fail(CYBQ_ERR_SHAPE, "gamma must hold K elements");
+                if (normed && (gi->second.dtype != gdt || n.norm_eps != eps))
+                    return fail(CYBQ_ERR_INVALID, "run_all needs one gamma type and one eps: use run()");
+                normed = true;
+                gdt = gi->second.dtype;
+                eps = n.norm_eps;
+                gam = gi->second.ptr;
+            }
+            gs.push_back(gam);
             const void* res = nullptr;
             if (n.epilogue == CYBQ_EPI_ADD) {
                 auto ri = edges.find(n.residual);
@@ -210,6 +225,9 @@ public:
             es.push_back((int)n.epilogue);
             rs.push_back(res);
         }
+        if (normed)
+            return wrap(cybq_matmul_many_norm(ctx_, (int64_t)nodes.size(), ws.data(), xs.data(), gs.data(), gdt, eps, ys.data(),
+                                              es.data(), rs.data(), x0.dtype, nodes[0].M, y0.dtype, stream));
         return wrap(cybq_matmul_many_ex(ctx_, (int64_t)nodes.size(), ws.data(), xs.data(), ys.data(), es.data(), rs.data(),
                                         x0.dtype, nodes[0].M, y0.dtype, stream));
     }

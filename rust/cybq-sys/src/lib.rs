@@ -84,6 +84,10 @@ extern "C" {
                                x: *const *const c_void, y: *const *mut c_void, epilogue: *const c_int,
                                residual: *const *const c_void, xdt: c_int, M: i64, ydt: c_int,
                                stream: *mut c_void) -> c_int;
+    pub fn cybq_matmul_many_norm(ctx: *mut cybq_ctx, count: i64, w: *const *const cybq_weight,
+                                 x: *const *const c_void, gamma: *const *const c_void, gdt: c_int, eps: c_float,
+                                 y: *const *mut c_void, epilogue: *const c_int, residual: *const *const c_void,
+                                 xdt: c_int, M: i64, ydt: c_int, stream: *mut c_void) -> c_int;
     pub fn cybq_dequant(ctx: *mut cybq_ctx, w: *const cybq_weight, out: *mut c_float, stream: *mut c_void) -> c_int;
     pub fn cybq_quantize(ctx: *mut cybq_ctx, quant: c_int, src: *const c_float, N: i64, K: i64, q_out: *mut c_void,
                          scales_out: *mut c_void, stream: *mut c_void) -> c_int;

@@ -154,8 +154,19 @@ int main(int argc, char** argv)
                 }
             }
         }
+        // the same node behind a plain one through run_all (one native walk with a gamma per node):
+        // bit for bit what run() wrote
+        {
+            std::vector<float> again((size_t)cnt);
+            if (hipMemset(y3, 0xff, (size_t)cnt * 4) != hipSuccess) { std::printf("ERROR memset\n"); return 1; }
+            s = be.run_all({nodes[0], nn}, edges);
+            if (!s) { std::printf("ERROR %d %s\n", s.code, s.text.c_str()); return 1; }
+            if (hipMemcpy(again.data(), y3, (size_t)cnt * 4, hipMemcpyDeviceToHost) != hipSuccess) { std::printf("ERROR copy\n"); return 1; }
+            if (std::memcmp(again.data(), got.data(), (size_t)cnt * 4) != 0) { std::printf("ERROR run_all with a folded norm differs from run\n"); return 1; }
+        }
         nn.norm_gamma = "no.such.edge";
         if (be.run(nn, edges).code != CYBQ_ERR_INVALID) { std::printf("ERROR missing gamma not reported\n"); return 1; }
+        if (be.run_all({nodes[0], nn}, edges).code != CYBQ_ERR_INVALID) { std::printf("ERROR missing gamma not reported by run_all\n"); return 1; }
 
         s = be.fuse_pairs("fused.gate_up", nodes[0].w, nodes[0].w);
         if (!s) { std::printf("ERROR %d %s\n", s.code, s.text.c_str()); return 1; }

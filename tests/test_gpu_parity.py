@@ -1095,6 +1095,49 @@ def test_decode_stack_with_epilogues(backend, oracle):
         w.free()
 
 
+def test_decode_stack_with_norms(backend, oracle):
+    """A whole layer's linear path in one native walk (cybq_matmul_many_norm): RMSNorm folded in front
+    of qkv and gate/up, SwiGLU and the two residual adds in the epilogues.  Every node of the last
+    layer against the float64 restatement, and against the one-node entry point bit for bit."""
+    from cyb_amd import stack
+    base = {"q_proj": (512, 512), "k_proj": (512, 128), "v_proj": (512, 128), "o_proj": (512, 512),
+            "gate_proj": (512, 1792), "up_proj": (512, 1792), "down_proj": (1792, 512)}
+    shapes = stack.fused_shapes(base)
+    st = stack.build(backend, layers=2, seed=8, keep_planar=2, shapes=shapes, order=list(shapes), epilogues=True, norms=True)
+    assert [g is not None for g in st.gammas] == [True, False, True, False] * 2
+    assert st.gammas[0] is not st.gammas[2] and st.gammas[0] is not st.gammas[4]
+    for M in (1, 2, 8, 40):
+        xdt = "bf16" if M > 16 else "f16"
+        edges = stack.edges_for(st, M, shapes=shapes, xdtype=torch.bfloat16 if M > 16 else None)
+        pl = stack.plan(st, edges)
+        backend.matmul_many(pl, M)
+        torch.cuda.synchronize()
+        bar = TIGHT if M <= 16 else 2 * FAST
+        for i in range(len(st.nodes) - 4, len(st.nodes)):                 # the last layer's outputs are still in place
+            node, epi, gamma = st.nodes[i], st.epilogues[i], st.gammas[i]
+            if gamma is None:
+                ref = _node_reference(oracle, st, node, epi, edges)
+            else:
+                qd, sd = st.planar[node.w]
+                q = formats.unpack_planar(qd.cpu().numpy(), 4, node.N, node.K)
+                s = sd.cpu().numpy().view(np.uint16).reshape(node.N, node.K // 32)
+                ref = _norm_ref(oracle, q, s, edges[node.x], gamma, st.eps, "f16" if M > 16 else xdt)
+                if epi == "swiglu":
+                    ref = _silu_mul(ref[:, :node.N // 2], ref[:, node.N // 2:])
+            got = edges[node.y]
+            assert oracle.rel_l2(got.cpu().numpy(), ref) < bar, (M, node.w, epi)
+            one = torch.empty_like(got)
+            res = edges[f"res.{node.N}"] if epi == "add" else None
+            if gamma is None:
+                backend.matmul_ex(st.weights[i], edges[node.x], one, epi, res)
+            else:
+                backend.matmul_norm(st.weights[i], edges[node.x], gamma, st.eps, one, epi, res)
+            torch.cuda.synchronize()
+            assert torch.equal(one, got), (M, node.w)
+    for w in st.weights:
+        w.free()
+
+
 def _node_reference(oracle, st, node, epi, edges, rows=None):
     """float64 oracle output of one stack node from the PLANAR buffers the stack kept."""
     qd, sd = st.planar[node.w]
