@@ -124,7 +124,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the prefill / sweep / stack extras")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="no timing: a plain 256 MiB device copy (calibration), then the decode and prefill "
-                         "kernels and the 16-row decode kernel on both sweep shapes, for rocprofv3 --pmc runs")
+                         "kernels, the 16-row decode kernel on both sweep shapes and the 8-row one with and without "
+                         "a folded norm, for rocprofv3 --pmc runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the op would shard by rows of W "
@@ -196,6 +197,15 @@ def main():
             yb = torch.empty((16, Nx), dtype=torch.float32, device=dev)
             for i in range(50):
                 be.matmul(wl[i % copies], xb, yb, stream=stream)
+        torch.cuda.synchronize()
+        # the same kernel at 8 rows with and without a folded RMSNorm (f16 gamma) on 4096 -> 14336
+        xb = torch.from_numpy(synth.activations(3, 8, K)).to(dev).to(torch.float16)
+        yb = torch.empty((8, N), dtype=torch.float32, device=dev)
+        gam = torch.from_numpy(1.0 + 0.1 * synth.activations(7, 1, K)[0]).to(dev).to(torch.float16)
+        for i in range(50):
+            be.matmul(ws[i % copies], xb, yb, stream=stream)
+        for i in range(50):
+            be.matmul_norm(ws[i % copies], xb, gam, 1e-5, yb, stream=stream)
         torch.cuda.synchronize()
         log("traffic probe done")
         return
