@@ -859,6 +859,40 @@ def test_folded_rmsnorm_with_swiglu_and_long_k(backend, oracle, M, xdt):
     assert oracle.rel_l2(y.cpu().numpy(), _silu_mul(g, u)) < (2 * FAST if M > 16 else TIGHT)
 
 
+@pytest.mark.parametrize("M,xdt,gdt", [(1, "f16", "f16"), (3, "f16", "f32"), (8, "bf16", "bf16"), (16, "f16", "f16"), (16, "bf16", "f32")])
+def test_folded_rmsnorm_very_long_k(backend, oracle, M, xdt, gdt):
+    # K far past anything a workgroup could keep of gamma in LDS at once
+    N, K = 48, 32768
+    q, s = _quant(oracle, 4, N, K, cfg=47)
+    qw = backend.upload_quantized(q, s, 4)
+    x = _x(M, K, xdt)
+    gamma = (1.0 + 0.25 * torch.from_numpy(synth.activations(54, 1, K)[0])).cuda().to(TDT[gdt])
+    y = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    backend.matmul_norm(qw, x, gamma, 1e-6, y)
+    torch.cuda.synchronize()
+    assert oracle.rel_l2(y.cpu().numpy(), _norm_ref(oracle, q, s, x, gamma, 1e-6, xdt)) < TIGHT
+
+
+@pytest.mark.parametrize("M", [1, 2, 4, 16])
+def test_folded_rmsnorm_counts_subnormal_inputs(backend, oracle, M):
+    # a row of f16 subnormals (|x| < 6.1e-5) with an eps far below its mean square: its squares must
+    # not be flushed on the way into the sum
+    N, K = 64, 1024
+    eps = 1e-14
+    q, s = _quant(oracle, 4, N, K, cfg=48)
+    qw = backend.upload_quantized(q, s, 4)
+    x = _x(M, K, "f16")
+    x[M - 1] = (x[M - 1].float() * 1e-5).to(torch.float16)
+    assert x[M - 1].float().abs().max().item() < 6.1e-5
+    gamma = torch.ones(K, dtype=torch.float16, device="cuda")
+    y = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    backend.matmul_norm(qw, x, gamma, eps, y)
+    torch.cuda.synchronize()
+    ref = _norm_ref(oracle, q, s, x, gamma, eps, "f16")
+    assert oracle.rel_l2(y[M - 1:].cpu().numpy(), ref[M - 1:]) < TIGHT
+    assert oracle.rel_l2(y.cpu().numpy(), ref) < TIGHT
+
+
 def _random_cases(seed, count):
     """Seeded draws over everything a call can vary in: block type, interchange layout, ragged N / K,
     batch rows on both sides of every kernel boundary, the three activation types, output type,
