@@ -500,8 +500,17 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
 // up; here the multiplying waves never wait for HBM.  Waves are dealt to the four SIMDs in turn,
 // so every SIMD carries one staging wave: the dequantisation runs in the issue slots the MFMAs
 // leave free.  MW*MF*16 x NF*16 outputs per workgroup, one barrier per K tile, no K split.
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
 template <int BITS, int NF, int MF, int MW, int XD>
-__global__ __launch_bounds__((MW + 4) * 64) __attribute__((amdgpu_waves_per_eu((MW + 4) / 4, (MW + 4) / 4))) void gemm_roles_kernel(
+__global__ __launch_bounds__((MW + 4) * 64) __attribute__((amdgpu_waves_per_eu((MW + 7) / 4, (MW + 7) / 4))) void gemm_roles_kernel(
     const uint8_t* __restrict__ wbase, const u32x4_t* __restrict__ x, int KT_, int NT_, int x_row_blocks, int M, int n_tiles,
     int m_tiles, int groups, int N_, void* __restrict__ y, int ydt, int K_, float out_scale, Epilogue epi, NormStats ns)
 {
@@ -510,7 +519,9 @@ __global__ __launch_bounds__((MW + 4) * 64) __attribute__((amdgpu_waves_per_eu((
     constexpr int WT = (NF + SW - 1) / SW;            // weight tiles a staging wave handles per K tile
     constexpr int TILE16 = 4 * 64;                    // u32x4 per column block per K tile
     constexpr int BUF16 = NF * TILE16;
-    constexpr int DEPTH = 4;                          // K tiles of packed weights in flight per staging wave
+    // K tiles of packed weights in flight per staging wave (8 measured the same at 64 and 128 rows, 16
+    // slower: 23 -> 30 us at 64 rows)
+    constexpr int DEPTH = 4;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     u32x4_t* ws = reinterpret_cast<u32x4_t*>(smem);   // [2][NF][4][64]
 
@@ -564,13 +575,29 @@ __global__ __launch_bounds__((MW + 4) * 64) __attribute__((amdgpu_waves_per_eu((
             fetch(wreg[R], kt + 1 + DEPTH);
             __syncthreads();
         };
-        for (int kt = 0; kt < KT; kt += DEPTH) {
-            k_tile(kt, std::integral_constant<int, 1>{});
-            if (kt + 1 < KT) k_tile(kt + 1, std::integral_constant<int, 2>{});
-            if (kt + 2 < KT) k_tile(kt + 2, std::integral_constant<int, 3>{});
-            if (kt + 3 < KT) k_tile(kt + 3, std::integral_constant<int, 0>{});
+        // Whole rounds in the loop, the remainder behind it: a tile skipped inside the loop is a path
+        // into the loop head with fewer loads outstanding, the one wait count an instruction carries has
+        // to be safe for that path, and the first use of a tile then also waits for the newest request.
+        // With few rows there is little arithmetic per K tile to hide that behind (4096 -> 14336 at 64
+        // rows 26.1 -> 22.8 us); the 256-row kernel measured better with the tighter counts (60.5 against
+        // 63 us at 512 rows).
+        int kt = 0;
+        if constexpr (MW <= 4) {
+            for (; kt + DEPTH <= KT; kt += DEPTH)
+                static_for<0, DEPTH>([&](auto i) { k_tile(kt + decltype(i)::value, std::integral_constant<int, (decltype(i)::value + 1) % DEPTH>{}); });
+            static_for<0, DEPTH - 1>([&](auto i) {
+                if (kt + decltype(i)::value < KT) k_tile(kt + decltype(i)::value, std::integral_constant<int, (decltype(i)::value + 1) % DEPTH>{});
+            });
+            return;
+        } else {
+            for (; kt < KT; kt += DEPTH) {
+                k_tile(kt, std::integral_constant<int, 1>{});
+                if (kt + 1 < KT) k_tile(kt + 1, std::integral_constant<int, 2>{});
+                if (kt + 2 < KT) k_tile(kt + 2, std::integral_constant<int, 3>{});
+                if (kt + 3 < KT) k_tile(kt + 3, std::integral_constant<int, 0>{});
+            }
+            return;
         }
-        return;
     }
 
     // ---- multiplying waves --------------------------------------------------------------------
@@ -618,7 +645,16 @@ __global__ __launch_bounds__((MW + 4) * 64) __attribute__((amdgpu_waves_per_eu((
         }
         __syncthreads();
     };
-    for (int kt = 0; kt < KT; kt += XD) {
+    int kt = 0;
+    if constexpr (MW <= 4) {                       // (whole rounds in the loop: see the staging waves)
+        for (; kt + XD <= KT; kt += XD) {
+            k_tile(kt, std::integral_constant<int, 0>{});
+            if constexpr (XD > 1) k_tile(kt + 1, std::integral_constant<int, 1>{});
+            if constexpr (XD > 2) k_tile(kt + 2, std::integral_constant<int, 2>{});
+            if constexpr (XD > 3) k_tile(kt + 3, std::integral_constant<int, 3>{});
+        }
+    }
+    for (; kt < KT; kt += XD) {
         k_tile(kt, std::integral_constant<int, 0>{});
         if constexpr (XD > 1) {
             if (kt + 1 < KT) k_tile(kt + 1, std::integral_constant<int, 1>{});
@@ -794,8 +830,12 @@ hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt
             const int64_t tiles64 = (w.NT + 3) / 4;                  // 64-column tiles
             if (tiles64 * 2 >= 3 * num_cus)          // more than one round of them: the plain kernel (48 against 58 us at N = 28672)
                 return launch_m<BITS, 0, 4, false, 2, 4>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
-            if (tiles64 * 4 >= 3 * num_cus)          // one round: the role-split kernel (30 against 34.5 us at N = 14336)
+            if (tiles64 * 4 >= 3 * num_cus) {        // one round: the role-split kernel (30 against 34.5 us at N = 14336)
+                // (every workgroup streams all the rows of X from the L2, and that stream is what these
+                // calls wait for: two multiplying waves = 64 rows when that covers the batch)
+                if (M <= 64) return launch_roles<BITS, 4, 2, 2, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
                 return launch_roles<BITS, 4, 2, 4, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
+            }
         }
         if (nf7) return launch_t<BITS, 0, 7, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
         return launch_t<BITS, 0, 8, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
