@@ -403,6 +403,19 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
     hipError_t e;
     if (M <= 16 || (M <= 32 && cybq::gemv_serves_32((int)xdt, (int)M, epi))) {
         e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->decode_exact, epi, st);
+    } else if (M <= 64 && (int64_t)w->N * w->K <= (int64_t)6144 * 4096 && cybq::gemv_serves_32((int)xdt, 32, epi)) {
+        // 33..64 rows on a small weight (up to 4096 -> 6144): the MFMA kernel would split K over
+        // workgroups and add the slabs in a second pass; two passes of the batched-rows decode kernel
+        // (32 rows, then the rest) are quicker although they stream the weights twice
+        // (4096 -> 4096 at 64 rows 21.8 -> 14.8 us, 4096 -> 1024 17.8 -> 12.6 us) - and exact
+        const int64_t n_out = epi.kind == cybq::kEpiSwiglu ? w->N / 2 : w->N;
+        const size_t yoff = (size_t)32 * n_out * dtype_size(ydt);
+        cybq::Epilogue ec = epi;
+        if (epi.kind == cybq::kEpiAdd) ec.residual = static_cast<const char*>(residual) + yoff;
+        e = cybq::launch_gemv(v, x, xdt, 32, y, ydt, ctx->num_cus, ctx->decode_exact, epi, st);
+        if (e == hipSuccess)
+            e = cybq::launch_gemv(v, static_cast<const char*>(x) + (size_t)32 * w->K * dtype_size(xdt), xdt, (int)M - 32,
+                                  static_cast<char*>(y) + yoff, ydt, ctx->num_cus, ctx->decode_exact, ec, st);
     } else if (!w->wide_scales && (xdt == CYBQ_F32 ? !ctx->prefill_exact : M > 32)) {
         e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, workspace, workspace_bytes,
                               epi, st);

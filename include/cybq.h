@@ -142,7 +142,8 @@ int cybq_weight_info(const cybq_weight* w, int* quant, int64_t* N, int64_t* K,
  *   y  [M,N] row-major, ydt in {F32,F16,BF16} (fp32 accumulator rounded once)
  *   M >= 1.  M <= 32 runs the HBM-streaming decode kernels (17..32 rows of 16-bit
  *   activations: one pass with two row blocks; with a folded norm two passes of 16
- *   rows), larger M the LDS-tiled MFMA prefill kernel (fp32
+ *   rows; 33..64 rows of 16-bit activations on a weight of up to 6144 x 4096
+ *   elements: two passes, 32 rows and the rest), larger M the LDS-tiled MFMA prefill kernel (fp32
  *   activations in CYBQ_PREFILL_EXACT mode: the decode kernel, 16 rows at a
  *   time; in FAST mode they are rounded once to f16 on the way in and take
  *   the prefill kernel from 17 rows on); there is no other path. */

@@ -143,12 +143,14 @@ int main(int argc, char** argv)
             for (int64_t k = 0; k < K0; k++) { const double v = h2f(xh[m * K0 + k]); ss += v * v; }
             const double rstd = 1.0 / std::sqrt(ss / (double)K0 + 1e-5);
             // (the plain and the folded call may run different kernels: both sum in fp32, in
-            // different orders, so elements are compared against the size of the row)
+            // different orders, so elements are compared against the size of the row; past 32 rows
+            // in FAST mode one of them may be the MFMA kernel with weights rounded to f16 while the
+            // other is a decode kernel)
             double row_max = 0;
             for (int64_t n = 0; n < N0; n++) row_max = std::max(row_max, std::fabs(plain[m * N0 + n] * rstd));
             for (int64_t n = 0; n < N0; n++) {
                 const double want_v = plain[m * N0 + n] * rstd;
-                if (std::fabs(got[m * N0 + n] - want_v) > 2e-6 * row_max + 1e-9) {
+                if (std::fabs(got[m * N0 + n] - want_v) > ((!exact && M > 32) ? 3e-3 : 2e-6) * row_max + 1e-9) {
                     std::printf("ERROR folded norm differs at %lld,%lld: %g vs %g\n", (long long)m, (long long)n, got[m * N0 + n], want_v);
                     return 1;
                 }
