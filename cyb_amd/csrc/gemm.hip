@@ -837,6 +837,38 @@ hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt
                 return launch_roles<BITS, 4, 2, 4, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
             }
         }
+        // A narrow output with a short K (the attention projections at a prefill chunk): 256 x 112 tiles
+        // would leave most CUs idle and get a K split with its second pass over the partial sums.
+        // One round of 128-row tiles of the role-split kernel, as wide as still gives every CU a tile,
+        // does without (X then crosses from the L2 once per column tile: K stays short for this).
+        if (epi.kind != kEpiSwiglu && w.KT <= 48 && M > 128) {
+            const int64_t tiles256 = (int64_t)((w.NT + 6) / 7) * ((M + 255) / 256);
+            if (tiles256 < num_cus) {
+                // (128-row tiles first, 64-row ones for batches they cannot spread over the chip; the
+                // width that fills most of one round, at least three quarters of it)
+                int best_nf = 0, best_mw = 0;
+                int64_t best_groups = 0;
+                for (int mw : {4, 2})
+                    for (int nf : {8, 6, 4}) {
+                        const int64_t g = (int64_t)((M + mw * 32 - 1) / (mw * 32)) * ((w.NT + nf - 1) / nf);
+                        if (g <= num_cus && g * 4 >= 3 * num_cus && (best_mw == 0 || (mw == best_mw && g > best_groups))) {
+                            best_nf = nf;
+                            best_mw = mw;
+                            best_groups = g;
+                        }
+                    }
+                if (best_mw == 4) {
+                    if (best_nf == 8) return launch_roles<BITS, 8, 2, 4, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
+                    if (best_nf == 6) return launch_roles<BITS, 6, 2, 4, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
+                    return launch_roles<BITS, 4, 2, 4, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
+                }
+                if (best_mw == 2) {
+                    if (best_nf == 8) return launch_roles<BITS, 8, 2, 2, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
+                    if (best_nf == 6) return launch_roles<BITS, 6, 2, 2, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
+                    return launch_roles<BITS, 4, 2, 2, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
+                }
+            }
+        }
         if (nf7) return launch_t<BITS, 0, 7, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
         return launch_t<BITS, 0, 8, false>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
     }

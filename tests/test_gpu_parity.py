@@ -637,14 +637,19 @@ def test_prefill_512_row_workgroups(backend, oracle, bits, xdt):
 
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("shape", [(14336, 384, 512), (4096, 384, 2048), (6144, 160, 1100), (14336, 384, 100), (28672, 160, 128),
-                                   (14344, 160, 520), (14342, 96, 515)])
+                                   (14344, 160, 520), (14342, 96, 515),
+                                   (4096, 416, 512), (6144, 160, 500), (8000, 96, 512), (4096, 160, 200), (6150, 96, 250),
+                                   (8000, 96, 230), (8704, 96, 192), (3840, 96, 320), (4096, 160, 64), (14336, 288, 50)])
 def test_prefill_role_split_kernel(backend, oracle, bits, shape):
     """FAST mode with enough 256-row tiles to fill the chip: some waves of a workgroup only multiply,
     the others only fetch and dequantise weights.  Seven and eight column blocks per tile, a ragged
     last row tile, every activation and output type, residual add and folded RMSNorm.  The last two
     shapes: up to 128 rows on a wide output run 128 x 64 tiles without a K split (role-split for one
     round of tiles, the plain kernel for more); then N that ends inside a column block, with rows of y
-    that are 16-byte aligned and rows that are not (element-wise stores)."""
+    that are 16-byte aligned and rows that are not (element-wise stores).  From (4096, 416, 512) on:
+    narrow outputs with a short K in one round of 128-row or 64-row tiles that are 4, 6 and 8 column
+    blocks wide (K of 3.25 and 2.25 tiles: a remainder behind the whole rounds of the K loops), then
+    two decode passes over 64 rows of a small weight and the 64-row tiles of a wide output."""
     N, K, M = shape
     q, s = _quant(oracle, bits, N, K, cfg=45)
     qw = backend.upload_quantized(q, s, bits)
