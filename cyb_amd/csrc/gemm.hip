@@ -828,9 +828,12 @@ hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt
         // its second pass over the partial sums
         if (M <= 128 && epi.kind != kEpiSwiglu) {
             const int64_t tiles64 = (w.NT + 3) / 4;                  // 64-column tiles
-            if (tiles64 * 2 >= 3 * num_cus)          // more than one round of them: the plain kernel (48 against 58 us at N = 28672)
+            if (tiles64 * 2 >= 3 * num_cus) {        // more than one round of them: the plain kernel (48 against 58 us at N = 28672),
+                // up to 64 rows the role-split one with its smaller workgroups (41.5 -> 39.5 us)
+                if (M <= 64) return launch_roles<BITS, 4, 2, 2, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
                 return launch_m<BITS, 0, 4, false, 2, 4>(w, x, M, y, ydt, out_scale, part, part_bytes, num_cus, epi, ns, st);
-            if (tiles64 * 4 >= 3 * num_cus) {        // one round: the role-split kernel (30 against 34.5 us at N = 14336)
+            }
+            if (tiles64 * 4 >= 3 * num_cus || (tiles64 * 2 >= num_cus && w.KT <= 48)) {      // (half a round still beats a K split on a short K)        // one round: the role-split kernel (30 against 34.5 us at N = 14336)
                 // (every workgroup streams all the rows of X from the L2, and that stream is what these
                 // calls wait for: two multiplying waves = 64 rows when that covers the batch)
                 if (M <= 64) return launch_roles<BITS, 4, 2, 2, 2>(w, x, M, y, ydt, out_scale, epi, ns, st);
