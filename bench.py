@@ -359,6 +359,22 @@ def main():
         log(f"prefill GEMM M=512: {elp * 1e6:.1f} us, {tfl:.1f} TFLOP/s, rel_l2 {relp:.2e}; dense bf16 {dense_us:.1f} us; "
             f"MFMA loop {mfma_tfl:.0f} TFLOP/s")
 
+        # ---- the same call at other row counts (bf16 activations, weights rotating through HBM)
+        rows_out = {}
+        for Mr in (64, 128, 256, 1024, 2048):
+            xr = torch.from_numpy(synth.activations(4, Mr, K)).to(dev).to(torch.bfloat16)
+            yr = torch.empty((Mr, N), dtype=torch.float32, device=dev)
+            nr = 50 if Mr <= 256 else 12
+            rpl = be.plan_many([ws[j % copies] for j in range(nr)], [xr] * nr, [yr] * nr)
+            be.matmul_many(rpl, Mr, stream)
+            tr, _ = timer.until(lambda i: be.matmul_many(rpl, Mr, stream), max_passes=40)
+            tr /= nr
+            rows_out[f"M{Mr}"] = {"us": round(tr * 1e6, 1), "tflops": round(2.0 * Mr * N * K / tr / 1e12, 1),
+                                  "frac_of_mfma_peak": round(2.0 * Mr * N * K / tr / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+            del xr, yr, rpl
+        extra["prefill_rows_sweep_4096x14336"] = rows_out
+        log("prefill rows sweep: " + " ".join(f"{k}:{v['us']}us" for k, v in rows_out.items()))
+
         # ---- batch sweep of the decode kernels on the same shape
         def sweep_shape(wl, Kx, Nx, Ms, bitsx=bits):
             out = {}
