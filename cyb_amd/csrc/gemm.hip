@@ -642,6 +642,9 @@ __global__ __launch_bounds__((MW + 4) * 64) __attribute__((amdgpu_waves_per_eu((
         for (int i = 0; i < READS; i++) {
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, MF, 0);
+            // (a group's X operands are requested again as soon as its last MFMA is out: left to itself
+            // the scheduler moves all of a tile's requests to its end, one K tile less of lead)
+            if (i % NF == NF - 1) __builtin_amdgcn_sched_group_barrier(0x020, MF, 0);
         }
         __syncthreads();
     };
