@@ -1179,6 +1179,65 @@ def test_decode_stack_with_norms(backend, oracle):
         w.free()
 
 
+def test_many_norm_without_gammas_is_many_ex_and_rejects_bad_arguments(backend, oracle):
+    """cybq_matmul_many_norm with no gamma anywhere is cybq_matmul_many_ex bit for bit; a node whose gamma is
+    NULL runs without a norm; errors come back as values."""
+    N, K, M = 96, 512, 5
+    q, s = _quant(oracle, 4, N, K, cfg=95)
+    w = backend.upload_quantized(q, s, 4)
+    x = _x(M, K, "f16", cfg=96)
+    gamma = (1.0 + 0.25 * torch.from_numpy(synth.activations(97, 1, K)[0])).cuda().to(torch.float16)
+    y_plain = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    y_norm = torch.empty_like(y_plain)
+    backend.matmul(w, x, y_plain)
+    backend.matmul_norm(w, x, gamma, 1e-5, y_norm)
+    ya, yb = torch.zeros_like(y_plain), torch.zeros_like(y_plain)
+    backend.matmul_many(backend.plan_many([w, w], [x, x], [ya, yb], gammas=[None, gamma], eps=1e-5), M)
+    torch.cuda.synchronize()
+    assert torch.equal(ya, y_plain) and torch.equal(yb, y_norm)
+    lib, ctx = backend._lib, backend._ctx
+    import ctypes
+    arr = lambda vals: (ctypes.c_void_p * len(vals))(*vals)
+    ws, xs, ys = arr([w.handle]), arr([x.data_ptr()]), arr([ya.data_ptr()])
+    ya.zero_()
+    rc = lib.cybq_matmul_many_norm(ctx, 1, ws, xs, None, 1, ctypes.c_float(1e-5), ys, None, None, 1, M, 0, None)
+    torch.cuda.synchronize()
+    assert rc == 0 and torch.equal(ya, y_plain)                         # no gamma array at all
+    gs = arr([gamma.data_ptr()])
+    assert lib.cybq_matmul_many_norm(ctx, 1, ws, xs, gs, 77, ctypes.c_float(1e-5), ys, None, None, 1, M, 0, None) != 0     # unknown gamma type
+    assert lib.cybq_matmul_many_norm(ctx, 1, ws, xs, gs, 1, ctypes.c_float(-1.0), ys, None, None, 1, M, 0, None) != 0    # negative eps
+    assert lib.cybq_matmul_many_norm(ctx, 1, None, xs, gs, 1, ctypes.c_float(1e-5), ys, None, None, 1, M, 0, None) != 0   # no weights
+    assert lib.cybq_matmul_many_norm(ctx, 0, ws, xs, gs, 1, ctypes.c_float(1e-5), ys, None, None, 1, M, 0, None) == 0     # nothing to do
+
+
+@pytest.mark.parametrize("M", [33, 40, 64])
+@pytest.mark.parametrize("xdt", ["f16", "bf16"])
+def test_rows_33_to_64_on_a_small_weight_are_two_decode_passes(backend, oracle, M, xdt):
+    """33..64 rows of 16-bit activations on a small weight: rows 0..31 carry the bits of a 32-row call,
+    the rest those of a call with the remaining rows (a row's bits do not depend on the batch it is in),
+    in both prefill modes, and the float64 result within the decode kernels' bar."""
+    N, K = 272, 1184
+    q, s = _quant(oracle, 4, N, K, cfg=98)
+    w = backend.upload_quantized(q, s, 4)
+    x = _x(M, K, xdt, cfg=99)
+    r = torch.from_numpy(synth.activations(100, M, N)).cuda()
+    for mode in ("fast", "exact"):
+        backend.set_prefill_mode(mode)
+        try:
+            y = torch.empty((M, N), dtype=torch.float32, device="cuda")
+            backend.matmul_ex(w, x, y, "add", r)
+            y_a = torch.empty((32, N), dtype=torch.float32, device="cuda")
+            y_b = torch.empty((M - 32, N), dtype=torch.float32, device="cuda")
+            backend.matmul_ex(w, x[:32].contiguous(), y_a, "add", r[:32].contiguous())
+            backend.matmul_ex(w, x[32:].contiguous(), y_b, "add", r[32:].contiguous())
+            torch.cuda.synchronize()
+            assert torch.equal(y[:32], y_a) and torch.equal(y[32:], y_b)
+            ref = oracle.matmul_f64(q, s, x.float().cpu().numpy()) + r.double().cpu().numpy()
+            assert oracle.rel_l2(y.cpu().numpy(), ref) < TIGHT
+        finally:
+            backend.set_prefill_mode("fast")
+
+
 def _node_reference(oracle, st, node, epi, edges, rows=None):
     """float64 oracle output of one stack node from the PLANAR buffers the stack kept."""
     qd, sd = st.planar[node.w]
