@@ -250,8 +250,11 @@ def main():
             c = (c + n) % copies
 
     # everything still cached from the set-up (clones, parity) is pushed out first
+    # (and repeated for some 20 ms: a device that has idled through the set-up runs its first
+    # milliseconds of load below its clocks)
     flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
-    flush.fill_(1)
+    for i in range(64):
+        flush.fill_(i & 1)
     torch.cuda.synchronize()
     del flush
     # (every plan is built before the warm-up: the timed passes follow it without the device idling
