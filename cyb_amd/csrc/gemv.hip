@@ -730,12 +730,26 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
         // its arithmetic.  So the strips are walked two requests ahead: strip s+2 is
         // requested, then strip s (whose tiles were requested two steps ago) is
         // multiplied while the others are on their way.
+        // bf16 activations with two to four strips: the weights enter the bf16 MFMA as 128 + u (256 + u for
+        // Q8) and one more MFMA of the activations against a constant operand takes the bias off.  That
+        // second product does not depend on the strip, so the tiles are walked K tile by K tile with all
+        // strips of a tile behind one bias product (its result is the C operand of their MFMAs):
+        // 4 + 4 NS instead of 8 NS MFMAs per tile.  Each strip still sums its tiles in the same order.
+        constexpr bool BY_TILE = XMODE == XBF16 && BITS == 4 && NS >= 2 && NS <= 4 && (TS == 4 || MB == 2);       // (the others would spill)
+        constexpr int WU = NS == 4 ? (TS < 2 ? TS : 2) : TS;       // BY_TILE: K tiles requested ahead (about eight weight tiles)
         TileRegs<BITS> buf[NS][TS];
         constexpr int AHEAD = NS < 2 ? NS : 2;
+        if constexpr (BY_TILE) {
 #pragma unroll
-        for (int s = 0; s < AHEAD; s++)
+            for (int u = 0; u < WU; u++)
 #pragma unroll
-            for (int u = 0; u < TS; u++) load_tile<BITS>(buf[s][u], w, sbase[s] + kt[u], lane);
+                for (int s = 0; s < NS; s++) load_tile<BITS>(buf[s][u], w, sbase[s] + kt[u], lane);
+        } else {
+#pragma unroll
+            for (int s = 0; s < AHEAD; s++)
+#pragma unroll
+                for (int u = 0; u < TS; u++) load_tile<BITS>(buf[s][u], w, sbase[s] + kt[u], lane);
+        }
         if (NORM) {
             // my tiles' gamma -> my LDS area (16 or 32 lanes hold a tile's 128 values; fp32, or as loaded
             // when x and gamma are both f16), read back below piece by piece: no other wave is involved
@@ -804,8 +818,43 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
                         a[b][u][j].u[p] =
                             (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane + (j % GPL) * 16, (int)raw[j / GPL][p]);
             }
+        if constexpr (BY_TILE) {
+            const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+            Frag16 off;
+            const uint32_t offw = BITS == 4 ? kBf16Neg136x2 : kBf16Neg128x2;
+            off.u = (u32x4_t){offw, offw, offw, offw};
 #pragma unroll
-        for (int s = 0; s < NS; s++) {
+            for (int u = 0; u < TS; u++) {
+                if (NS > 2) __builtin_amdgcn_sched_barrier(0);
+                if (u + WU < TS) {
+#pragma unroll
+                    for (int s = 0; s < NS; s++) load_tile<BITS>(buf[s][u + WU], w, sbase[s] + kt[u + WU], lane);
+                }
+                if (NS > 2) __builtin_amdgcn_sched_barrier(0);
+                float4_t bias[MB][4];
+#pragma unroll
+                for (int b = 0; b < MB; b++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) bias[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[b][u][j].b, off.b, zero, 0, 0, 0);
+#pragma unroll
+                for (int s = 0; s < NS; s++) {
+                    Frag16 bop[4];
+                    tile_operands<BITS, XMODE>(buf[s][u], magic, bop);
+                    u32x2_t sc = buf[s][u].s;
+                    sc[0] = valid[u] ? sc[0] : 0u;
+                    sc[1] = valid[u] ? sc[1] : 0u;
+#pragma unroll
+                    for (int b = 0; b < MB; b++) {
+                        float4_t d[4];
+#pragma unroll
+                        for (int j = 0; j < 4; j++) d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[b][u][j].b, bop[j].b, bias[b][j], 0, 0, 0);
+                        tile_accum<4>(sc, d, acc[s][b]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < (BY_TILE ? 0 : NS); s++) {
             if (NS > 2) __builtin_amdgcn_sched_barrier(0);
             if (s + AHEAD < NS) {
 #pragma unroll
