@@ -648,7 +648,11 @@ __device__ __forceinline__ void norm_piece(u32x4_t& v, const GammaPiece& gp, boo
 // two activation operands, the weights still stream once).
 // gamma / gamma_dt (NORM) sit ahead of y in the argument list: everything the first loads need is
 // then in the argument registers the hardware fills before the kernel starts.
-template <int BITS, int XMODE, int TS, int NS, bool NORM, int XR, int MB = 1>
+// SUB (f16 activations, Q4, decode mode STREAM): the weights enter the MFMA as the f16 subnormals
+// 4u * 2^-24 / 64u * 2^-24 (six vector instructions per eight weights instead of nine), the bias comes off
+// through the MFMA's C operand like with bf16 activations, 1/16 for the odd groups rides on their scale
+// and 2^22 on the final sums.
+template <int BITS, int XMODE, int TS, int NS, bool NORM, int XR, int MB = 1, bool SUB = false>
 // (waves_per_eu: the scheduler would otherwise trade the up-front loads for occupancy)
 __global__ __launch_bounds__((TS <= 2 && MB == 1 && !NORM) ? 1024 : 512)
 __attribute__((amdgpu_waves_per_eu(2, (TS <= 2 && MB == 1 && !NORM) ? 4 : 2)))
@@ -735,7 +739,8 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
         // second product does not depend on the strip, so the tiles are walked K tile by K tile with all
         // strips of a tile behind one bias product (its result is the C operand of their MFMAs):
         // 4 + 4 NS instead of 8 NS MFMAs per tile.  Each strip still sums its tiles in the same order.
-        constexpr bool BY_TILE = XMODE == XBF16 && BITS == 4 && NS >= 2 && NS <= 4 && (TS == 4 || MB == 2);       // (the others would spill)
+        constexpr bool BY_TILE = (XMODE == XBF16 || SUB) && BITS == 4 && NS >= 2 && NS <= 4 && (TS == 4 || MB == 2);       // (the others would spill)
+        static_assert(!SUB || (BY_TILE && XMODE == XF16 && !NORM), "subnormal operands: f16 activations, walked by tile");
         constexpr int WU = NS == 4 ? (TS < 2 ? TS : 2) : TS;       // BY_TILE: K tiles requested ahead (about eight weight tiles)
         TileRegs<BITS> buf[NS][TS];
         constexpr int AHEAD = NS < 2 ? NS : 2;
@@ -820,9 +825,11 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
             }
         if constexpr (BY_TILE) {
             const float4_t zero = {0.f, 0.f, 0.f, 0.f};
-            Frag16 off;
-            const uint32_t offw = BITS == 4 ? kBf16Neg136x2 : kBf16Neg128x2;
+            Frag16 off, off_odd;            // the constant operand(s) that take the bias off
+            const uint32_t offw = SUB ? kSubBiasL : (BITS == 4 ? kBf16Neg136x2 : kBf16Neg128x2);
+            const uint32_t offw_odd = SUB ? kSubBiasH : offw;
             off.u = (u32x4_t){offw, offw, offw, offw};
+            off_odd.u = (u32x4_t){offw_odd, offw_odd, offw_odd, offw_odd};
 #pragma unroll
             for (int u = 0; u < TS; u++) {
                 if (NS > 2) __builtin_amdgcn_sched_barrier(0);
@@ -835,11 +842,22 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
 #pragma unroll
                 for (int b = 0; b < MB; b++)
 #pragma unroll
-                    for (int j = 0; j < 4; j++) bias[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[b][u][j].b, off.b, zero, 0, 0, 0);
+                    for (int j = 0; j < 4; j++) {
+                        if constexpr (SUB)
+                            bias[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[b][u][j].h, ((j & 1) ? off_odd : off).h, zero, 0, 0, 0);
+                        else bias[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[b][u][j].b, off.b, zero, 0, 0, 0);
+                    }
 #pragma unroll
                 for (int s = 0; s < NS; s++) {
                     Frag16 bop[4];
-                    tile_operands<BITS, XMODE>(buf[s][u], magic, bop);
+                    if constexpr (SUB) {
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            uint32_t bw[4];
+                            unpack_q4_sub(buf[s][u].q[0][2 * (j >> 1)], buf[s][u].q[0][2 * (j >> 1) + 1], j & 1, bw);
+                            bop[j].u = (u32x4_t){bw[0], bw[1], bw[2], bw[3]};
+                        }
+                    } else tile_operands<BITS, XMODE>(buf[s][u], magic, bop);
                     u32x2_t sc = buf[s][u].s;
                     sc[0] = valid[u] ? sc[0] : 0u;
                     sc[1] = valid[u] ? sc[1] : 0u;
@@ -847,8 +865,19 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
                     for (int b = 0; b < MB; b++) {
                         float4_t d[4];
 #pragma unroll
-                        for (int j = 0; j < 4; j++) d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[b][u][j].b, bop[j].b, bias[b][j], 0, 0, 0);
-                        tile_accum<4>(sc, d, acc[s][b]);
+                        for (int j = 0; j < 4; j++) {
+                            if constexpr (SUB) d[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[b][u][j].h, bop[j].h, bias[b][j], 0, 0, 0);
+                            else d[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[b][u][j].b, bop[j].b, bias[b][j], 0, 0, 0);
+                        }
+                        if constexpr (SUB) {
+#pragma unroll
+                            for (int j = 0; j < 4; j++) {
+                                const uint32_t sb = (j & 1) ? (sc[j >> 1] >> 16) : (sc[j >> 1] & 0xffffu);
+                                const float sf = (j & 1) ? f16_bits_to_f32(sb) * 0.0625f : f16_bits_to_f32(sb);
+#pragma unroll
+                                for (int r = 0; r < 4; r++) acc[s][b][r] = __builtin_fmaf(sf, d[j][r], acc[s][b][r]);
+                            }
+                        } else tile_accum<4>(sc, d, acc[s][b]);
                     }
                 }
             }
@@ -917,7 +946,8 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
         }
     }
     __syncthreads();
-    float rstd[4] = {1.f, 1.f, 1.f, 1.f};             // of the rows this lane's outputs belong to
+    constexpr float kOut = SUB ? kSubUnscale : 1.f;
+    float rstd[4] = {kOut, kOut, kOut, kOut};         // of the rows this lane's outputs belong to (SUB: 2^22 of the operands)
     if (NORM) {
         // (eight slots whatever the wave count, all reads in flight at once; rows past the batch read
         // slots nobody wrote and are not stored)
@@ -956,7 +986,7 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
 
 template <int BITS, int XMODE, int TS, int NS, int XR, int MB = 1>
 hipError_t launch_rows_x(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
-                         hipStream_t st)
+                         bool sub, hipStream_t st)
 {
     size_t lds = (size_t)NS * MB * nwaves * 4 * 64 * sizeof(float) + 8 * 16 * sizeof(float);
     const unsigned groups = (unsigned)((w.NT + NS - 1) / NS);
@@ -971,6 +1001,18 @@ hipError_t launch_rows_x(const WeightView& w, const void* x, int M, void* y, int
             return hipGetLastError();
         }
     }
+    // decode mode STREAM, Q4 and f16 activations, two to four strips: subnormal operands
+    // (with two row blocks, 17..32 rows, it measures 0.3 us slower than the integer operands, but a row keeps
+    // the bits it has in a batch of up to 16)
+    if constexpr (BITS == 4 && XMODE == XF16 && NS >= 2 && NS <= 4 && (TS == 4 || MB == 2)) {
+        if (sub && !epi.gamma) {
+            if constexpr (NS * MB * 8 * 1024 + 512 > 64 * 1024)
+                (void)LdsRequest<&gemv_rows_kernel<BITS, XMODE, TS, NS, false, XR, MB, true>, 150 * 1024>::registered;
+            hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS, false, XR, MB, true>), dim3(groups), dim3(nwaves * 64), lds, st,
+                               w.base, reinterpret_cast<const uint16_t*>(x), nullptr, w.KT, w.K, w.NT, M, nwaves, 0, w.N, y, ydt, epi);
+            return hipGetLastError();
+        }
+    }
     // (the exchange area alone passes 64 KB with eight strips, or four strips and two row blocks)
     if constexpr (NS * MB * 8 * 1024 + 512 > 64 * 1024)
         (void)LdsRequest<&gemv_rows_kernel<BITS, XMODE, TS, NS, false, XR, MB>, 150 * 1024>::registered;
@@ -982,11 +1024,11 @@ hipError_t launch_rows_x(const WeightView& w, const void* x, int M, void* y, int
 // (the x load pattern follows the batch: up to 4, up to 8, up to 16 rows per load)
 template <int BITS, int XMODE, int TS, int NS>
 hipError_t launch_rows_t(const WeightView& w, const void* x, int M, void* y, int ydt, int nwaves, const Epilogue& epi,
-                         hipStream_t st)
+                         bool sub, hipStream_t st)
 {
-    if (M <= 4) return launch_rows_x<BITS, XMODE, TS, NS, 4>(w, x, M, y, ydt, nwaves, epi, st);
-    if (M <= 8) return launch_rows_x<BITS, XMODE, TS, NS, 8>(w, x, M, y, ydt, nwaves, epi, st);
-    return launch_rows_x<BITS, XMODE, TS, NS, 16>(w, x, M, y, ydt, nwaves, epi, st);
+    if (M <= 4) return launch_rows_x<BITS, XMODE, TS, NS, 4>(w, x, M, y, ydt, nwaves, epi, sub, st);
+    if (M <= 8) return launch_rows_x<BITS, XMODE, TS, NS, 8>(w, x, M, y, ydt, nwaves, epi, sub, st);
+    return launch_rows_x<BITS, XMODE, TS, NS, 16>(w, x, M, y, ydt, nwaves, epi, sub, st);
 }
 
 // strips per workgroup: as many as keeps about one workgroup per CU, at most 4
@@ -1000,7 +1042,7 @@ int strips_per_group(const WeightView& w, int num_cus, const Epilogue& epi)
 
 template <int BITS, int XMODE>
 hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int ydt, int tuned_waves, int num_cus,
-                       const Epilogue& epi, hipStream_t st)
+                       const Epilogue& epi, bool sub, hipStream_t st)
 {
     // 8 waves split K (fewer when the strip has fewer tiles), 4 tiles of x per wave and slab
     const int ns = strips_per_group(w, num_cus, epi);
@@ -1015,18 +1057,18 @@ hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int y
         // instead of four halve the registers, two workgroups share a CU and one's ramp and tail
         // overlap the other's stream (128256 rows at 8 rows: 70 -> 54 us)
         if (ns == 4 && (int64_t)w.NT >= (int64_t)8 * num_cus && !epi.gamma)
-            return launch_rows_t<BITS, XMODE, 2, 4>(w, x, M, y, ydt, nwaves, epi, st);
-        if (seven && epi.kind == kEpiSwiglu) return launch_rows_t<BITS, XMODE, 4, 8>(w, x, M, y, ydt, nwaves, epi, st);
-        if (seven && epi.kind != kEpiSwiglu) return launch_rows_t<BITS, XMODE, 4, 7>(w, x, M, y, ydt, nwaves, epi, st);
-        if (ns == 4) return launch_rows_t<BITS, XMODE, 4, 4>(w, x, M, y, ydt, nwaves, epi, st);
+            return launch_rows_t<BITS, XMODE, 2, 4>(w, x, M, y, ydt, nwaves, epi, sub, st);
+        if (seven && epi.kind == kEpiSwiglu) return launch_rows_t<BITS, XMODE, 4, 8>(w, x, M, y, ydt, nwaves, epi, sub, st);
+        if (seven && epi.kind != kEpiSwiglu) return launch_rows_t<BITS, XMODE, 4, 7>(w, x, M, y, ydt, nwaves, epi, sub, st);
+        if (ns == 4) return launch_rows_t<BITS, XMODE, 4, 4>(w, x, M, y, ydt, nwaves, epi, sub, st);
     } else if constexpr (XMODE == XF16) {
         // Q8 tiles are twice the registers: four strips x four tiles of f16 operands would spill.  Two
         // strips x two tiles (80 registers, six waves per SIMD) stream best there; bf16 operands fit
-        if (ns == 4) return launch_rows_t<BITS, XMODE, 2, 2>(w, x, M, y, ydt, nwaves, epi, st);
+        if (ns == 4) return launch_rows_t<BITS, XMODE, 2, 2>(w, x, M, y, ydt, nwaves, epi, sub, st);
     } else {
-        if (ns == 4) return launch_rows_t<BITS, XMODE, 4, 4>(w, x, M, y, ydt, nwaves, epi, st);
+        if (ns == 4) return launch_rows_t<BITS, XMODE, 4, 4>(w, x, M, y, ydt, nwaves, epi, sub, st);
     }
-    if (ns == 2) return launch_rows_t<BITS, XMODE, 4, 2>(w, x, M, y, ydt, nwaves, epi, st);
+    if (ns == 2) return launch_rows_t<BITS, XMODE, 4, 2>(w, x, M, y, ydt, nwaves, epi, sub, st);
     if constexpr (BITS == 4) {
         // one strip per workgroup and a long K: eight tiles per wave and slab (fewer round trips), unless
         // that leaves more of the last slab empty than seven or four would - tiles past the end are still loaded
@@ -1036,30 +1078,30 @@ hipError_t launch_rows(const WeightView& w, const void* x, int M, void* y, int y
         if (w.KT > nwaves * 4) {
             // (seven or eight tiles of full-width x loads and a folded norm do not fit the registers)
             const bool fits = !epi.gamma || M <= 8;
-            if (pad(8) <= pad(7) && pad(8) <= pad(4) && fits) return launch_rows_t<BITS, XMODE, 8, 1>(w, x, M, y, ydt, nwaves, epi, st);
-            if (pad(7) <= pad(4) && fits) return launch_rows_t<BITS, XMODE, 7, 1>(w, x, M, y, ydt, nwaves, epi, st);
+            if (pad(8) <= pad(7) && pad(8) <= pad(4) && fits) return launch_rows_t<BITS, XMODE, 8, 1>(w, x, M, y, ydt, nwaves, epi, sub, st);
+            if (pad(7) <= pad(4) && fits) return launch_rows_t<BITS, XMODE, 7, 1>(w, x, M, y, ydt, nwaves, epi, sub, st);
         }
     }
-    return launch_rows_t<BITS, XMODE, 4, 1>(w, x, M, y, ydt, nwaves, epi, st);
+    return launch_rows_t<BITS, XMODE, 4, 1>(w, x, M, y, ydt, nwaves, epi, sub, st);
 }
 
 // 17 .. 32 rows: two activation operands per weight operand.  Two tiles of x per wave and slab
 // (a wave holds 2 x 2 x 4 operand fragments) when a workgroup has several strips, four with one.
 template <int BITS, int XMODE>
 hipError_t launch_rows2(const WeightView& w, const void* x, int M, void* y, int ydt, int tuned_waves, int num_cus,
-                        const Epilogue& epi, hipStream_t st)
+                        const Epilogue& epi, bool sub, hipStream_t st)
 {
     const int ns = strips_per_group(w, num_cus, epi);
     int nwaves = tuned_waves > 0 ? min(tuned_waves, 8) : 8;
     while (nwaves > 1 && nwaves * 2 > w.KT) nwaves >>= 1;
     if constexpr (BITS == 4) {
         if (w.NT == 7 * num_cus && epi.kind != kEpiSwiglu)
-            return launch_rows_x<BITS, XMODE, 2, 7, 16, 2>(w, x, M, y, ydt, nwaves, epi, st);
-        if (ns == 4) return launch_rows_x<BITS, XMODE, 2, 4, 16, 2>(w, x, M, y, ydt, nwaves, epi, st);
+            return launch_rows_x<BITS, XMODE, 2, 7, 16, 2>(w, x, M, y, ydt, nwaves, epi, sub, st);
+        if (ns == 4) return launch_rows_x<BITS, XMODE, 2, 4, 16, 2>(w, x, M, y, ydt, nwaves, epi, sub, st);
     }
-    if (ns >= 2) return launch_rows_x<BITS, XMODE, 2, 2, 16, 2>(w, x, M, y, ydt, nwaves, epi, st);
-    if constexpr (BITS == 4) return launch_rows_x<BITS, XMODE, 4, 1, 16, 2>(w, x, M, y, ydt, nwaves, epi, st);
-    return launch_rows_x<BITS, XMODE, 2, 1, 16, 2>(w, x, M, y, ydt, nwaves, epi, st);
+    if (ns >= 2) return launch_rows_x<BITS, XMODE, 2, 2, 16, 2>(w, x, M, y, ydt, nwaves, epi, sub, st);
+    if constexpr (BITS == 4) return launch_rows_x<BITS, XMODE, 4, 1, 16, 2>(w, x, M, y, ydt, nwaves, epi, sub, st);
+    return launch_rows_x<BITS, XMODE, 2, 1, 16, 2>(w, x, M, y, ydt, nwaves, epi, sub, st);
 }
 
 int g_tune_waves = 0, g_tune_unroll = 0, g_tune_rows = 0;
@@ -1190,19 +1232,19 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
     if (M > 16) {
         if (!gemv_serves_32(xdt, M, epi)) return hipErrorInvalidValue;
         if (w.bits == 4) {
-            if (xdt == kF16) return launch_rows2<4, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
-            return launch_rows2<4, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
+            if (xdt == kF16) return launch_rows2<4, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, !exact_operands, st);
+            return launch_rows2<4, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, !exact_operands, st);
         }
-        if (xdt == kF16) return launch_rows2<8, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
-        return launch_rows2<8, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
+        if (xdt == kF16) return launch_rows2<8, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, !exact_operands, st);
+        return launch_rows2<8, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, !exact_operands, st);
     }
     if (rows_kernel && xdt != kF32) {
         if (w.bits == 4) {
-            if (xdt == kF16) return launch_rows<4, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
-            return launch_rows<4, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
+            if (xdt == kF16) return launch_rows<4, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, !exact_operands, st);
+            return launch_rows<4, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, !exact_operands, st);
         }
-        if (xdt == kF16) return launch_rows<8, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
-        return launch_rows<8, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, st);
+        if (xdt == kF16) return launch_rows<8, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, !exact_operands, st);
+        return launch_rows<8, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, !exact_operands, st);
     }
 
     if (w.bits == 4) {

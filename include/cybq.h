@@ -87,7 +87,9 @@ typedef enum cybq_dtype { CYBQ_F32 = 0, CYBQ_F16 = 1, CYBQ_BF16 = 2 } cybq_dtype
  *          the fp32 CPU path only by accumulation order.  Half the throughput. */
 typedef enum cybq_prefill_mode { CYBQ_PREFILL_FAST = 0, CYBQ_PREFILL_EXACT = 1 } cybq_prefill_mode;
 
-/* How the decode kernel for one and two rows of 16-bit activations forms its weight operands.  Both
+/* How the decode kernels for one and two rows of 16-bit activations - and, for Q4 with f16
+ * activations, the batched-rows kernel for 3 .. 32 rows on outputs wide enough for two to four
+ * 16-row strips per workgroup - form their weight operands.  Both
  * accumulate in fp32 and stay far inside the 1e-3 tolerance.
  *   STREAM (default) the packed nibbles / bytes are used straight from memory - as f16 subnormals
  *          (q + bias) * 2^-22 with f16 activations, as the bf16 numbers 128 + (q + bias) with bf16

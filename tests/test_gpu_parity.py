@@ -215,6 +215,44 @@ def test_decode_17_to_32_rows_in_one_pass(backend, oracle, bits, xdt, shape):
         assert ((y3.double() - ref).norm() / ref.norm()).item() < TIGHT
 
 
+@pytest.mark.parametrize("N", [8192, 12288])
+def test_decode_modes_in_the_batched_rows_kernel(backend, oracle, N):
+    """3 .. 32 f16 rows on outputs wide enough for two / four strips per workgroup: STREAM feeds the Q4
+    weights as f16 subnormals there too (bias off through the MFMA's C operand, one bias product per K
+    tile for all strips), EXACT the integer operands; both inside the tight bar, and not the same bits."""
+    K = 640
+    q, s = _quant(oracle, 4, N, K, cfg=29)
+    qw = backend.upload_quantized(q, s, 4)
+    qz = backend.upload_quantized(np.zeros((N, K), np.int8), s, 4)
+    wd = torch.from_numpy(oracle.dequant(q, s)).cuda().double()
+    x = _x(32, K, "f16", cfg=30)
+    try:
+        for M in (3, 8, 16, 24, 32):
+            xm = x[:M].contiguous()
+            ref = xm.double() @ wd.T
+            outs = {}
+            for mode in ("stream", "exact"):
+                backend.set_decode_mode(mode)
+                y = _run(backend, qw, xm)
+                err = ((y.double() - ref).norm() / ref.norm()).item()
+                assert err < (TIGHT if mode == "stream" else 1e-6), (M, mode, err)
+                outs[mode] = y
+                z = _run(backend, qz, xm)
+                if mode == "exact":
+                    assert not z.any()
+                else:
+                    assert z.abs().max().item() < 1e-4 * ref.abs().mean().item()
+            assert not torch.equal(outs["stream"], outs["exact"]), M
+            # bf16 rows on the same strips: biased operands, the bias product shared by a tile's strips
+            xb = _x(M, K, "bf16", cfg=31)
+            yb = _run(backend, qw, xb)
+            refb = xb.double() @ wd.T
+            assert ((yb.double() - refb).norm() / refb.norm()).item() < TIGHT, M
+            assert _run(backend, qz, xb).abs().max().item() < 1e-4 * refb.abs().mean().item()      # (the bias cancels to rounding)
+    finally:
+        backend.set_decode_mode("stream")
+
+
 def test_decode_long_k_uses_several_slabs(backend, oracle):
     # M * K * 2 B exceeds the kernel's LDS budget: x is staged slab by slab
     N, K = 64, 14336
