@@ -958,7 +958,31 @@ def _random_cases(seed, count):
 
 @pytest.mark.parametrize("case", _random_cases(int(__import__("os").environ.get("CYBQ_FUZZ_SEED", "20240607")), int(__import__("os").environ.get("CYBQ_FUZZ_COUNT", "72"))), ids=lambda c: "-".join(str(v) for v in c.values()))
 def test_random_calls_match_float64(backend, oracle, case):
-    c = case
+    _check_random_case(backend, oracle, case)
+
+
+def _random_wide_cases(seed, count):
+    """The same draws over outputs wide enough for workgroups of two, four, seven or eight strips, several
+    rounds of workgroups, one round of narrow prefill tiles: the variants the model shapes run, on a short K."""
+    rng = np.random.default_rng(seed)
+    rows = [1, 2, 3, 4, 7, 8, 12, 16, 17, 24, 32, 33, 48, 64, 100, 128, 200, 256, 300, 512]
+    cases = []
+    for i in range(count):
+        epi = ["none", "add", "swiglu"][int(rng.integers(0, 3))]
+        N = int(rng.choice([4096, 7168, 14336])) if epi == "swiglu" else int(rng.choice([6144, 8192, 9008, 12288, 14336, 16400, 28672]))
+        cases.append(dict(i=1000 + i, bits=int(rng.choice([4, 4, 8])), layout=int(rng.choice([formats.PLANAR, formats.BLOCK_AOS])),
+                          N=N, K=32 * int(rng.integers(1, 25)), M=int(rng.choice(rows)), xdt=str(rng.choice(["f16", "bf16", "f32"])),
+                          ydt=str(rng.choice(["f32", "f32", "f16", "bf16"])), epi=epi, norm=bool(rng.random() < 0.3),
+                          gdt=str(rng.choice(["f32", "f16", "bf16"])), mode=str(rng.choice(["fast", "fast", "exact"]))))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_wide_cases(20240608, int(__import__("os").environ.get("CYBQ_FUZZ_WIDE_COUNT", "48"))), ids=lambda c: "-".join(str(v) for v in c.values()))
+def test_random_wide_calls_match_float64(backend, oracle, case):
+    _check_random_case(backend, oracle, case)
+
+
+def _check_random_case(backend, oracle, c):
     bits, N, K, M = c["bits"], c["N"], c["K"], c["M"]
     backend.set_prefill_mode(c["mode"])
     try:
