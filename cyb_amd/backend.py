@@ -92,6 +92,7 @@ def load_library() -> ctypes.CDLL:
     # diagnostics (cyb_amd/csrc/cybq_debug.h), not part of the operator interface
     lib.cybq_debug_set_gemv_tuning.argtypes = [ci, ci, ci]
     lib.cybq_debug_read_weight.argtypes = [vp, i64, vp, ci, vp, vp, vp]
+    lib.cybq_debug_read_pattern.argtypes = [vp, i64, vp, ci, vp]
     lib.cybq_debug_mfma_loop.argtypes = [vp, ci, ci, vp, vp]
     _lib = lib
     return lib
@@ -424,6 +425,11 @@ class Backend:
         weight of `plan` (with_io: also the activation read and a 16-float store per strip)."""
         self._check(self._lib.cybq_debug_read_weight(self._ctx, plan.count, plan.w, 1 if with_io else 0, _ptr(x), _ptr(y),
                                                      stream))
+
+    def debug_read_pattern(self, plan: "MatmulPlan", pattern: int, stream: int = 0) -> None:
+        """Diagnostics: the weights of `plan` read by another pure-read pattern (1 .. 6, cybq_debug.h), one
+        launch per weight."""
+        self._check(self._lib.cybq_debug_read_pattern(self._ctx, plan.count, plan.w, pattern, stream))
 
     def debug_mfma_loop(self, waves_per_simd: int, iters: int, sink, stream: int = 0) -> None:
         """Diagnostics: `iters` x 16 independent v_mfma_f32_16x16x32_f16 per wave on every SIMD."""

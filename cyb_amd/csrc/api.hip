@@ -6,6 +6,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -35,6 +36,12 @@ struct cybq_weight {
     // some |scale| * qmax exceeds what f16 holds: the prefill kernels, which form scale * q in
     // f16, would overflow; such a tensor takes the decode kernels (scale applied in fp32) for any M
     bool wide_scales = false;
+    // cybq_weight_from_device: the repack kernel ORs "some scale is wide" into a word behind the tiles and a
+    // copy of it to `scan_host` (pinned) is queued behind the kernel; the first call that needs the answer
+    // waits for `scan_done` (long since complete in practice) and moves it into wide_scales
+    hipEvent_t scan_done = nullptr;
+    uint32_t* scan_host = nullptr;
+    std::once_flag scan_once;
 };
 
 namespace cybq {
@@ -76,6 +83,7 @@ constexpr int64_t kStaticMaxK = 32768;          // 256 staged rows of 2-byte act
 constexpr int kMaxDevices = 64;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 void* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;              // contexts may be created from several threads
 
 int fail(cybq_ctx* ctx, int code, const char* what)
 {
@@ -140,6 +148,8 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 size_t dtype_size(int dt) { return dt == CYBQ_F32 ? 4 : 2; }
 bool dtype_ok(int dt) { return dt == CYBQ_F32 || dt == CYBQ_F16 || dt == CYBQ_BF16; }
 
+constexpr size_t kWeightTailBytes = 256;
+
 int alloc_weight(cybq_ctx* ctx, int bits, int64_t N, int64_t K, cybq_weight** out)
 {
     cybq_weight* w = new (std::nothrow) cybq_weight();
@@ -151,13 +161,34 @@ int alloc_weight(cybq_ctx* ctx, int bits, int64_t N, int64_t K, cybq_weight** ou
     w->NT = (int)((N + cybq::kTileN - 1) / cybq::kTileN);
     w->KT = (int)((K + cybq::kTileK - 1) / cybq::kTileK);
     w->bytes = (size_t)w->NT * w->KT * cybq::tile_bytes(bits);
-    hipError_t e = hipMalloc(reinterpret_cast<void**>(&w->data), w->bytes);
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&w->data), w->bytes + kWeightTailBytes);      // (tail: the scan's flag word)
     if (e != hipSuccess) {
         delete w;
         return fail_hip(ctx, e, "hipMalloc(weight)");
     }
     *out = w;
     return CYBQ_OK;
+}
+
+void release_weight(cybq_weight* w)
+{
+    if (w->scan_done) (void)hipEventDestroy(w->scan_done);
+    if (w->scan_host) (void)hipHostFree(w->scan_host);
+    (void)hipFree(w->data);
+    delete w;
+}
+
+// wide_scales of a weight whose scales were scanned on the device: the answer is taken the first time it is needed
+bool weight_is_wide(const cybq_weight* cw)
+{
+    cybq_weight* w = const_cast<cybq_weight*>(cw);
+    if (w->scan_host) {
+        std::call_once(w->scan_once, [w]() {
+            if (w->scan_done) (void)hipEventSynchronize(w->scan_done);
+            w->wide_scales = w->wide_scales || *w->scan_host != 0u;
+        });
+    }
+    return w->wide_scales;
 }
 
 int check_weight_shape(cybq_ctx* ctx, int quant, int64_t N, int64_t K)
@@ -211,11 +242,14 @@ int cybq_init(int device, cybq_ctx** out)
     // this device: launches never touch function attributes
     e = cybq::raise_all_lds_limits();
     if (e != hipSuccess) { (void)hipGetLastError(); return CYBQ_ERR_HIP; }
-    if (device < kMaxDevices && !g_scratch_ptr[device]) {       // this device's copy of the static scratch
-        void* p = nullptr;
-        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-        if (e != hipSuccess || !p) { (void)hipGetLastError(); return CYBQ_ERR_HIP; }
-        g_scratch_ptr[device] = p;
+    if (device < kMaxDevices) {       // this device's copy of the static scratch
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (!g_scratch_ptr[device]) {
+            void* p = nullptr;
+            e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !p) { (void)hipGetLastError(); return CYBQ_ERR_HIP; }
+            g_scratch_ptr[device] = p;
+        }
     }
     cybq_ctx* ctx = new (std::nothrow) cybq_ctx();
     if (!ctx) return CYBQ_ERR_NOMEM;
@@ -277,12 +311,11 @@ int cybq_weight_upload(cybq_ctx* ctx, cybq_quant quant, cybq_layout layout, int6
         e = hipMemcpy(q_tmp, q, q_src_bytes, hipMemcpyHostToDevice);
         if (e == hipSuccess && s_src_bytes) e = hipMemcpy(s_tmp, scales, s_src_bytes, hipMemcpyHostToDevice);
         if (e == hipSuccess)
-            e = cybq::launch_repack(quant, layout, q_tmp, s_tmp, w->data, (int)N, (int)K, w->NT, w->KT, nullptr);
+            e = cybq::launch_repack(quant, layout, q_tmp, s_tmp, w->data, (int)N, (int)K, w->NT, w->KT, nullptr, nullptr);
         if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
         if (e != hipSuccess) {
             rc = fail_hip(ctx, e, "weight upload");
-            (void)hipFree(w->data);
-            delete w;
+            release_weight(w);
             w = nullptr;
         }
     }
@@ -310,11 +343,23 @@ int cybq_weight_from_device(cybq_ctx* ctx, cybq_quant quant, int64_t N, int64_t 
     cybq_weight* w = nullptr;
     rc = alloc_weight(ctx, quant, N, K, &w);
     if (rc) return rc;
-    hipError_t e = cybq::launch_repack(quant, CYBQ_LAYOUT_PLANAR, q_dev, scales_dev, w->data, (int)N, (int)K,
-                                       w->NT, w->KT, static_cast<hipStream_t>(stream));
+    // the scales are scanned by the repack kernel itself: a word behind the tiles collects "some |scale| * qmax leaves
+    // f16", its copy to pinned host memory is queued behind the kernel and read by the first call that needs it
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    uint32_t* flag = reinterpret_cast<uint32_t*>(w->data + w->bytes);
+    hipError_t e = hipHostMalloc(reinterpret_cast<void**>(&w->scan_host), sizeof(uint32_t), hipHostMallocDefault);
+    if (e == hipSuccess) {
+        *w->scan_host = 0u;
+        e = hipEventCreateWithFlags(&w->scan_done, hipEventDisableTiming);
+    }
+    if (e == hipSuccess) e = hipMemsetAsync(flag, 0, sizeof(uint32_t), st);
+    if (e == hipSuccess)
+        e = cybq::launch_repack(quant, CYBQ_LAYOUT_PLANAR, q_dev, scales_dev, w->data, (int)N, (int)K, w->NT, w->KT, flag, st);
+    if (e == hipSuccess) e = hipMemcpyAsync(w->scan_host, flag, sizeof(uint32_t), hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipEventRecord(w->scan_done, st);
     if (e != hipSuccess) {
-        (void)hipFree(w->data);
-        delete w;
+        (void)hipStreamSynchronize(st);          // nothing may still write the pinned word
+        release_weight(w);
         return fail_hip(ctx, e, "repack launch");
     }
     *out = w;
@@ -334,12 +379,11 @@ int cybq_weight_clone(cybq_ctx* ctx, const cybq_weight* src, cybq_weight** out)
     if (rc) return rc;
     hipError_t e = hipMemcpy(w->data, src->data, src->bytes, hipMemcpyDeviceToDevice);
     if (e != hipSuccess) {
-        (void)hipFree(w->data);
-        delete w;
+        release_weight(w);
         return fail_hip(ctx, e, "weight clone");
     }
     w->paired = src->paired;
-    w->wide_scales = src->wide_scales;
+    w->wide_scales = weight_is_wide(src);
     *out = w;
     return CYBQ_OK;
 }
@@ -348,7 +392,11 @@ int cybq_weight_free(cybq_ctx* ctx, cybq_weight* w)
 {
     if (!w) return CYBQ_OK;
     hipError_t e = hipSetDevice(w->device);
-    if (e == hipSuccess) e = hipFree(w->data);
+    if (e == hipSuccess) {
+        if (w->scan_done) (void)hipEventDestroy(w->scan_done);
+        if (w->scan_host) (void)hipHostFree(w->scan_host);
+        e = hipFree(w->data);
+    }
     delete w;
     if (e != hipSuccess) return fail_hip(ctx, e, "hipFree(weight)");
     return CYBQ_OK;
@@ -408,15 +456,17 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
         // workgroups and add the slabs in a second pass; two passes of the batched-rows decode kernel
         // (32 rows, then the rest) are quicker although they stream the weights twice
         // (4096 -> 4096 at 64 rows 21.8 -> 14.8 us, 4096 -> 1024 17.8 -> 12.6 us) - and exact
+        // (a context in CYBQ_PREFILL_EXACT mode asked for exact operands at this row count)
+        const bool exact_ops = ctx->decode_exact || ctx->prefill_exact;
         const int64_t n_out = epi.kind == cybq::kEpiSwiglu ? w->N / 2 : w->N;
         const size_t yoff = (size_t)32 * n_out * dtype_size(ydt);
         cybq::Epilogue ec = epi;
         if (epi.kind == cybq::kEpiAdd) ec.residual = static_cast<const char*>(residual) + yoff;
-        e = cybq::launch_gemv(v, x, xdt, 32, y, ydt, ctx->num_cus, ctx->decode_exact, epi, st);
+        e = cybq::launch_gemv(v, x, xdt, 32, y, ydt, ctx->num_cus, exact_ops, epi, st);
         if (e == hipSuccess)
             e = cybq::launch_gemv(v, static_cast<const char*>(x) + (size_t)32 * w->K * dtype_size(xdt), xdt, (int)M - 32,
-                                  static_cast<char*>(y) + yoff, ydt, ctx->num_cus, ctx->decode_exact, ec, st);
-    } else if (!w->wide_scales && (xdt == CYBQ_F32 ? !ctx->prefill_exact : M > 32)) {
+                                  static_cast<char*>(y) + yoff, ydt, ctx->num_cus, exact_ops, ec, st);
+    } else if (!weight_is_wide(w) && (xdt == CYBQ_F32 ? !ctx->prefill_exact : M > 32)) {
         e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, workspace, workspace_bytes,
                               epi, st);
     } else {
@@ -427,10 +477,13 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
         // rows of 16-bit activations with a folded norm: two passes of the batched-rows
         // kernel stream the weights twice and are still quicker than a 128-row MFMA tile
         // mostly empty (without the norm they are one pass, two row blocks per weight operand).
+        // A tensor with wide scales (scale * q leaves f16) is walked the same way for any M, 32 rows at a
+        // time where the batched-rows kernel takes them in one pass: the weights stream once per 32 rows.
         e = hipSuccess;
         const int64_t n_out = epi.kind == cybq::kEpiSwiglu ? w->N / 2 : w->N;
-        for (int64_t m0 = 0; m0 < M && e == hipSuccess; m0 += 16) {
-            int mm = (int)((M - m0) < 16 ? (M - m0) : 16);
+        const int64_t step = cybq::gemv_serves_32((int)xdt, 32, epi) ? 32 : 16;
+        for (int64_t m0 = 0; m0 < M && e == hipSuccess; m0 += step) {
+            int mm = (int)((M - m0) < step ? (M - m0) : step);
             const char* xp = static_cast<const char*>(x) + (size_t)m0 * w->K * dtype_size(xdt);
             const size_t yoff = (size_t)m0 * n_out * dtype_size(ydt);
             cybq::Epilogue ec = epi;
@@ -469,12 +522,16 @@ int cybq_matmul_static(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_
                        cybq_dtype ydt, void* stream)
 {
     if (!ctx) return CYBQ_ERR_INVALID;
-    if (ctx->device >= kMaxDevices || !g_scratch_ptr[ctx->device])
-        return fail(ctx, CYBQ_ERR_UNSUPPORTED, "no static scratch on this device");
+    void* static_scratch = nullptr;
+    if (ctx->device < kMaxDevices) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        static_scratch = g_scratch_ptr[ctx->device];
+    }
+    if (!static_scratch) return fail(ctx, CYBQ_ERR_UNSUPPORTED, "no static scratch on this device");
     if (w && M > 16 && w->K > kStaticMaxK)
         return fail(ctx, CYBQ_ERR_UNSUPPORTED, "cybq_matmul_static: K beyond 32768 does not fit the static scratch for more than 16 rows");
     return matmul_fused(ctx, w, x, xdt, M, nullptr, CYBQ_F32, 0.f, y, ydt, CYBQ_EPI_NONE, nullptr, stream,
-                        g_scratch_ptr[ctx->device], kStaticScratchBytes);
+                        static_scratch, kStaticScratchBytes);
 }
 
 int cybq_weight_fuse_pairs(cybq_ctx* ctx, const cybq_weight* gate, const cybq_weight* up, cybq_weight** out)
@@ -497,12 +554,11 @@ int cybq_weight_fuse_pairs(cybq_ctx* ctx, const cybq_weight* gate, const cybq_we
     if (e == hipSuccess) e = hipMemcpy2D(w->data + sb, 2 * sb, up->data, sb, sb, up->NT, hipMemcpyDeviceToDevice);
     if (e == hipSuccess) e = hipDeviceSynchronize();
     if (e != hipSuccess) {
-        (void)hipFree(w->data);
-        delete w;
+        release_weight(w);
         return fail_hip(ctx, e, "weight fuse");
     }
     w->paired = true;
-    w->wide_scales = gate->wide_scales || up->wide_scales;
+    w->wide_scales = weight_is_wide(gate) || weight_is_wide(up);
     *out = w;
     return CYBQ_OK;
 }
@@ -615,6 +671,24 @@ int cybq_debug_read_weight(cybq_ctx* ctx, int64_t count, const cybq_weight* cons
         if (e == hipErrorInvalidValue) {
             (void)hipGetLastError();
             return fail(ctx, CYBQ_ERR_UNSUPPORTED, "probe needs K % 512 == 0 and K <= 16384");
+        }
+        if (e != hipSuccess) return fail_hip(ctx, e, "probe launch");
+    }
+    return CYBQ_OK;
+}
+
+int cybq_debug_read_pattern(cybq_ctx* ctx, int64_t count, const cybq_weight* const* w, int pattern, void* stream)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    if (count < 0 || (count > 0 && !w)) return fail(ctx, CYBQ_ERR_INVALID, "w is NULL");
+    DeviceGuard guard(ctx->device);
+    if (guard.err != hipSuccess) return fail_hip(ctx, guard.err, "hipSetDevice");
+    for (int64_t i = 0; i < count; i++) {
+        if (!w[i]) return fail(ctx, CYBQ_ERR_INVALID, "w[i] is NULL");
+        hipError_t e = cybq::launch_read_pattern(view_of(w[i]), pattern, ctx->num_cus, static_cast<hipStream_t>(stream));
+        if (e == hipErrorInvalidValue) {
+            (void)hipGetLastError();
+            return fail(ctx, CYBQ_ERR_UNSUPPORTED, "unknown pattern, or a strip pattern on a tensor that is not Q4 with K = 4096");
         }
         if (e != hipSuccess) return fail_hip(ctx, e, "probe launch");
     }

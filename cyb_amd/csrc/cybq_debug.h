@@ -31,6 +31,16 @@ int cybq_debug_set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll)
 int cybq_debug_read_weight(cybq_ctx* ctx, int64_t count, const cybq_weight* const* w, int with_io, const void* x, void* y,
                            void* stream);
 
+/* The same bytes read in other ways, again with nothing done to the data: how long a launch that only
+ * reads the tensor takes, whatever its decomposition.  `count` launches back to back, one per tensor.
+ *   pattern 1  a strip per workgroup as in the decode kernel, but 4 waves x 2 sets (Q4, K = 4096 only)
+ *   pattern 2  a strip per workgroup, 2 waves x 4 sets (Q4, K = 4096 only)
+ *   pattern 3  flat: every wave reads one contiguous 8 KiB, all of it requested at once, one round
+ *   pattern 4  persistent grid: one 16-wave workgroup per CU walks the tensor 4 KiB per wave and round
+ *   pattern 5  persistent grid with the next chunk requested before the current one is consumed
+ *   pattern 6  flat, 4 KiB per wave straight into LDS (no registers held while a request is in flight) */
+int cybq_debug_read_pattern(cybq_ctx* ctx, int64_t count, const cybq_weight* const* w, int pattern, void* stream);
+
 /* A loop of independent v_mfma_f32_16x16x32_f16 on every SIMD of the chip: `waves_per_simd`
  * waves each issue `iters` x 16 instructions.  flops = CUs * 4 * waves_per_simd * iters * 16 * 16384. */
 int cybq_debug_mfma_loop(cybq_ctx* ctx, int waves_per_simd, int iters, float* sink, void* stream);

@@ -14,8 +14,9 @@ namespace cybq {
 constexpr int kF32 = 0, kF16 = 1, kBF16 = 2;
 
 // q: PLANAR q plane (4-byte aligned) with `scales`, or BLOCK_AOS blocks (2-byte aligned, scales unused)
+// wide_flag: device word that receives 1 when some scale times the largest q leaves f16 (nullptr: no scan)
 hipError_t launch_repack(int bits, int layout, const void* q, const void* scales, uint8_t* dst, int N, int K, int NT, int KT,
-                         hipStream_t st);
+                         uint32_t* wide_flag, hipStream_t st);
 hipError_t launch_dequant(const WeightView& w, float* out, hipStream_t st);
 
 // decode path, 1 <= M <= 16 per call, and 17 .. 32 rows where gemv_serves_32 says so (api.hip
@@ -56,6 +57,8 @@ struct LdsRequest {
 
 // measurement probes (debug.hip)
 hipError_t launch_read_probe(const WeightView& w, bool io, const void* x, void* y, hipStream_t st);
+// other pure-read patterns over the same bytes (pattern 1 .. 6, see cybq_debug.h)
+hipError_t launch_read_pattern(const WeightView& w, int pattern, int num_cus, hipStream_t st);
 hipError_t launch_mfma_loop(int num_cus, int waves_per_simd, int iters, float* sink, hipStream_t st);
 
 // test/bench hook: overrides the decode kernel's launch heuristics (0 = automatic)

@@ -47,6 +47,110 @@ __global__ __launch_bounds__(1024) void read_probe_kernel(const uint8_t* __restr
     if (r == 0x12345679u && y) y[0] = 1.f;              // never true in practice: keeps every wave's loads alive
 }
 
+// ---- other ways of reading the same bytes (nothing is done with the data): what the memory system gives a
+// launch that only reads a tensor, whatever the decomposition
+
+// the strip-per-workgroup pattern with fewer, fatter waves: wave wv of `nwaves` owns SETS sets of four tiles
+template <int SETS>
+__global__ __launch_bounds__(512) void read_strip_sets_kernel(const uint8_t* __restrict__ wbase, int KT, int nwaves, float* __restrict__ sink)
+{
+    constexpr int TB = kTileBytes<4>, QB = kTileQBytes<4>;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int row = lane & 15, blk = lane >> 4;
+    u32x4_t q[SETS][4];
+    u32x2_t sc[SETS];
+#pragma unroll
+    for (int h = 0; h < SETS; h++) {
+        const uint8_t* sb = wbase + (int64_t)((int)blockIdx.x * KT + 4 * (wv + nwaves * h)) * TB;
+        sc[h] = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(sb + ((uint32_t)blk * TB + QB + row * 8)));
+#pragma unroll
+        for (int b = 0; b < 4; b++) q[h][b] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(sb + b * TB + lane * 16));
+    }
+    uint32_t r = 0;
+#pragma unroll
+    for (int h = 0; h < SETS; h++) {
+        r ^= sc[h][0] ^ sc[h][1];
+#pragma unroll
+        for (int b = 0; b < 4; b++) r ^= q[h][b][0] ^ q[h][b][1] ^ q[h][b][2] ^ q[h][b][3];
+    }
+    if (r == 0x12345679u && sink) sink[0] = 1.f;
+}
+
+// flat: wave w of the launch reads the chunks w, w + W, ... of U KiB each, a chunk's U loads requested together
+// (one round when the grid covers the tensor, a grid-stride loop over it otherwise: a persistent grid)
+template <int U>
+__global__ __launch_bounds__(1024) void read_flat_kernel(const u32x4_t* __restrict__ p, uint32_t n16, float* __restrict__ sink)
+{
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint32_t nw = (gridDim.x * blockDim.x) >> 6;
+    u32x4_t acc = {0u, 0u, 0u, 0u};
+    for (uint32_t base = wave * (U * 64); base < n16; base += nw * (U * 64)) {
+        u32x4_t v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) v[u] = __builtin_nontemporal_load(p + min(base + u * 64 + lane, n16 - 1));
+#pragma unroll
+        for (int u = 0; u < U; u++) acc ^= v[u];
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345679u && sink) sink[0] = 1.f;
+}
+
+// the same persistent walk with the next chunk requested before the current one is consumed (two register sets)
+template <int U>
+__global__ __launch_bounds__(1024) void read_flat_ahead_kernel(const u32x4_t* __restrict__ p, uint32_t n16, float* __restrict__ sink)
+{
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint32_t step = ((gridDim.x * blockDim.x) >> 6) * (U * 64);
+    u32x4_t acc = {0u, 0u, 0u, 0u};
+    u32x4_t va[U], vb[U];
+    uint32_t base = wave * (U * 64);
+    if (base < n16) {
+#pragma unroll
+        for (int u = 0; u < U; u++) va[u] = __builtin_nontemporal_load(p + min(base + u * 64 + lane, n16 - 1));
+    }
+    // (two chunks per round so that the register sets are compile-time names)
+    for (; base < n16; base += 2 * step) {
+        if (base + step < n16) {
+#pragma unroll
+            for (int u = 0; u < U; u++) vb[u] = __builtin_nontemporal_load(p + min(base + step + u * 64 + lane, n16 - 1));
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) acc ^= va[u];
+        if (base + 2 * step < n16) {
+#pragma unroll
+            for (int u = 0; u < U; u++) va[u] = __builtin_nontemporal_load(p + min(base + 2 * step + u * 64 + lane, n16 - 1));
+        }
+        if (base + step < n16) {
+#pragma unroll
+            for (int u = 0; u < U; u++) acc ^= vb[u];
+        }
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345679u && sink) sink[0] = 1.f;
+}
+
+// straight into LDS (no registers held while a request is in flight), U KiB per wave and round
+template <int U>
+__global__ __launch_bounds__(512) void read_lds_kernel(const u32x4_t* __restrict__ p, uint32_t n16, float* __restrict__ sink)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t ring[8 * U * 1024];
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint32_t nw = (gridDim.x * blockDim.x) >> 6;
+    uint8_t* mine = ring + (threadIdx.x >> 6) * (U * 1024);
+    uint32_t acc = 0;
+    for (uint32_t base = wave * (U * 64); base < n16; base += nw * (U * 64)) {
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p + min(base + u * 64 + lane, n16 - 1)),
+                                             (__attribute__((address_space(3))) void*)(mine + u * 1024), 16, 0, 0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        acc ^= *reinterpret_cast<const uint32_t*>(mine + lane * 4);
+    }
+    if (acc == 0x12345679u && sink) sink[0] = 1.f;
+}
+
 __global__ __launch_bounds__(256) void mfma_loop_kernel(int iters, float* __restrict__ sink)
 {
     Frag16 a, b;
@@ -87,6 +191,38 @@ hipError_t launch_read_probe(const WeightView& w, bool io, const void* x, void* 
     else if (per_wave == 1) CYBQ_PROBE(8, 1);
     else CYBQ_PROBE(8, 2);
 #undef CYBQ_PROBE
+    return hipGetLastError();
+}
+
+hipError_t launch_read_pattern(const WeightView& w, int pattern, int num_cus, hipStream_t st)
+{
+    const int64_t bytes = (int64_t)w.NT * w.KT * tile_bytes(w.bits);
+    if (bytes < 16 || bytes / 16 > 0x7fffffff) return hipErrorInvalidValue;
+    const uint32_t n16 = (uint32_t)(bytes / 16);
+    const u32x4_t* p = reinterpret_cast<const u32x4_t*>(w.base);
+    float* sink = nullptr;
+    auto waves_to_groups = [](int64_t waves, int per_group) { return (unsigned)((waves + per_group - 1) / per_group); };
+    switch (pattern) {
+        case 1:      // a strip per workgroup, 4 waves x 2 sets
+        case 2:      // a strip per workgroup, 2 waves x 4 sets
+            if (w.bits != 4 || w.KT != 32) return hipErrorInvalidValue;
+            if (pattern == 1) hipLaunchKernelGGL((read_strip_sets_kernel<2>), dim3((unsigned)w.NT), dim3(256), 0, st, w.base, w.KT, 4, sink);
+            else hipLaunchKernelGGL((read_strip_sets_kernel<4>), dim3((unsigned)w.NT), dim3(128), 0, st, w.base, w.KT, 2, sink);
+            break;
+        case 3:      // flat, one round: 8 KiB per wave, four waves per workgroup
+            hipLaunchKernelGGL((read_flat_kernel<8>), dim3(waves_to_groups((n16 + 511) / 512, 4)), dim3(256), 0, st, p, n16, sink);
+            break;
+        case 4:      // persistent grid: one 16-wave workgroup per CU, 4 KiB per wave and round
+            hipLaunchKernelGGL((read_flat_kernel<4>), dim3((unsigned)num_cus), dim3(1024), 0, st, p, n16, sink);
+            break;
+        case 5:      // persistent grid, the next chunk requested before the current one is consumed
+            hipLaunchKernelGGL((read_flat_ahead_kernel<2>), dim3((unsigned)num_cus), dim3(1024), 0, st, p, n16, sink);
+            break;
+        case 6:      // straight into LDS, 4 KiB per wave, one round
+            hipLaunchKernelGGL((read_lds_kernel<4>), dim3(waves_to_groups((n16 + 255) / 256, 8)), dim3(512), 0, st, p, n16, sink);
+            break;
+        default: return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

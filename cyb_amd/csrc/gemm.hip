@@ -1043,7 +1043,7 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void* __restrict_
     if (amax > 0.f && amax < __builtin_inff()) {
         int e;
         (void)frexpf(amax, &e);
-        s = ldexpf(1.0f, 14 - e);
+        s = ldexpf(1.0f, min(14 - e, 126));        // (rows below 2^-112: 2^126 keeps s and 1 / s normal numbers)
     }
     if (lane == 0 && rb * 16 + r0 + r < M) {
         unscale[row] = 1.0f / s;

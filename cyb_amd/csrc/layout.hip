@@ -61,7 +61,7 @@ constexpr int kRepackTiles = 4;
 
 template <int BITS, int LAYOUT>
 __global__ __launch_bounds__(256) void repack_kernel(const uint8_t* __restrict__ q, const uint16_t* __restrict__ scales,
-                                                      uint8_t* __restrict__ dst, int N, int K, int KT)
+                                                      uint8_t* __restrict__ dst, int N, int K, int KT, uint32_t* __restrict__ wide_flag)
 {
     constexpr int CT = kRepackTiles;
     constexpr int GB = kSrcGroupBytes<BITS, LAYOUT>;
@@ -133,6 +133,12 @@ __global__ __launch_bounds__(256) void repack_kernel(const uint8_t* __restrict__
             else v = (uint16_t)(rows[r][gl * GB] | (rows[r][gl * GB + 1] << 8));
         }
         reinterpret_cast<uint16_t*>(tile + kTileQBytes<BITS>)[lane] = v;
+        // a scale whose product with the largest q leaves f16 (or that is not finite): the prefill kernels, which
+        // form scale * q in f16, cannot serve this tensor; every thread that sees one stores the same 1
+        if (wide_flag) {
+            const bool wide = ((v >> 10) & 31u) == 31u || f16_bits_to_f32(v & 0x7fffu) * (BITS == 4 ? 8.0f : 128.0f) > 65504.0f;
+            if (wide) *wide_flag = 1u;
+        }
     }
 }
 
@@ -169,24 +175,25 @@ __global__ void dequant_kernel(WeightView w, float* __restrict__ out)
 }
 
 template <int BITS, int LAYOUT>
-hipError_t launch_repack_t(const void* q, const void* scales, uint8_t* dst, int N, int K, int NT, int KT, hipStream_t st)
+hipError_t launch_repack_t(const void* q, const void* scales, uint8_t* dst, int N, int K, int NT, int KT, uint32_t* wide_flag,
+                           hipStream_t st)
 {
     const int64_t groups = (int64_t)((KT + kRepackTiles - 1) / kRepackTiles) * NT;
     if (groups > 0x7fffffff) return hipErrorInvalidValue;
     hipLaunchKernelGGL((repack_kernel<BITS, LAYOUT>), dim3((unsigned)groups), dim3(256), 0, st, (const uint8_t*)q, (const uint16_t*)scales, dst, N, K,
-                       KT);
+                       KT, wide_flag);
     return hipGetLastError();
 }
 
 }  // namespace
 
 hipError_t launch_repack(int bits, int layout, const void* q, const void* scales, uint8_t* dst, int N, int K, int NT, int KT,
-                         hipStream_t st)
+                         uint32_t* wide_flag, hipStream_t st)
 {
-    if (bits == 4 && layout == 0) return launch_repack_t<4, 0>(q, scales, dst, N, K, NT, KT, st);
-    if (bits == 4 && layout == 1) return launch_repack_t<4, 1>(q, scales, dst, N, K, NT, KT, st);
-    if (bits == 8 && layout == 0) return launch_repack_t<8, 0>(q, scales, dst, N, K, NT, KT, st);
-    if (bits == 8 && layout == 1) return launch_repack_t<8, 1>(q, scales, dst, N, K, NT, KT, st);
+    if (bits == 4 && layout == 0) return launch_repack_t<4, 0>(q, scales, dst, N, K, NT, KT, wide_flag, st);
+    if (bits == 4 && layout == 1) return launch_repack_t<4, 1>(q, scales, dst, N, K, NT, KT, wide_flag, st);
+    if (bits == 8 && layout == 0) return launch_repack_t<8, 0>(q, scales, dst, N, K, NT, KT, wide_flag, st);
+    if (bits == 8 && layout == 1) return launch_repack_t<8, 1>(q, scales, dst, N, K, NT, KT, wide_flag, st);
     return hipErrorInvalidValue;
 }
 

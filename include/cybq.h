@@ -75,7 +75,9 @@ typedef enum cybq_layout { CYBQ_LAYOUT_PLANAR = 0, CYBQ_LAYOUT_BLOCK_AOS = 1 } c
 typedef enum cybq_dtype { CYBQ_F32 = 0, CYBQ_F16 = 1, CYBQ_BF16 = 2 } cybq_dtype;
 
 /* How the prefill kernel (M > 32) feeds the matrix cores.  Both stay inside the
- * operator's 1e-3 relative-L2 tolerance; the decode kernels (M <= 32) are always exact.
+ * operator's 1e-3 relative-L2 tolerance.  (Calls of up to 32 rows, and 33 .. 64 rows on weights of up
+ * to 6144 x 4096, take the decode kernels, whose operand form cybq_decode_mode describes; with
+ * CYBQ_PREFILL_EXACT those 33 .. 64-row calls use the decode kernels' EXACT operands.)
  *   FAST   (default) one f16 MFMA per 32-group; the weight operand is
  *          round_f16(scale * q), relative error <= 2^-11 per weight (about 2e-4
  *          relative L2 on y).  bf16 and fp32 activations become f16 operands behind a
@@ -87,15 +89,21 @@ typedef enum cybq_dtype { CYBQ_F32 = 0, CYBQ_F16 = 1, CYBQ_BF16 = 2 } cybq_dtype
  *          the fp32 CPU path only by accumulation order.  Half the throughput. */
 typedef enum cybq_prefill_mode { CYBQ_PREFILL_FAST = 0, CYBQ_PREFILL_EXACT = 1 } cybq_prefill_mode;
 
-/* How the decode kernels for one and two rows of 16-bit activations - and, for Q4 with f16
- * activations, the batched-rows kernel for 3 .. 32 rows on outputs wide enough for two to four
- * 16-row strips per workgroup - form their weight operands.  Both
- * accumulate in fp32 and stay far inside the 1e-3 tolerance.
+/* How the decode kernels form their weight operands.  Every form accumulates in fp32, applies the
+ * f16 group scale in fp32 and stays far inside the 1e-3 tolerance.  Which form runs:
+ *   f16 activations   1 - 2 rows: STREAM -> subnormal operands, EXACT -> exact integers.
+ *                     3 - 32 rows (and the 33 - 64-row walk): STREAM -> subnormal operands for Q4 on
+ *                     outputs wide enough for two to four 16-row strips per workgroup, exact integers
+ *                     otherwise; EXACT -> exact integers.
+ *   bf16 activations  any row count, either mode: the bf16 numbers 128 + (q + bias) with the bias
+ *                     removed inside the accumulation (bf16 has no packed add to take it off
+ *                     beforehand); the mode only chooses the kernel for 1 - 2 rows.
+ *   fp32 activations  exact integers in either mode (activations split into two f16 halves).
  *   STREAM (default) the packed nibbles / bytes are used straight from memory - as f16 subnormals
- *          (q + bias) * 2^-22 with f16 activations, as the bf16 numbers 128 + (q + bias) with bf16
- *          activations - and the bias is removed inside the same fp32 accumulation; about 4e-7
- *          (bf16: 1e-6) relative L2 (the sums carry the bias until it cancels: a tensor of zeros
- *          gives values around 1e-7 of the activations' scale, not exact zeros), the quickest form.
+ *          (q + bias) * 2^-22 with f16 activations - and the bias is removed inside the same fp32
+ *          accumulation; about 4e-7 (bf16: 1e-6) relative L2.  The sums carry the bias until it
+ *          cancels: a tensor of zeros gives values around 1e-7 of the activations' scale, not exact
+ *          zeros (the same holds for bf16 activations in either mode).  The quickest form.
  *   EXACT  the weight operand is the exact integer q (more unpack arithmetic per byte);
  *          about 3e-7 relative L2, and a tensor of zeros gives exact zeros. */
 typedef enum cybq_decode_mode { CYBQ_DECODE_STREAM = 0, CYBQ_DECODE_EXACT = 1 } cybq_decode_mode;
@@ -254,9 +262,9 @@ int cybq_quantize(cybq_ctx* ctx, cybq_quant quant, const float* src, int64_t N, 
  * (the output of cybq_quantize); stream-ordered, allocates the handle.  The buffers must stay
  * valid until the work queued on `stream` has run; other calls that read the new weight
  * (cybq_weight_clone, cybq_weight_fuse_pairs, a matmul on another stream) must be ordered after it
- * by the caller.  The scales are not inspected here: they must keep |scale| * 8 (Q4) or
- * |scale| * 128 (Q8) within f16's range, which the output of cybq_quantize does for finite
- * weights up to 65504. */
+ * by the caller.  The scales are scanned on the device by the same kernel (a tensor whose
+ * |scale| * 8 (Q4) or |scale| * 128 (Q8) leaves f16's range is served by the decode kernels for
+ * every M, as after cybq_weight_upload); the first call that needs the answer waits for that kernel. */
 int cybq_weight_from_device(cybq_ctx* ctx, cybq_quant quant, int64_t N, int64_t K,
                             const void* q_dev, const void* scales_dev, void* stream,
                             cybq_weight** out);

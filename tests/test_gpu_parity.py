@@ -529,13 +529,19 @@ def test_prefill_fast_mode_activation_range(backend, oracle, xdt):
     x[8] *= 1e12
     x[9] = 0.0
     x[10, 1:] = 0.0
+    x[11] *= 1e-36                 # largest magnitude below 2^-113: the row's power of two stops at 2^126
+    if xdt == "f32":               # a row of fp32 subnormals (made on the host: bit patterns, not device arithmetic)
+        x[12] = torch.from_numpy(synth.activations(21, 40, K)[12] * np.float32(1e-40)).cuda()
     backend.set_prefill_mode("fast")
     y = _run(backend, qw, x).cpu().numpy()
     assert np.isfinite(y).all()
     assert not y[9].any()
     ref = oracle.matmul_f64(q, s, x.float().cpu().numpy())
-    for rows in ([0], [1], [2], [3], [4], [5], [6], [7], [8], [10], list(range(11, 40))):
+    for rows in ([0], [1], [2], [3], [4], [5], [6], [7], [8], [10], [11], list(range(13, 40))):
         assert oracle.rel_l2(y[rows], ref[rows]) < FAST, rows
+    # (the subnormal row: its operands keep what f16 holds below 2^126 times the row, and the result is itself
+    # an fp32 subnormal - finite, and as close as those two allow; with bf16 it is an ordinary row)
+    assert oracle.rel_l2(y[[12]], ref[[12]]) < (2e-2 if xdt == "f32" else FAST)
     # a folded norm sees the same rows (gamma of mixed magnitudes)
     gamma = torch.from_numpy(np.abs(synth.activations(22, 1, K))[0] * 10.0 + 1e-3).cuda()
     yn = torch.empty((40, N), dtype=torch.float32, device="cuda")
@@ -549,19 +555,35 @@ def test_prefill_fast_mode_activation_range(backend, oracle, xdt):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
-def test_scales_beyond_f16_products(backend, oracle, bits):
+@pytest.mark.parametrize("xdt", ["f16", "bf16", "f32"])
+def test_scales_beyond_f16_products(backend, oracle, bits, xdt):
     """scale * q would leave f16's range: such tensors take the decode kernels (scale in fp32) on both
-    sides of the prefill boundary."""
+    sides of the prefill boundary - whether the handle was built from host buffers (scanned on the host)
+    or from device buffers (scanned by the repack kernel)."""
     N, K = 64, 256
     q, s = _quant(oracle, bits, N, K)
     s = s.copy()
     s[::3, ::2] = np.float16(30000.0).view(np.uint16)
-    qw = backend.upload_quantized(q, s, bits, formats.BLOCK_AOS)
-    for M in (4, 32, 33, 100):
-        x = _x(M, K, "f16")
-        y = _run(backend, qw, x).cpu().numpy()
-        assert np.isfinite(y).all(), M
-        assert oracle.rel_l2(y, oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT, M
+    qd = torch.from_numpy(formats.pack_planar(q, bits)).cuda()
+    sd = torch.from_numpy(s.view(np.int16)).cuda()
+    handles = [backend.upload_quantized(q, s, bits, formats.BLOCK_AOS), backend.weight_from_device(bits, N, K, qd, sd)]
+    for qw in handles:
+        for M in (4, 32, 33, 100):
+            x = _x(M, K, xdt)
+            y = _run(backend, qw, x).cpu().numpy()
+            assert np.isfinite(y).all(), M
+            assert oracle.rel_l2(y, oracle.matmul_f64(q, s, x.float().cpu().numpy())) < TIGHT, M
+    # pairs built from a wide tensor stay wide
+    if bits == 4:
+        pair = backend.fuse_pairs(handles[1], handles[1])
+        x = _x(40, K, "f16")
+        y = torch.empty((40, N), dtype=torch.float32, device="cuda")
+        backend.matmul_ex(pair, x, y, "swiglu")
+        torch.cuda.synchronize()
+        assert torch.isfinite(y).all()
+        pair.free()
+    for qw in handles:
+        qw.free()
 
 
 def test_prefill_rows_agree_with_decode_rows(backend, oracle, prefill_mode):
@@ -1277,7 +1299,8 @@ def test_many_norm_without_gammas_is_many_ex_and_rejects_bad_arguments(backend, 
 def test_rows_33_to_64_on_a_small_weight_are_two_decode_passes(backend, oracle, M, xdt):
     """33..64 rows of 16-bit activations on a small weight: rows 0..31 carry the bits of a 32-row call,
     the rest those of a call with the remaining rows (a row's bits do not depend on the batch it is in),
-    in both prefill modes, and the float64 result within the decode kernels' bar."""
+    in both prefill modes (prefill EXACT asks the decode kernels for their exact operands), and the
+    float64 result within the decode kernels' bar."""
     N, K = 272, 1184
     q, s = _quant(oracle, 4, N, K, cfg=98)
     w = backend.upload_quantized(q, s, 4)
@@ -1290,6 +1313,7 @@ def test_rows_33_to_64_on_a_small_weight_are_two_decode_passes(backend, oracle, 
             backend.matmul_ex(w, x, y, "add", r)
             y_a = torch.empty((32, N), dtype=torch.float32, device="cuda")
             y_b = torch.empty((M - 32, N), dtype=torch.float32, device="cuda")
+            backend.set_decode_mode("exact" if mode == "exact" else "stream")
             backend.matmul_ex(w, x[:32].contiguous(), y_a, "add", r[:32].contiguous())
             backend.matmul_ex(w, x[32:].contiguous(), y_b, "add", r[32:].contiguous())
             torch.cuda.synchronize()
@@ -1298,6 +1322,16 @@ def test_rows_33_to_64_on_a_small_weight_are_two_decode_passes(backend, oracle, 
             assert oracle.rel_l2(y.cpu().numpy(), ref) < TIGHT
         finally:
             backend.set_prefill_mode("fast")
+            backend.set_decode_mode("stream")
+    if xdt == "f16":
+        # prefill EXACT at these row counts: a tensor of zeros gives exact zeros (the exact integer operands)
+        wz = backend.upload_quantized(np.zeros_like(q), s, 4)
+        backend.set_prefill_mode("exact")
+        try:
+            assert not _run(backend, wz, x).any()
+        finally:
+            backend.set_prefill_mode("fast")
+        wz.free()
 
 
 def _node_reference(oracle, st, node, epi, edges, rows=None):
@@ -1468,6 +1502,30 @@ def test_first_call_of_a_kernel_may_sit_inside_a_capture(oracle):
         qw.free()
     finally:
         be.close()
+
+
+def test_read_pattern_probes_run(backend, oracle):
+    """The pure-read probes the benchmark records as ceilings: every pattern runs on the headline tensor's
+    K and on a ragged tensor (flat patterns), and the strip patterns refuse shapes they do not cover."""
+    q, s = _quant(oracle, 4, 272, 4096, cfg=61)
+    w = backend.upload_quantized(q, s, 4)
+    q2, s2 = _quant(oracle, 8, 40, 416, cfg=62)
+    w2 = backend.upload_quantized(q2, s2, 8)
+    xd = torch.zeros(8, dtype=torch.float16, device="cuda")            # (a plan wants edges; the probes read none)
+    yd = torch.zeros(8, dtype=torch.float32, device="cuda")
+    plan = backend.plan_many([w, w], [xd, xd], [yd, yd])
+    plan2 = backend.plan_many([w2], [xd], [yd])
+    for pattern in range(1, 7):
+        backend.debug_read_pattern(plan, pattern)
+    for pattern in (3, 4, 5, 6):
+        backend.debug_read_pattern(plan2, pattern)
+    torch.cuda.synchronize()
+    for pattern in (1, 2, 0, 7):
+        with pytest.raises(CybqError) as e:
+            backend.debug_read_pattern(plan2, pattern)
+        assert e.value.status == -7
+    w.free()
+    w2.free()
 
 
 def test_container_to_backend(backend, oracle, tmp_path):

@@ -58,3 +58,53 @@ def test_static_scratch_limits(backend, oracle):
     backend.matmul_static(qw, x[:4].contiguous(), y[:4])                     # decode rows: no limit
     torch.cuda.synchronize()
     qw.free()
+
+
+def test_static_entry_point_allocates_nothing(oracle):
+    """The property the entry point exists for: a call makes no device allocation.  On a fresh context a
+    512-row call on a long K (staging pass, multiply split four ways over K, slab adding: every user of
+    the scratch) is recorded into a HIP graph - an allocation during capture fails - and replayed against the
+    eager result; and the free device memory is the same before and after a run of eager calls."""
+    from cyb_amd import Backend
+    be = Backend(0)
+    try:
+        N, K, M = 4096, 14336, 512
+        q, s = oracle.quantize(synth.weights(79, N, K), 4)
+        qw = be.upload_quantized(q, s, 4)
+        x = torch.from_numpy(synth.activations(79, M, K)).cuda().to(torch.bfloat16)
+        x1 = x[:1].to(torch.float16).contiguous()
+        y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        y1 = torch.zeros((1, N), dtype=torch.float32, device="cuda")
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):           # first launches of these kernels on this context
+            st = torch.cuda.current_stream().cuda_stream
+            be.matmul_static(qw, x, y, stream=st)
+            be.matmul_static(qw, x1, y1, stream=st)
+        want, want1 = torch.empty_like(y), torch.empty_like(y1)
+        be.matmul(qw, x, want)
+        be.matmul(qw, x1, want1)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            y.zero_()
+            y1.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            err = ((y.double() - want.double()).norm() / want.double().norm()).item()
+            assert err < 2e-6, err
+            assert torch.equal(y1, want1)
+        rows = [0, 255, 511]
+        assert oracle.rel_l2(y[rows].cpu().numpy(), oracle.matmul_f64(q, s, x[rows].float().cpu().numpy())) < 5e-4
+        # eager calls: free device memory does not move
+        be.matmul_static(qw, x, y)
+        torch.cuda.synchronize()
+        free0 = torch.cuda.mem_get_info()[0]
+        for _ in range(5):
+            be.matmul_static(qw, x, y)
+            be.matmul_static(qw, x1, y1)
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free0
+        qw.free()
+    finally:
+        be.close()
