@@ -280,8 +280,23 @@ def main():
         ceilings[label] = {"us": round(cus, 3), "GB/s": round((alg_bytes if io else alg_w) / (t / ceil_n) / 1e9, 1),
                            "frac_of_hbm_peak": round((alg_bytes if io else alg_w) / (t / ceil_n) / 1e9 / HBM_PEAK_GBS, 4)}
         log(f"ceiling {label}: {cus:.2f} us")
-    ceilings["what"] = ("the one-row kernel's own memory requests (one workgroup per 16-row strip, whole strip requested "
-                        "up front) with no arithmetic; second line adds its activation read and its 57 KB of stores")
+    ceilings["what"] = ("the one-row kernel's own memory requests (one workgroup per 16-row strip, 8 waves x 4 tiles, whole strip "
+                        "requested up front) with no arithmetic; second line adds its activation read and its 57 KB of stores")
+    # the same bytes through other pure-read patterns (cybq_debug_read_pattern): what a launch that only reads
+    # the tensor takes on this box, whatever its decomposition
+    patterns = {1: "strip_per_workgroup_4_waves_x_2_sets", 2: "strip_per_workgroup_2_waves_x_4_sets",
+                3: "flat_8KiB_per_wave_one_round", 4: "persistent_grid_one_16_wave_workgroup_per_CU",
+                5: "persistent_grid_next_chunk_requested_ahead", 6: "flat_4KiB_per_wave_straight_into_LDS"}
+    other = {}
+    for pat, label in patterns.items():
+        walk(200, lambda p: be.debug_read_pattern(p, pat, stream))
+        t, _ = timer.until(lambda i: walk(ceil_n, lambda p: be.debug_read_pattern(p, pat, stream)))
+        other[label] = {"us": round(t / ceil_n * 1e6, 3), "frac_of_hbm_peak": round(alg_w / (t / ceil_n) / 1e9 / HBM_PEAK_GBS, 4)}
+        log(f"read pattern {label}: {t / ceil_n * 1e6:.2f} us")
+    ceilings["other_pure_read_patterns"] = other
+    best_read = min([ceilings["bare_read_of_the_weight_bytes"]["us"]] + [v["us"] for v in other.values()])
+    ceilings["best_pure_read_us"] = best_read
+    ceilings["kernel_over_best_pure_read"] = round(us / best_read, 4)
     ceilings["kernel_over_bare_read"] = round(us / ceilings["bare_read_of_the_weight_bytes"]["us"], 4)
     ceilings["kernel_over_read_with_io"] = round(us / ceilings["read_plus_x_load_and_y_store"]["us"], 4)
     # the same launches with exact integer weight operands (cybq_set_decode_mode EXACT)
@@ -399,10 +414,11 @@ def main():
         log("prefill rows sweep: " + " ".join(f"{k}:{v['us']}us" for k, v in rows_out.items()))
 
         # ---- batch sweep of the decode kernels on the same shape
-        def sweep_shape(wl, Kx, Nx, Ms, bitsx=bits):
+        def sweep_shape(wl, Kx, Nx, Ms, bitsx=bits, xdtype=torch.float16, roofline=False):
             out = {}
+            xsize = 4 if xdtype == torch.float32 else 2
             for Mb in Ms:
-                xb = torch.from_numpy(synth.activations(3, Mb, Kx, outliers=0.001)).to(dev).to(torch.float16)
+                xb = torch.from_numpy(synth.activations(3, Mb, Kx, outliers=0.001)).to(dev).to(xdtype)
                 yb = [torch.empty((Mb, Nx), dtype=torch.float32, device=dev)]
                 n = 240
                 cur = [0]
@@ -420,9 +436,19 @@ def main():
                 one(0)
                 t, _ = timer.until(one)
                 e = t / n
-                g = formats.matmul_bytes(bitsx, Nx, Kx, Mb, 2, 4) / e / 1e9
+                g = formats.matmul_bytes(bitsx, Nx, Kx, Mb, xsize, 4) / e / 1e9
                 out[f"M{Mb}"] = {"us": round(e * 1e6, 2), "GB/s": round(g, 1), "frac_of_hbm_peak": round(g / HBM_PEAK_GBS, 4)}
+                if roofline:
+                    out[f"M{Mb}"]["roofline"] = {"bound": "hbm", "achieved": round(g, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                                 "frac": round(g / HBM_PEAK_GBS, 4),
+                                                 "algorithmic_bytes": int(formats.matmul_bytes(bitsx, Nx, Kx, Mb, xsize, 4))}
             return out
+
+        def copies_of(q_, s_, bitsx):
+            """Device copies of one tensor, three times the last-level cache in all."""
+            n = max(2, (3 * MALL_BYTES) // formats.weight_bytes(bitsx, q_.shape[0], q_.shape[1]) + 1)
+            first = be.upload_quantized(q_, s_, bitsx)
+            return [first] + [first.clone() for _ in range(n - 1)]
 
         extra["decode_batch_sweep_4096x14336"] = sweep_shape(ws, K, N, (2, 4, 8, 16, 32))
         for t in ws[1:]:
@@ -447,6 +473,46 @@ def main():
         for t in w8:
             t.free()
         del w8
+
+        # ---- the BASELINE configs the lines above do not cover, each with its own roofline object
+        base = {}
+        # configs[0]: Q8 2048 x 2048, x f32, one row
+        q1, s1 = formats.quantize(synth.weights(1, 2048, 2048), formats.Q8)
+        w1 = copies_of(q1, s1, formats.Q8)
+        base["cfg0_q8_gemv_2048x2048_x_f32_M1"] = sweep_shape(w1, 2048, 2048, (1,), formats.Q8, torch.float32, True)["M1"]
+        for t in w1:
+            t.free()
+        del w1, q1, s1
+        # configs[1]: the two smaller decode shapes at one row
+        for Nx in (4096, 1024):
+            qs_, ss_ = formats.quantize(synth.weights(2, Nx, K), bits)
+            wsm = copies_of(qs_, ss_, bits)
+            base[f"cfg1_q4_gemv_4096x{Nx}_M1"] = sweep_shape(wsm, K, Nx, (1,), bits, torch.float16, True)["M1"]
+            for t in wsm:
+                t.free()
+            del wsm, qs_, ss_
+        # configs[3]: the down-projection shape of the prefill GEMM (K = 14336 -> N = 4096), bf16 rows
+        qd, sd = formats.quantize(synth.weights(6, K, N), bits)
+        wd = copies_of(qd, sd, bits)
+        for Mr in (128, 512, 2048):
+            xr = torch.from_numpy(synth.activations(4, Mr, N)).to(dev).to(torch.bfloat16)
+            yr = torch.empty((Mr, K), dtype=torch.float32, device=dev)
+            nr = 50 if Mr <= 512 else 12
+            rpl = be.plan_many([wd[j % len(wd)] for j in range(nr)], [xr] * nr, [yr] * nr)
+            be.matmul_many(rpl, Mr, stream)
+            tr, _ = timer.until(lambda i: be.matmul_many(rpl, Mr, stream), max_passes=40)
+            tr /= nr
+            tf = 2.0 * Mr * N * K / tr / 1e12
+            base[f"cfg3_q4_prefill_14336x4096_M{Mr}"] = {
+                "us": round(tr * 1e6, 1), "tflops": round(tf, 1),
+                "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                             "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "algorithmic_flops": int(2 * Mr * N * K)}}
+            del xr, yr, rpl
+        for t in wd:
+            t.free()
+        del wd, qd, sd
+        extra["baseline_configs_not_covered_above"] = base
+        log("other BASELINE configs: " + " ".join(f"{k}:{v['us']}us" for k, v in base.items()))
 
         # ---- LM head: 4096 -> 128256 (/root/reference/decide/pipeline.md:51), weights made on the device
         NL = 128256
@@ -526,33 +592,41 @@ def main():
                                  "frac_of_hbm_peak": round(st.step_bytes(Ms) / per / 1e9 / HBM_PEAK_GBS, 4),
                                  "linear_stack_tok_per_s": round(Ms / per, 1)}
                 log(f"decode stack {label} M={Ms}: {per * 1e6:.0f} us/step")
-                if shapes is not None and not epis:
-                    # what the epilogues replace: the same step with SwiGLU and the two residual adds as
-                    # launches of their own between the linears (plain torch ops on the same buffers)
-                    gu, res_o, res_d = edges["out.gate_up_proj"], edges["out.o_proj"], edges["out.down_proj"]
-                    h = gu.shape[1] // 2
-                    act = torch.empty((Ms, h), dtype=torch.float32, device=dev)
-                    r0 = torch.zeros_like(res_o)
+                if shapes is not None and not norms:
+                    # the same step recorded once into a HIP graph and replayed (no host work per launch)
+                    side = torch.cuda.Stream()
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph, stream=side):
+                        be.matmul_many(pl, Ms, torch.cuda.current_stream().cuda_stream)
+                    graph.replay()
+                    perg, _ = timer.until(lambda i: graph.replay())
+                    res[f"M{Ms}"]["us_per_step_replayed_from_a_hip_graph"] = round(perg * 1e6, 1)
+                    log(f"  ... replayed from a HIP graph: {perg * 1e6:.0f} us/step")
+                    del graph
+                if norms:
+                    # what the folded norms replace: the fused-epilogue step with the two RMSNorms of every layer as
+                    # launches of their own in front of qkv and gate/up.  Each is stood in for by ONE elementwise
+                    # launch with a norm's traffic (x and gamma in, x' out, no row reduction): a stand-alone norm
+                    # kernel costs at least that
+                    xin = edges["in.4096"]
+                    xn = torch.empty_like(xin)
+                    node_plans = []
+                    for i, n in enumerate(st.nodes):
+                        r = edges[f"res.{n.N}"] if st.epilogues[i] == "add" else None
+                        node_plans.append(be.plan_many([st.weights[i]], [xn if st.gammas[i] is not None else edges[n.x]],
+                                                       [edges[n.y]], [st.epilogues[i]], [r]))
 
-                    def step_with_elementwise():
-                        for layer in range(32):
-                            be.matmul_many(layer_plans[layer][0], Ms, stream)       # qkv, o
-                            torch.add(res_o, r0, out=res_o)
-                            be.matmul_many(layer_plans[layer][1], Ms, stream)       # gate_up
-                            torch.mul(torch.nn.functional.silu(gu[:, :h]), gu[:, h:], out=act)
-                            be.matmul_many(layer_plans[layer][2], Ms, stream)       # down
-                            torch.add(res_d, r0, out=res_d)
+                    def step_with_norm_launches():
+                        for i, npl in enumerate(node_plans):
+                            if st.gammas[i] is not None:
+                                torch.mul(xin, st.gammas[i], out=xn)
+                            be.matmul_many(npl, Ms, stream)
 
-                    xs_all, ys_all = [edges[n.x] for n in st.nodes], [edges[n.y] for n in st.nodes]
-                    layer_plans = []
-                    for layer in range(32):
-                        b0 = layer * 4
-                        layer_plans.append([be.plan_many(st.weights[b0 + a:b0 + b], xs_all[b0 + a:b0 + b], ys_all[b0 + a:b0 + b])
-                                            for a, b in ((0, 2), (2, 3), (3, 4))])
-                    step_with_elementwise()
-                    per2, _ = timer.until(lambda i: step_with_elementwise())
-                    res[f"M{Ms}"]["us_per_step_with_swiglu_and_residual_as_separate_launches"] = round(per2 * 1e6, 1)
-                    log(f"  ... with SwiGLU / residual adds as separate launches: {per2 * 1e6:.0f} us/step")
+                    step_with_norm_launches()
+                    per3, _ = timer.until(lambda i: step_with_norm_launches())
+                    res[f"M{Ms}"]["us_per_step_with_the_two_rmsnorms_as_separate_launches"] = round(per3 * 1e6, 1)
+                    log(f"  ... with the RMSNorms as separate launches: {per3 * 1e6:.0f} us/step")
+                    del node_plans
             if shapes is not None and not epis:
                 # prefill of one 512-token chunk through the same stack (bf16 activations), and both
                 # phases in the units the reference's UI reports (tok_in_s / tok_out_s,

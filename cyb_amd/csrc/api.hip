@@ -263,6 +263,13 @@ int cybq_init(int device, cybq_ctx** out)
         delete ctx;
         return CYBQ_ERR_NOMEM;
     }
+    // the decode kernels' tickets (start of the scratch's tail) are zero at rest
+    if (hipMemset(static_cast<char*>(ctx->workspace) + ctx->workspace_bytes - cybq::kDecodeScratchBytes, 0, (size_t)1 << 16) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipFree(ctx->workspace);
+        delete ctx;
+        return CYBQ_ERR_HIP;
+    }
     *out = ctx;
     return CYBQ_OK;
 }
@@ -449,8 +456,16 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
     hipStream_t st = static_cast<hipStream_t>(stream);
     cybq::WeightView v = view_of(w);
     hipError_t e;
+    // the tail of the scratch belongs to the decode kernels (tickets and slabs of a K split), the rest to prefill
+    void* dscr = nullptr;
+    size_t dscr_bytes = 0;
+    if (workspace && workspace_bytes > 2 * cybq::kDecodeScratchBytes) {
+        workspace_bytes -= cybq::kDecodeScratchBytes;
+        dscr = static_cast<char*>(workspace) + workspace_bytes;
+        dscr_bytes = cybq::kDecodeScratchBytes;
+    }
     if (M <= 16 || (M <= 32 && cybq::gemv_serves_32((int)xdt, (int)M, epi))) {
-        e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->decode_exact, epi, st);
+        e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->decode_exact, epi, dscr, dscr_bytes, st);
     } else if (M <= 64 && (int64_t)w->N * w->K <= (int64_t)6144 * 4096 && cybq::gemv_serves_32((int)xdt, 32, epi)) {
         // 33..64 rows on a small weight (up to 4096 -> 6144): the MFMA kernel would split K over
         // workgroups and add the slabs in a second pass; two passes of the batched-rows decode kernel
@@ -462,10 +477,10 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
         const size_t yoff = (size_t)32 * n_out * dtype_size(ydt);
         cybq::Epilogue ec = epi;
         if (epi.kind == cybq::kEpiAdd) ec.residual = static_cast<const char*>(residual) + yoff;
-        e = cybq::launch_gemv(v, x, xdt, 32, y, ydt, ctx->num_cus, exact_ops, epi, st);
+        e = cybq::launch_gemv(v, x, xdt, 32, y, ydt, ctx->num_cus, exact_ops, epi, dscr, dscr_bytes, st);
         if (e == hipSuccess)
             e = cybq::launch_gemv(v, static_cast<const char*>(x) + (size_t)32 * w->K * dtype_size(xdt), xdt, (int)M - 32,
-                                  static_cast<char*>(y) + yoff, ydt, ctx->num_cus, exact_ops, ec, st);
+                                  static_cast<char*>(y) + yoff, ydt, ctx->num_cus, exact_ops, ec, dscr, dscr_bytes, st);
     } else if (!weight_is_wide(w) && (xdt == CYBQ_F32 ? !ctx->prefill_exact : M > 32)) {
         e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, workspace, workspace_bytes,
                               epi, st);
@@ -488,7 +503,7 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
             const size_t yoff = (size_t)m0 * n_out * dtype_size(ydt);
             cybq::Epilogue ec = epi;
             if (epi.kind == cybq::kEpiAdd) ec.residual = static_cast<const char*>(residual) + yoff;
-            e = cybq::launch_gemv(v, xp, xdt, mm, static_cast<char*>(y) + yoff, ydt, ctx->num_cus, ctx->decode_exact, ec, st);
+            e = cybq::launch_gemv(v, xp, xdt, mm, static_cast<char*>(y) + yoff, ydt, ctx->num_cus, ctx->decode_exact, ec, dscr, dscr_bytes, st);
         }
     }
     if (e != hipSuccess) return fail_hip(ctx, e, "matmul launch");

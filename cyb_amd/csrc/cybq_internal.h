@@ -24,8 +24,12 @@ hipError_t launch_dequant(const WeightView& w, float* out, hipStream_t st);
 bool gemv_serves_32(int xdt, int M, const Epilogue& epi);
 // exact_operands: keep the weight operands exact integers for one and two f16 rows too (the LDS
 // kernel) instead of the subnormal-operand kernel of gemv1.hip
+// scratch: device memory the batched-rows kernel may use when it splits K over workgroups (few strips, a
+// long K): a ticket word per strip group at its start - zero at rest - and the slabs of partial sums behind
+// them; nullptr = never split.  Calls that share it must not overlap.
+constexpr size_t kDecodeScratchBytes = (size_t)8 << 20;
 hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
-                       int num_cus, bool exact_operands, const Epilogue& epi, hipStream_t st);
+                       int num_cus, bool exact_operands, const Epilogue& epi, void* scratch, size_t scratch_bytes, hipStream_t st);
 // decode kernel for one and two rows (f16 / bf16 activations, no folded norm): weight operands are f16 subnormals
 // (bf16: 128 + u),
 // the +8 / +128 bias comes off inside the MFMA accumulation (gemv1.hip)

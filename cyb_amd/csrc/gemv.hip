@@ -652,13 +652,22 @@ __device__ __forceinline__ void norm_piece(u32x4_t& v, const GammaPiece& gp, boo
 // 4u * 2^-24 / 64u * 2^-24 (six vector instructions per eight weights instead of nine), the bias comes off
 // through the MFMA's C operand like with bf16 activations, 1/16 for the odd groups rides on their scale
 // and 2^22 on the final sums.
-template <int BITS, int XMODE, int TS, int NS, bool NORM, int XR, int MB = 1, bool SUB = false>
+// KS: K is split over `splits` workgroups per strip group (few strips and a long K: with one workgroup per
+// strip every CU pulls all of x out of the L2, M x K x 2 bytes against its 37 KB x strips of weights).  Workgroup
+// (group, split) walks the K tiles [split * kt_per_split, ...) of the group's NS strips and leaves its sums in
+// its slab of `slabs`; a ticket per group tells the workgroup that arrives last, which adds the slabs in split
+// order - a fixed order whoever arrives when - and writes y.  Slabs and ticket travel past the caches (stores
+// and loads at system scope, waited for before the ticket is taken): nothing is flushed, nothing invalidated.
+// The ticket is left at zero again for the next launch; launches that share `slabs` must not overlap.
+template <int BITS, int XMODE, int TS, int NS, bool NORM, int XR, int MB = 1, bool SUB = false, bool KS = false>
 // (waves_per_eu: the scheduler would otherwise trade the up-front loads for occupancy)
 __global__ __launch_bounds__((TS <= 2 && MB == 1 && !NORM) ? 1024 : 512)
 __attribute__((amdgpu_waves_per_eu(2, (TS <= 2 && MB == 1 && !NORM) ? 4 : 2)))
 void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restrict__ x, const void* __restrict__ gamma, int KT_, int K,
-                      int NT, int M, int nwaves, int gamma_dt, int N, void* __restrict__ y, int ydt, Epilogue epi)
+                      int NT, int M, int nwaves, int gamma_dt, int N, void* __restrict__ y, int ydt, Epilogue epi, int splits,
+                      int kt_per_split, float* __restrict__ slabs, unsigned* __restrict__ tickets)
 {
+    static_assert(!KS || !NORM, "the K split has no folded-norm form");
     const WeightView w = {wbase, N, K, NT, KT_, BITS};
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t magic = (BITS == 4 && XMODE == XBF16) ? q4_magic_vgpr_bf16() : q4_magic_vgpr();
@@ -666,8 +675,15 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
     const int lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int oct = lane >> 4;
-    const int strip0 = blockIdx.x * NS;
-    const int KT = w.KT;
+    int group = blockIdx.x, split = 0, kt_lo = 0;
+    int KT = w.KT;                                   // K tiles this workgroup walks: [kt_lo, kt_lo + KT)
+    if constexpr (KS) {
+        group = (int)blockIdx.x / splits;
+        split = (int)blockIdx.x - group * splits;
+        kt_lo = split * kt_per_split;
+        KT = min(kt_per_split, w.KT - kt_lo);
+    }
+    const int strip0 = group * NS;
     // x is read the way memory likes it - one load instruction covers XR rows (the batch rounded
     // up to 4, 8 or 16) x P = 64 / XR neighbouring 16 B pieces, lane l takes piece l % P of row
     // l / P - and then moved across lanes into MFMA A-operand order (lane l: row l%16, k octet
@@ -702,7 +718,7 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
 
     int64_t sbase[NS];
 #pragma unroll
-    for (int s = 0; s < NS; s++) sbase[s] = (int64_t)min(strip0 + s, w.NT - 1) * KT;
+    for (int s = 0; s < NS; s++) sbase[s] = (int64_t)min(strip0 + s, w.NT - 1) * w.KT;
 
     for (int slab0 = 0; slab0 < KT; slab0 += nwaves * TS) {
         // my K tiles of this slab and their x operands (clamped past the end; such tiles get scale 0)
@@ -714,7 +730,7 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
         for (int u = 0; u < TS; u++) {
             const int t = slab0 + wv + nwaves * u;
             valid[u] = t < KT;
-            kt[u] = min(t, KT - 1);
+            kt[u] = kt_lo + min(t, KT - 1);
             if (NORM)
                 graw[u] = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const uint8_t*>(gamma) +
                                                             ((size_t)min(kt[u] * kTileK + g_first, w.K - g_count) << g_shift));
@@ -974,6 +990,45 @@ void gemv_rows_kernel(const uint8_t* __restrict__ wbase, const uint16_t* __restr
         }
         return;
     }
+    if constexpr (KS) {
+        constexpr int OUTS = NS * MB * 4;                 // output registers of a workgroup, 64 lanes each
+        const int groups = (int)gridDim.x / splits;
+        float* mine = slabs + ((size_t)split * groups + group) * (OUTS * 64);
+        for (int p = wv; p < OUTS; p += nwaves) {
+            const int r = p & 3, sb = p >> 2;
+            const float v = sum_partials(red + (sb * nwaves * 4 + r) * 64 + lane, nwaves, 4 * 64) * rstd[r];
+            __hip_atomic_store(mine + p * 64 + lane, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // my part of the slab has reached memory
+        __syncthreads();                                          // (and everybody is done reading `red`)
+        unsigned* flag = reinterpret_cast<unsigned*>(red);
+        if (tid == 0) {
+            const unsigned old = __hip_atomic_fetch_add(tickets + group, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const bool last = old + 1u == (unsigned)splits;
+            if (last) __hip_atomic_store(tickets + group, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *flag = last ? 1u : 0u;
+        }
+        __syncthreads();
+        if (*flag == 0u) return;
+        const size_t slab_stride = (size_t)groups * (OUTS * 64);
+        const float* first = slabs + (size_t)group * (OUTS * 64);
+        for (int p = wv; p < OUTS; p += nwaves) {
+            const int r = p & 3, b = (p >> 2) % MB, s = (p >> 2) / MB;
+            float part[4];                                 // (at most four splits: rows_split_plan)
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                part[k] = __hip_atomic_load(first + (size_t)min(k, splits - 1) * slab_stride + p * 64 + lane, __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_SYSTEM);
+            float v = part[0];
+#pragma unroll
+            for (int k = 1; k < 4; k++) v += k < splits ? part[k] : 0.f;
+            const int nt = strip0 + s;
+            const int n = nt * 16 + (lane & 15);
+            const int m = 16 * b + 4 * oct + r;
+            if (nt < w.NT && m < M && n < w.N) emit(y, ydt, epi, (int64_t)m * w.N + n, v);
+        }
+        return;
+    }
     for (int p = wv; p < NS * MB * 4; p += nwaves) {
         const int r = p & 3, b = (p >> 2) % MB, s = (p >> 2) / MB;
         const int nt = strip0 + s;
@@ -997,7 +1052,7 @@ hipError_t launch_rows_x(const WeightView& w, const void* x, int M, void* y, int
             (void)LdsRequest<&gemv_rows_kernel<BITS, XMODE, TS, NS, true, XR>, 150 * 1024>::registered;
             if (lds > 150 * 1024) return hipErrorInvalidValue;
             hipLaunchKernelGGL(kern, dim3(groups), dim3(nwaves * 64), lds, st, w.base, reinterpret_cast<const uint16_t*>(x), epi.gamma,
-                               w.KT, w.K, w.NT, M, nwaves, epi.gamma_dt, w.N, y, ydt, epi);
+                               w.KT, w.K, w.NT, M, nwaves, epi.gamma_dt, w.N, y, ydt, epi, 1, 0, nullptr, nullptr);
             return hipGetLastError();
         }
     }
@@ -1009,7 +1064,8 @@ hipError_t launch_rows_x(const WeightView& w, const void* x, int M, void* y, int
             if constexpr (NS * MB * 8 * 1024 + 512 > 64 * 1024)
                 (void)LdsRequest<&gemv_rows_kernel<BITS, XMODE, TS, NS, false, XR, MB, true>, 150 * 1024>::registered;
             hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS, false, XR, MB, true>), dim3(groups), dim3(nwaves * 64), lds, st,
-                               w.base, reinterpret_cast<const uint16_t*>(x), nullptr, w.KT, w.K, w.NT, M, nwaves, 0, w.N, y, ydt, epi);
+                               w.base, reinterpret_cast<const uint16_t*>(x), nullptr, w.KT, w.K, w.NT, M, nwaves, 0, w.N, y, ydt, epi, 1, 0, nullptr,
+                               nullptr);
             return hipGetLastError();
         }
     }
@@ -1017,8 +1073,68 @@ hipError_t launch_rows_x(const WeightView& w, const void* x, int M, void* y, int
     if constexpr (NS * MB * 8 * 1024 + 512 > 64 * 1024)
         (void)LdsRequest<&gemv_rows_kernel<BITS, XMODE, TS, NS, false, XR, MB>, 150 * 1024>::registered;
     hipLaunchKernelGGL((gemv_rows_kernel<BITS, XMODE, TS, NS, false, XR, MB>), dim3(groups), dim3(nwaves * 64), lds, st, w.base,
-                       reinterpret_cast<const uint16_t*>(x), nullptr, w.KT, w.K, w.NT, M, nwaves, 0, w.N, y, ydt, epi);
+                       reinterpret_cast<const uint16_t*>(x), nullptr, w.KT, w.K, w.NT, M, nwaves, 0, w.N, y, ydt, epi, 1, 0, nullptr, nullptr);
     return hipGetLastError();
+}
+
+// Few strips and a long K (the down projection): four strips per workgroup, K split four ways over
+// workgroups, the slabs added by the workgroup that arrives last (gemv_rows_kernel, KS).
+struct SplitPlan {
+    int splits, kt_per_split, nwaves, groups;
+};
+
+constexpr int kSplitStrips = 4, kSplitWays = 4;
+
+bool rows_split_plan(const WeightView& w, int xdt, int M, int num_cus, const Epilogue& epi, size_t scratch_bytes, SplitPlan& sp)
+{
+    if (w.bits != 4 || xdt == kF32 || epi.gamma || epi.kind == kEpiSwiglu) return false;
+    // a long K and about one strip per CU (14336 -> 4096 on 256 CUs: 12.6 against 13.9 us at 16 rows, 17.4 against
+    // 21.5 at 32; with K = 11008 or a quarter of the strips the split only costs: its slabs and ticket add 2.5 - 3 us)
+    if (w.KT < 96 || (int64_t)w.NT * 2 > (int64_t)num_cus * 3 || (int64_t)w.NT * 4 < (int64_t)num_cus * 3) return false;
+    sp.splits = kSplitWays;
+    sp.kt_per_split = (w.KT + sp.splits - 1) / sp.splits;
+    sp.splits = (w.KT + sp.kt_per_split - 1) / sp.kt_per_split;                         // no empty split
+    sp.nwaves = min(8, (sp.kt_per_split + 3) / 4);
+    sp.groups = (w.NT + kSplitStrips - 1) / kSplitStrips;
+    const size_t need = (size_t)sp.splits * sp.groups * (kSplitStrips * 2 * 4 * 64) * sizeof(float) + (size_t)sp.groups * sizeof(unsigned) + 256;
+    return sp.splits > 1 && sp.splits <= 4 && sp.groups * sizeof(unsigned) <= ((size_t)1 << 16) && need <= scratch_bytes;
+}
+
+template <int XMODE, int XR, int MB>
+hipError_t launch_rows_split_x(const WeightView& w, const void* x, int M, void* y, int ydt, const Epilogue& epi, bool sub,
+                               const SplitPlan& sp, void* scratch, hipStream_t st)
+{
+    constexpr int NS = kSplitStrips, TS = MB == 1 ? 4 : 2;
+    // tickets first (one word per group, zero at rest), slabs behind them
+    unsigned* tickets = reinterpret_cast<unsigned*>(scratch);
+    float* slabs = reinterpret_cast<float*>(static_cast<char*>(scratch) + (((size_t)sp.groups * sizeof(unsigned) + 255) & ~(size_t)255));
+    const size_t lds = (size_t)NS * MB * sp.nwaves * 4 * 64 * sizeof(float) + 8 * 16 * sizeof(float);
+    const dim3 grid((unsigned)(sp.groups * sp.splits)), block((unsigned)sp.nwaves * 64);
+    const uint16_t* xp = reinterpret_cast<const uint16_t*>(x);
+    if constexpr (XMODE == XF16) {
+        if (sub) {
+            if constexpr (NS * MB * 8 * 1024 + 512 > 64 * 1024)
+                (void)LdsRequest<&gemv_rows_kernel<4, XMODE, TS, NS, false, XR, MB, true, true>, 150 * 1024>::registered;
+            hipLaunchKernelGGL((gemv_rows_kernel<4, XMODE, TS, NS, false, XR, MB, true, true>), grid, block, lds, st, w.base, xp, nullptr, w.KT,
+                               w.K, w.NT, M, sp.nwaves, 0, w.N, y, ydt, epi, sp.splits, sp.kt_per_split, slabs, tickets);
+            return hipGetLastError();
+        }
+    }
+    if constexpr (NS * MB * 8 * 1024 + 512 > 64 * 1024)
+        (void)LdsRequest<&gemv_rows_kernel<4, XMODE, TS, NS, false, XR, MB, false, true>, 150 * 1024>::registered;
+    hipLaunchKernelGGL((gemv_rows_kernel<4, XMODE, TS, NS, false, XR, MB, false, true>), grid, block, lds, st, w.base, xp, nullptr, w.KT, w.K,
+                       w.NT, M, sp.nwaves, 0, w.N, y, ydt, epi, sp.splits, sp.kt_per_split, slabs, tickets);
+    return hipGetLastError();
+}
+
+template <int XMODE>
+hipError_t launch_rows_split(const WeightView& w, const void* x, int M, void* y, int ydt, const Epilogue& epi, bool sub,
+                             const SplitPlan& sp, void* scratch, hipStream_t st)
+{
+    if (M > 16) return launch_rows_split_x<XMODE, 16, 2>(w, x, M, y, ydt, epi, sub, sp, scratch, st);
+    if (M <= 4) return launch_rows_split_x<XMODE, 4, 1>(w, x, M, y, ydt, epi, sub, sp, scratch, st);
+    if (M <= 8) return launch_rows_split_x<XMODE, 8, 1>(w, x, M, y, ydt, epi, sub, sp, scratch, st);
+    return launch_rows_split_x<XMODE, 16, 1>(w, x, M, y, ydt, epi, sub, sp, scratch, st);
 }
 
 // (the x load pattern follows the batch: up to 4, up to 8, up to 16 rows per load)
@@ -1105,6 +1221,7 @@ hipError_t launch_rows2(const WeightView& w, const void* x, int M, void* y, int 
 }
 
 int g_tune_waves = 0, g_tune_unroll = 0, g_tune_rows = 0;
+constexpr int kSplitMinRows = 12;
 
 constexpr int kLdsBudget = 64 * 1024;      // what a slab of x aims for
 constexpr int kLdsCap = 150 * 1024;         // what a launch may ask for
@@ -1181,7 +1298,7 @@ hipError_t launch_u(const WeightView& w, const void* x, int M, void* y, int ydt,
 void set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll)
 {
     g_tune_waves = waves_per_group;
-    g_tune_rows = rows_kernel;       // 0 automatic, 1 always the register kernel, 2 never
+    g_tune_rows = rows_kernel;       // 0 automatic, 1 always the register kernel, 2 never, 3 / 4: always, K split never / whenever it applies
     g_tune_unroll = unroll;
 }
 
@@ -1192,7 +1309,7 @@ bool gemv_serves_32(int xdt, int M, const Epilogue& epi)
 }
 
 hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
-                       int num_cus, bool exact_operands, const Epilogue& epi, hipStream_t st)
+                       int num_cus, bool exact_operands, const Epilogue& epi, void* scratch, size_t scratch_bytes, hipStream_t st)
 {
     // Waves per workgroup (= split of a strip's K tiles).  Depends on the weight
     // shape only, never on M, so that the summation order is the same for every
@@ -1228,9 +1345,17 @@ hipError_t launch_gemv(const WeightView& w, const void* x, int xdt, int M, void*
     // (Q8 on wide outputs: up to four rows the LDS kernel is still the quicker one, 24.0 against
     // 27.6 us at 4096 -> 28672)
     const bool wide_q8 = w.bits == 8 && (w.NT + num_cus / 2) / num_cus >= 3;
-    const bool rows_kernel = g_tune_rows == 1 || (g_tune_rows == 0 && M >= (wide_q8 ? 5 : 3));
+    const bool rows_kernel = g_tune_rows == 1 || g_tune_rows >= 3 || (g_tune_rows == 0 && M >= (wide_q8 ? 5 : 3));
+    if (M > 16 && !gemv_serves_32(xdt, M, epi)) return hipErrorInvalidValue;
+    // few strips, a long K, twelve rows or more: K split over workgroups (tuning 3: never, 4: from three rows on)
+    if (rows_kernel && xdt != kF32 && scratch && g_tune_rows != 3 && g_tune_waves == 0 && (M >= kSplitMinRows || g_tune_rows == 4)) {
+        SplitPlan sp;
+        if (rows_split_plan(w, xdt, M, num_cus, epi, scratch_bytes, sp)) {
+            if (xdt == kF16) return launch_rows_split<XF16>(w, x, M, y, ydt, epi, !exact_operands, sp, scratch, st);
+            return launch_rows_split<XBF16>(w, x, M, y, ydt, epi, !exact_operands, sp, scratch, st);
+        }
+    }
     if (M > 16) {
-        if (!gemv_serves_32(xdt, M, epi)) return hipErrorInvalidValue;
         if (w.bits == 4) {
             if (xdt == kF16) return launch_rows2<4, XF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, !exact_operands, st);
             return launch_rows2<4, XBF16>(w, x, M, y, ydt, g_tune_waves, num_cus, epi, !exact_operands, st);

@@ -253,6 +253,64 @@ def test_decode_modes_in_the_batched_rows_kernel(backend, oracle, N):
         backend.set_decode_mode("stream")
 
 
+@pytest.mark.parametrize("xdt", ["f16", "bf16"])
+def test_decode_long_k_split_over_workgroups(backend, oracle, xdt):
+    """About one strip per CU and a long K: from twelve rows on the batched-rows kernel splits K four ways over
+    workgroups, partial sums meet in slabs and the workgroup that arrives last adds them in split order.
+    Ragged N (a last strip of 8 rows, a strip group of one strip) and a K whose tiles do not divide by four;
+    against float64, run to run (the ticket is back at zero), across batch sizes, with the residual epilogue,
+    with exact operands, and against the kernel without the split."""
+    N, K = 193 * 16 - 8, 97 * 128
+    q, s = _quant(oracle, 4, N, K, cfg=45)
+    qw = backend.upload_quantized(q, s, 4)
+    wd = torch.from_numpy(oracle.dequant(q, s)).cuda().double()
+    x = _x(32, K, xdt, cfg=46)
+    ref = x.double() @ wd.T
+    try:
+        y32 = _run(backend, qw, x)
+        assert ((y32.double() - ref).norm() / ref.norm()).item() < TIGHT
+        for _ in range(3):
+            assert torch.equal(_run(backend, qw, x), y32)
+        for M in (12, 16, 17, 24):                       # one and two row blocks: a row keeps its bits
+            assert torch.equal(_run(backend, qw, x[:M].contiguous()), y32[:M]), M
+        backend.set_gemv_tuning(0, 4, 0)                 # the split from three rows on (the narrower x load patterns)
+        for M in (3, 5, 8):
+            assert torch.equal(_run(backend, qw, x[:M].contiguous()), y32[:M]), M
+        backend.set_gemv_tuning(0, 3, 0)                 # never split: another order of summation, the same sums
+        y_plain = _run(backend, qw, x)
+        assert not torch.equal(y_plain, y32)
+        assert ((y_plain.double() - y32.double()).norm() / ref.norm()).item() < 2e-6
+        backend.set_gemv_tuning(0, 0, 0)
+        r = torch.from_numpy(synth.activations(47, 32, N)).cuda()
+        ya = torch.empty((32, N), dtype=torch.float32, device="cuda")
+        backend.matmul_ex(qw, x, ya, "add", r)
+        torch.cuda.synchronize()
+        assert torch.equal(ya, y32 + r)
+        for ydt in ("f16", "bf16"):
+            assert torch.equal(_run(backend, qw, x, ydt), y32.to(TDT[ydt]))
+        backend.set_decode_mode("exact")
+        ye = _run(backend, qw, x[:16].contiguous())
+        assert ((ye.double() - ref[:16]).norm() / ref[:16].norm()).item() < (1e-6 if xdt == "f16" else TIGHT)
+        # recorded into a graph (no allocation, no memset: the ticket resets itself) and replayed
+        backend.set_decode_mode("stream")
+        yg = torch.zeros((32, N), dtype=torch.float32, device="cuda")
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            backend.matmul(qw, x, yg, stream=torch.cuda.current_stream().cuda_stream)
+        for _ in range(3):
+            yg.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(yg, y32)
+            assert torch.equal(_run(backend, qw, x), y32)            # eager calls between the replays
+    finally:
+        backend.set_gemv_tuning(0, 0, 0)
+        backend.set_decode_mode("stream")
+    qw.free()
+
+
 def test_decode_long_k_uses_several_slabs(backend, oracle):
     # M * K * 2 B exceeds the kernel's LDS budget: x is staged slab by slab
     N, K = 64, 14336
