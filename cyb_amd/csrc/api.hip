@@ -104,7 +104,14 @@ int fail_hip(cybq_ctx* ctx, hipError_t e, const char* where)
 // devices inside one process.
 struct DeviceGuard {
     hipError_t err;
-    explicit DeviceGuard(int device) : err(hipSetDevice(device)) {}
+    // (asking for the current device is a thread-local read; setting it again is not free, and a decode
+    // launch is a few microseconds of host time in all)
+    explicit DeviceGuard(int device)
+    {
+        int cur = -1;
+        err = hipGetDevice(&cur);
+        if (err != hipSuccess || cur != device) err = hipSetDevice(device);
+    }
 };
 
 cybq::WeightView view_of(const cybq_weight* w)

@@ -950,16 +950,16 @@ __global__ __launch_bounds__(256) void stage_x_kernel(const u32x4_t* __restrict_
 }
 
 // The same restaging for FAST mode when the activations are not f16 (bf16 or fp32 in, f16 operands
-// out), with a power-of-two scale PER ROW: a workgroup owns four rows, wave r owns row r.  First
-// the wave reads its row for the largest magnitude (of x, or of x * gamma with a folded norm,
-// whose sum of squares it also takes), picks the power of two s that brings it just under 2^14 and
-// leaves 1 / s in `unscale` for the multiply's epilogue; then the four rows go through LDS in
-// pieces of 512 k, every value multiplied by its row's s on the way to f16, and leave as 64-byte
-// runs (four neighbouring rows of one k octet in operand order).
+// out), with a power-of-two scale PER ROW: a workgroup owns four rows.  First a row is read for the
+// largest magnitude (of x, or of x * gamma with a folded norm, whose sum of squares is also taken),
+// which picks the power of two s that brings it just under 2^14 and leaves 1 / s in `unscale` for
+// the multiply's epilogue; then the four rows go through LDS in pieces of 512 k, every value
+// multiplied by its row's s on the way to f16, and leave as 64-byte runs (four neighbouring rows of
+// one k octet in operand order).
 // Whatever the magnitude of a row, its largest element lands in [2^13, 2^14) and elements down to
-// 2^-27 of it stay normal f16 numbers.  Rows of up to CH * 512 elements stay in registers between
-// the two steps (CH chunks of 8 values per lane, all requested at once); longer rows are read
-// again, CH chunks at a time (the second read hits the L2).
+// 2^-27 of it stay normal f16 numbers.  Rows of up to 4 * CH * 512 elements stay in registers
+// between the two steps (CH chunks of 8 values per lane in each of a row's four waves, all requested
+// at once); longer rows are read again (the second read hits the L2).
 template <int XT>
 struct RowChunk {                 // 8 consecutive activations of a row as loaded
     u32x4_t v[XT == 2 ? 2 : 1];
@@ -994,30 +994,42 @@ __device__ __forceinline__ void row_chunk_values(const RowChunk<XT>& c, float v[
     }
 }
 
+// A workgroup owns four rows and gives every row four waves: wave (r, p) takes the pieces of 512 k
+// numbered p, p + 4, ... of row r (CH of them at most stay in registers between the two steps), the
+// four parts of a row meet once through LDS for the row's largest magnitude (and sum of squares, added
+// in part order).  One wave per row took 5 - 7 us for 512 rows of 4096 and 10 - 12 us for rows of 14336,
+// most of it the latency of one wave walking its row.
 template <int XT, bool NORM, int CH>
-__global__ __launch_bounds__(256) void stage_rows_kernel(const void* __restrict__ src, u32x4_t* __restrict__ dst, int M, int K,
-                                                         Epilogue epi, float* __restrict__ ssq, float* __restrict__ unscale)
+__global__ __launch_bounds__(1024) void stage_rows_kernel(const void* __restrict__ src, u32x4_t* __restrict__ dst, int M, int K,
+                                                          Epilogue epi, float* __restrict__ ssq, float* __restrict__ unscale)
 {
     static_assert(XT == 1 || XT == 2, "bf16 or fp32 activations");
-    __shared__ u32x4_t tile[2][4 * kStagePitch];
+    constexpr int PW = 4;                                      // waves per row
+    __shared__ u32x4_t tile[PW][2][4 * kStagePitch];
+    __shared__ float amax_part[4][PW], sq_part[4][PW];
     const int rb = blockIdx.x >> 2, r0 = (blockIdx.x & 3) * 4;          // row block, first of this workgroup's rows in it
-    const int t = threadIdx.x, lane = t & 63, r = t >> 6;
+    const int t = threadIdx.x, lane = t & 63, wv = t >> 6;
+    const int r = wv & 3, part = wv >> 2;                               // my row of the four, my part of the row
     const int64_t row = min(rb * 16 + r0 + r, M - 1);      // (rows past M repeat the last one and are never read back)
     const int K8 = K >> 3, G = K8 >> 2;
-    const bool resident = K8 <= 64 * CH;
+    const int pieces = (K8 + 63) >> 6;                     // pieces of 64 chunks (512 k) in a row
+    const bool resident = pieces <= PW * CH;
 
     // ---- the row's largest magnitude (and sum of squares)
     RowChunk<XT> keep[CH];
     float amax = 0.f, sq = 0.f;
-    for (int c0 = 0; c0 < K8; c0 += 64 * CH) {
-#pragma unroll
-        for (int i = 0; i < CH; i++)
-            if (c0 + i * 64 < K8) keep[i] = load_row_chunk<XT>(src, row, K, min(c0 + i * 64 + lane, K8 - 1));
+    for (int p0 = 0; p0 < pieces; p0 += PW * CH) {
 #pragma unroll
         for (int i = 0; i < CH; i++) {
-            const int c = c0 + i * 64 + lane;
+            const int piece = p0 + i * PW + part;
+            if (piece < pieces) keep[i] = load_row_chunk<XT>(src, row, K, min(piece * 64 + lane, K8 - 1));
+        }
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const int piece = p0 + i * PW + part;
+            const int c = piece * 64 + lane;
             float v[8];
-            if (c < K8) {
+            if (piece < pieces && c < K8) {
                 row_chunk_values<XT>(keep[i], v);
                 if (NORM) {
                     float g[8];
@@ -1038,6 +1050,13 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void* __restrict_
         amax = fmaxf(amax, __shfl_xor(amax, off, 64));
         if (NORM) sq += __shfl_xor(sq, off, 64);
     }
+    if (lane == 0) {
+        amax_part[r][part] = amax;
+        if (NORM) sq_part[r][part] = sq;
+    }
+    __syncthreads();
+    amax = fmaxf(fmaxf(amax_part[r][0], amax_part[r][1]), fmaxf(amax_part[r][2], amax_part[r][3]));
+    if (NORM) sq = ((sq_part[r][0] + sq_part[r][1]) + sq_part[r][2]) + sq_part[r][3];
     // amax = f * 2^e with f in [0.5, 1): s = 2^(14 - e) puts it in [2^13, 2^14); zero, Inf and NaN rows keep s = 1
     float s = 1.0f;
     if (amax > 0.f && amax < __builtin_inff()) {
@@ -1045,12 +1064,12 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void* __restrict_
         (void)frexpf(amax, &e);
         s = ldexpf(1.0f, min(14 - e, 126));        // (rows below 2^-112: 2^126 keeps s and 1 / s normal numbers)
     }
-    if (lane == 0 && rb * 16 + r0 + r < M) {
+    if (lane == 0 && part == 0 && rb * 16 + r0 + r < M) {
         unscale[row] = 1.0f / s;
         if (NORM) ssq[row] = sq;
     }
 
-    // ---- scale, round to f16, through LDS into operand order (two tiles: one barrier per piece)
+    // ---- scale, round to f16, through LDS into operand order (two tiles per part: one barrier per piece)
     auto convert = [&](const RowChunk<XT>& ch, int c) {
         float v[8];
         row_chunk_values<XT>(ch, v);
@@ -1068,24 +1087,27 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void* __restrict_
         }
         return a.u;
     };
-    const int gl = t >> 4, oct = (t >> 2) & 3, rr = t & 3;  // when writing out: group within the piece, k octet, row
-    int piece = 0;
-    for (int c0 = 0; c0 < K8; c0 += 64 * CH) {
+    const int tp = r * 64 + lane;                           // my place among the 256 threads of my part
+    const int gl = tp >> 4, oct = (tp >> 2) & 3, rr = tp & 3;  // when writing out: group within the piece, k octet, row
+    int round = 0;
+    for (int p0 = 0; p0 < pieces; p0 += PW * CH) {
         if (!resident) {
 #pragma unroll
-            for (int i = 0; i < CH; i++)
-                if (c0 + i * 64 < K8) keep[i] = load_row_chunk<XT>(src, row, K, min(c0 + i * 64 + lane, K8 - 1));
+            for (int i = 0; i < CH; i++) {
+                const int piece = p0 + i * PW + part;
+                if (piece < pieces) keep[i] = load_row_chunk<XT>(src, row, K, min(piece * 64 + lane, K8 - 1));
+            }
         }
 #pragma unroll
         for (int i = 0; i < CH; i++) {
-            const int cb = c0 + i * 64;
-            if (cb < K8) {                                   // (uniform over the workgroup)
-                u32x4_t* tl = tile[piece & 1];
-                tl[r * kStagePitch + lane] = convert(keep[i], cb + lane);
+            if (p0 + i * PW < pieces) {                      // (uniform over the workgroup: some part has this piece)
+                const int piece = p0 + i * PW + part;
+                u32x4_t* tl = tile[part][round & 1];
+                if (piece < pieces) tl[r * kStagePitch + lane] = convert(keep[i], piece * 64 + lane);
                 __syncthreads();
-                const int g = (cb >> 2) + gl;
-                if (g < G) dst[((int64_t)rb * G + g) * 64 + oct * 16 + r0 + rr] = tl[rr * kStagePitch + gl * 4 + oct];
-                piece++;
+                const int g = piece * 16 + gl;
+                if (piece < pieces && g < G) dst[((int64_t)rb * G + g) * 64 + oct * 16 + r0 + rr] = tl[rr * kStagePitch + gl * 4 + oct];
+                round++;
             }
         }
     }
@@ -1135,21 +1157,21 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
             // per-row scaled f16 operands; one sum of squares per row
             ns = NormStats{ssq_part, 1, unscale};
             const dim3 rgrid((unsigned)((mc + 15) / 16) * 4);
-            // chunks of 512 k a lane keeps in registers: the whole row when it has at most 16384 (bf16) or
-            // 8192 (fp32) elements
-            const int batches = (K8 + 63) / 64;
+            // pieces of 512 k a lane keeps in registers (a row is split over four waves): the whole row when it has
+            // at most 16384 (bf16) or 8192 (fp32) elements
+            const int batches = ((K8 + 63) / 64 + 3) / 4;
 #define CYBQ_STAGE_ROWS(XT, NORM, CH) \
-    hipLaunchKernelGGL((stage_rows_kernel<XT, NORM, CH>), rgrid, dim3(256), 0, st, xs, xst, mc, w.K, epi, ssq_part, unscale)
+    hipLaunchKernelGGL((stage_rows_kernel<XT, NORM, CH>), rgrid, dim3(1024), 0, st, xs, xst, mc, w.K, epi, ssq_part, unscale)
 #define CYBQ_STAGE_ROWS_CH(XT, NORM, C1, C2, C3)              \
     do {                                                      \
         if (batches <= C1) CYBQ_STAGE_ROWS(XT, NORM, C1);     \
         else if (batches <= C2) CYBQ_STAGE_ROWS(XT, NORM, C2); \
         else CYBQ_STAGE_ROWS(XT, NORM, C3);                   \
     } while (0)
-            if (xdt == kF32 && epi.gamma) CYBQ_STAGE_ROWS_CH(2, true, 4, 8, 16);
-            else if (xdt == kF32) CYBQ_STAGE_ROWS_CH(2, false, 4, 8, 16);
-            else if (epi.gamma) CYBQ_STAGE_ROWS_CH(1, true, 8, 16, 32);
-            else CYBQ_STAGE_ROWS_CH(1, false, 8, 16, 32);
+            if (xdt == kF32 && epi.gamma) CYBQ_STAGE_ROWS_CH(2, true, 1, 2, 4);
+            else if (xdt == kF32) CYBQ_STAGE_ROWS_CH(2, false, 1, 2, 4);
+            else if (epi.gamma) CYBQ_STAGE_ROWS_CH(1, true, 2, 4, 8);
+            else CYBQ_STAGE_ROWS_CH(1, false, 2, 4, 8);
 #undef CYBQ_STAGE_ROWS_CH
 #undef CYBQ_STAGE_ROWS
         } else if (epi.gamma) {
