@@ -35,8 +35,8 @@ MIN_TIMED_S = 0.050
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the
 # same counter reads for a plain 256 MiB copy; profiles/decode_gemv_q4_4096x14336_m1.md and
 # profiles/prefill_gemm_q4_4096x14336_m512.md
-TRAFFIC_DECODE_BYTES = 33_191_700
-TRAFFIC_PREFILL_M512_BYTES = 121_400_000      # multiply 112.9 MB + activation staging pass 8.5 MB
+TRAFFIC_DECODE_BYTES = 33_191_800              # (16180.5 KiB x 1.9998 + 56.0 KiB) x 1024
+TRAFFIC_PREFILL_M512_BYTES = 121_400_000      # multiply 113.0 MB + activation staging pass 8.4 MB
 
 
 def log(*a):
