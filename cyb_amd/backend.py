@@ -90,6 +90,7 @@ def load_library() -> ctypes.CDLL:
     lib.cybq_dequant.argtypes = [vp, vp, vp, vp]
     lib.cybq_quantize.argtypes = [vp, ci, vp, i64, i64, vp, vp, vp]
     # diagnostics (cyb_amd/csrc/cybq_debug.h), not part of the operator interface
+    lib.cybq_debug_set_gemm_tuning.argtypes = [ci]
     lib.cybq_debug_set_gemv_tuning.argtypes = [ci, ci, ci]
     lib.cybq_debug_read_weight.argtypes = [vp, i64, vp, ci, vp, vp, vp]
     lib.cybq_debug_read_pattern.argtypes = [vp, i64, vp, ci, vp]
@@ -434,6 +435,11 @@ class Backend:
     def debug_mfma_loop(self, waves_per_simd: int, iters: int, sink, stream: int = 0) -> None:
         """Diagnostics: `iters` x 16 independent v_mfma_f32_16x16x32_f16 per wave on every SIMD."""
         self._check(self._lib.cybq_debug_mfma_loop(self._ctx, waves_per_simd, iters, _ptr(sink), stream))
+
+    def set_gemm_tuning(self, rows_kernel: int = 0) -> None:
+        """Experiments only: 2 keeps 33..64-row prefill calls away from the K-splitting kernel, 1 sends them
+        there whatever the output width, 0 restores the automatic choice."""
+        self._lib.cybq_debug_set_gemm_tuning(rows_kernel)
 
     def set_gemv_tuning(self, waves: int = 0, rows_kernel: int = 0, unroll: int = 0) -> None:
         """Diagnostics: waves per workgroup; decode kernel choice (0 auto, 1 always the

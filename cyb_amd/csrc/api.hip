@@ -674,6 +674,12 @@ int cybq_quantize(cybq_ctx* ctx, cybq_quant quant, const float* src, int64_t N, 
 
 /* ---- diagnostics declared in cybq_debug.h (not part of the operator interface) ---- */
 
+int cybq_debug_set_gemm_tuning(int rows_kernel)
+{
+    cybq::set_gemm_tuning(rows_kernel);
+    return CYBQ_OK;
+}
+
 int cybq_debug_set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll)
 {
     cybq::set_gemv_tuning(waves_per_group, rows_kernel, unroll);

@@ -1,0 +1,212 @@
+// gemm_rows.hip - prefill kernel for few rows (33 .. 64) on a wide output, FAST mode (f16 operands).
+//
+// With so few rows a CU's share of the product is small (64 rows x 56 columns at N = 14336) and what
+// the tiled kernels of gemm.hip spend per K tile - a barrier, every weight operand read from LDS by
+// every multiplying wave - no longer hides behind arithmetic: their K loop costs 0.45 - 0.6 us per K
+// tile whatever the tile holds.
+//
+// Here the waves of a workgroup share nothing until the end.  The workgroup owns all rows of the call
+// and NF column blocks of 16; wave w takes the K tiles w, w + WAVES, ... and, for those, multiplies ALL
+// rows against ALL column blocks (MF x NF accumulator blocks per wave).  A weight tile is then needed by
+// exactly one wave: global memory -> registers -> dequantised in registers (round_f16(scale * q), the
+// operand of FAST mode) -> MFMA B operand, no LDS, no barrier; and every row of X enters the CU once
+// (staged operand order, 1 KB per load) and meets all NF column blocks from registers.  One wave per SIMD
+// owns the register file (accumulators, a K tile of X and four K tiles of packed weights in flight).  At
+// the end the waves' partial sums meet through LDS and are added in wave order (fixed order: results are
+// reproducible and a row's bits do not depend on the other rows of the batch).
+//
+// 4096 -> 14336 at 33 .. 64 bf16 rows: 18.1 - 19.1 us per call (with the staging pass) against 21.5 - 22.1 for
+// the tiled kernel; 4096 -> 28672 31 - 33 against 38 - 39; 8192 -> 14336 30 - 32 against 36.5 - 38.  With eight
+// row blocks per wave (65 .. 128 rows) the operands no longer fit the register file next to 128 accumulator
+// registers and the kernel measured slower than the tiled one (31 against 27 us): those calls stay there.
+#include <algorithm>
+#include <type_traits>
+
+#include "cybq_device.h"
+#include "cybq_internal.h"
+
+namespace cybq {
+
+namespace {
+
+#include "gemm_parts.h"
+
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for_r(F&& f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for_r<I + 1, N>(f);
+    }
+}
+
+// group j of a native tile -> the FAST-mode B operand round_f16(scale * q), in registers
+template <int BITS>
+__device__ __forceinline__ void dequant_group(const WRegs<BITS>& r, int j, uint32_t magic, Frag16& b)
+{
+    uint32_t bw[4];
+    if (BITS == 4) unpack_q4_f16(r.q[0][2 * (j >> 1)], r.q[0][2 * (j >> 1) + 1], j & 1, magic, bw);
+    else unpack_q8_f16(r.q[(BITS == 4) ? 0 : (j >> 1)][(j & 1) * 2], r.q[(BITS == 4) ? 0 : (j >> 1)][(j & 1) * 2 + 1], bw);
+    const uint32_t sb = (j & 1) ? (r.s[j >> 1] >> 16) : (r.s[j >> 1] & 0xffffu);
+    const _Float16 sh = __builtin_bit_cast(_Float16, (uint16_t)sb);
+    const half2_t s2 = {sh, sh};
+#pragma unroll
+    for (int p = 0; p < 4; p++) b.u[p] = as_u32(as_h2(bw[p]) * s2);
+}
+
+// MF row blocks of 16 (all rows of the call: M <= 16 * MF; MF = 4), NF column blocks per workgroup, WAVES
+// waves that split K, DEPTH K tiles of packed weights and XD K tiles of X in flight per wave.
+template <int BITS, int MF, int NF, int WAVES, int DEPTH, int XD>
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVES / 4, WAVES / 4))) void gemm_rows_kernel(
+    const uint8_t* __restrict__ wbase, const u32x4_t* __restrict__ x, int KT_, int NT_, int x_row_blocks, int M, int N_,
+    void* __restrict__ y, int ydt, int K_, Epilogue epi, NormStats ns)
+{
+    const WeightView w = {wbase, N_, K_, NT_, KT_, BITS};
+    constexpr int FR = MF * NF;                        // accumulator blocks per wave
+    static_assert(DEPTH % XD == 0 && MF == 4, "shape");
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    float4_t* part = reinterpret_cast<float4_t*>(smem);                                    // [WAVES][FR][64]
+    float* stg = reinterpret_cast<float*>(smem + (size_t)WAVES * FR * 1024);               // [MF][16 * NF * 16]
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nt0 = (int)blockIdx.x * NF;
+    const int KT = w.KT, K = w.K, G = K / kGroup;
+    const uint32_t magic = q4_magic_vgpr();
+    const int T = KT > wv ? (KT - wv + WAVES - 1) / WAVES : 0;        // my K tiles: number t is tile wv + WAVES * t
+    // Workgroups that run side by side read the same rows of X: walking K in the same order they would all
+    // ask the same L2 channels for the same lines at the same moment, so every column tile starts its walk
+    // at another K tile and wraps around (the order depends on the column tile only, not on M).
+    const int kt0 = (int)blockIdx.x % KT;
+    // (a tile number past my last one is clamped to the last K tile: loaded again, never used)
+    auto tile_of = [&](int t) __attribute__((always_inline)) {
+        const int kt = min(wv + WAVES * t, KT - 1) + kt0;
+        return kt >= KT ? kt - KT : kt;
+    };
+    // (row blocks and column blocks past the end are clamped to the last real one: computed again, never
+    // stored; the offsets are wave-uniform, the lane's part of an address is one register)
+    const u32x4_t* xl = x + lane;
+    int xrow[MF];
+#pragma unroll
+    for (int i = 0; i < MF; i++) xrow[i] = __builtin_amdgcn_readfirstlane(min(i, x_row_blocks - 1) * G * 64);
+    int64_t wtile[NF];
+#pragma unroll
+    for (int f = 0; f < NF; f++) wtile[f] = (int64_t)min(nt0 + f, w.NT - 1) * w.KT;
+    auto load_x = [&](Frag16 (&dst)[MF], int t, int j) __attribute__((always_inline)) {
+        const int g = min(tile_of(t) * 4 + j, G - 1);
+#pragma unroll
+        for (int i = 0; i < MF; i++) dst[i].u = xl[xrow[i] + g * 64];
+    };
+    auto fetch = [&](WRegs<BITS> (&dst)[NF], int t) __attribute__((always_inline)) {
+        const int kt = tile_of(t);
+#pragma unroll
+        for (int f = 0; f < NF; f++) load_wtile<BITS>(dst[f], w, wtile[f] + kt, lane);
+    };
+
+    float4_t acc[MF][NF];
+#pragma unroll
+    for (int i = 0; i < MF; i++)
+#pragma unroll
+        for (int f = 0; f < NF; f++) acc[i][f] = (float4_t){0.f, 0.f, 0.f, 0.f};
+
+    WRegs<BITS> wreg[DEPTH][NF];
+    Frag16 xa[XD][4][MF];
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) fetch(wreg[d], d);
+#pragma unroll
+    for (int d = 0; d < XD; d++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) load_x(xa[d][j], d, j);
+
+    // my K tile number t (register sets R = t % DEPTH, R % XD): multiply; its X registers take the rows of tile
+    // t + XD group by group as they fall free; its weight registers take tile t + DEPTH
+    auto k_tile = [&](int t, auto residue) __attribute__((always_inline)) {
+        constexpr int R = decltype(residue)::value;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+#pragma unroll
+            for (int f = 0; f < NF; f++) {
+                Frag16 b;
+                dequant_group<BITS>(wreg[R][f], j, magic, b);
+#pragma unroll
+                for (int i = 0; i < MF; i++) acc[i][f] = mma<0>(xa[R % XD][j][i], b, acc[i][f]);
+            }
+            load_x(xa[R % XD][j], t + XD, j);
+        }
+        fetch(wreg[R], t + DEPTH);
+    };
+    int t = 0;
+    for (; t + DEPTH <= T; t += DEPTH)
+        static_for_r<0, DEPTH>([&](auto i) __attribute__((always_inline)) { k_tile(t + decltype(i)::value, i); });
+    static_for_r<0, DEPTH - 1>([&](auto i) __attribute__((always_inline)) {
+        if (t + decltype(i)::value < T) k_tile(t + decltype(i)::value, i);
+    });
+
+    // ---- the partial sums meet: every wave leaves all of its blocks, waves 0 .. MF-1 finish a row block each
+#pragma unroll
+    for (int i = 0; i < MF; i++)
+#pragma unroll
+        for (int f = 0; f < NF; f++) part[(wv * FR + i * NF + f) * 64 + lane] = acc[i][f];
+    __syncthreads();
+    if (wv >= MF) return;
+    float4_t tot[1][NF];
+#pragma unroll
+    for (int f = 0; f < NF; f++) {
+        const int blk = wv * NF + f;
+        float4_t s = part[blk * 64 + lane];
+#pragma unroll
+        for (int p = 1; p < WAVES; p++) s += part[(p * FR + blk) * 64 + lane];
+        tot[0][f] = s;
+    }
+    const int m0 = wv * 16;
+    if (epi.gamma || ns.unscale) {
+#pragma unroll
+        for (int r4 = 0; r4 < 4; r4++) {
+            const float rs = row_factor(ns, epi.gamma != nullptr, min(m0 + (lane >> 4) * 4 + r4, M - 1), K, epi.eps);
+#pragma unroll
+            for (int f = 0; f < NF; f++) tot[0][f][r4] *= rs;
+        }
+    }
+    write_rows<1, NF>(tot, stg + wv * (16 * NF * 16), m0, nt0, M, w.N, y, ydt, 1.0f, epi, lane);
+}
+
+template <int BITS, int MF, int NF, int WAVES, int DEPTH, int XD>
+hipError_t launch_rows_t(const WeightView& w, const void* x, int M, void* y, int ydt, const Epilogue& epi, const NormStats& ns,
+                         hipStream_t st)
+{
+    constexpr int lds = WAVES * MF * NF * 1024 + MF * 16 * NF * 16 * 4;
+    (void)LdsRequest<&gemm_rows_kernel<BITS, MF, NF, WAVES, DEPTH, XD>, lds>::registered;
+    const unsigned groups = (unsigned)((w.NT + NF - 1) / NF);
+    hipLaunchKernelGGL((gemm_rows_kernel<BITS, MF, NF, WAVES, DEPTH, XD>), dim3(groups), dim3(WAVES * 64), lds, st, w.base,
+                       reinterpret_cast<const u32x4_t*>(x), w.KT, w.NT, (M + 15) / 16, M, w.N, y, ydt, w.K, epi, ns);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool gemm_rows_serves(const WeightView& w, int M, int num_cus, const Epilogue& epi)
+{
+    if (M <= 32 || M > 64 || epi.kind == kEpiSwiglu) return false;
+    // A call takes about 1.6 us per K tile of a wave whatever the number of workgroups (4096 -> 8192, 128
+    // workgroups: 16.6 us against 20.9 for the tiled kernels; 4096 -> 14336, 224: 18.1 against 21.5): from
+    // half a round of 64-column workgroups up, and for K up to 8192 (beyond that the tiled kernels split K
+    // over workgroups: 14336 -> 4096 33.6 against 43 us here).
+    const int64_t groups = (w.NT + 3) / 4;
+    return groups * 2 >= (int64_t)num_cus && w.KT >= 16 && w.KT <= 64;
+}
+
+hipError_t launch_gemm_rows(const WeightView& w, const void* x_staged, int M, void* y, int ydt, const Epilogue& epi,
+                            const float* ssq_part, int ssq_blocks, const float* unscale, hipStream_t st)
+{
+    const NormStats ns = {ssq_part, ssq_blocks, unscale};
+    // four waves, one per SIMD with the whole register file: four K tiles of packed weights and one K tile of
+    // X in flight per wave.  Measured against it on 4096 -> 14336 at 64 bf16 rows (19.1 us per call with the
+    // staging pass; the tiled kernel 22.1): eight waves with two / three weight tiles in flight 22.8 / 20.2;
+    // X two / four K tiles ahead 21.7 / 20.4; eight weight tiles ahead 23.9; MFMAs and dequantisation
+    // interleaved by scheduling hints 21.2; four staging + four multiplying waves sharing K slots through
+    // LDS 26.7.
+    if (w.bits == 8) return launch_rows_t<8, 4, 4, 4, 4, 1>(w, x_staged, M, y, ydt, epi, ns, st);
+    return launch_rows_t<4, 4, 4, 4, 4, 1>(w, x_staged, M, y, ydt, epi, ns, st);
+}
+
+}  // namespace cybq

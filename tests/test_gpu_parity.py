@@ -795,6 +795,58 @@ def test_prefill_role_split_kernel(backend, oracle, bits, shape):
     assert ((y3.double() - ref).norm() / ref.norm()).item() < 2 * FAST
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("shape", [(14336, 2048, 64), (8200, 4096 + 128, 33), (8198, 4096 + 256, 47), (14336, 4096, 48),
+                                   (28672, 2048, 40), (8192, 8192, 64)])
+def test_prefill_few_rows_waves_split_k(backend, oracle, bits, shape):
+    """33 .. 64 rows in FAST mode on an output at least half a round of 64-column workgroups wide, K of 16 ..
+    64 tiles: the kernel whose four waves split K and share nothing until the end (no LDS on the way, one
+    partial-sum exchange).  K tile counts that do not divide by four (waves with unequal shares), N that ends
+    inside a column block with rows of y aligned and not, every activation and output type, residual add,
+    folded RMSNorm; the tiled kernels (the same call with the kernel switched off) agree within the mode's
+    tolerance; a row's bits do not depend on the rows it travels with; reproducible.  (Weights of more than
+    6144 x 4096 elements: smaller ones take two passes of the batched-rows decode kernel at these row counts.)"""
+    N, K, M = shape
+    q, s = _quant(oracle, bits, N, K, cfg=61)
+    qw = backend.upload_quantized(q, s, bits)
+    wd = torch.from_numpy(oracle.dequant(q, s)).cuda().double()
+    r = torch.from_numpy(synth.activations(63, M, N)).cuda()
+    try:
+        for xdt, ydt in (("bf16", "f32"), ("f16", "bf16"), ("f32", "f16"), ("f16", "f32")):
+            x = _x(M, K, xdt, cfg=62)
+            ref = x.double() @ wd.T
+            y = _run(backend, qw, x, ydt)
+            bar = FAST if ydt == "f32" else 4e-3            # (a 16-bit output rounds every element once more)
+            assert ((y.double() - ref).norm() / ref.norm()).item() < bar, (xdt, ydt)
+            assert torch.equal(_run(backend, qw, x, ydt), y)             # reproducible
+            backend.set_gemm_tuning(2)                                     # the tiled kernels on the same call
+            y_tiled = _run(backend, qw, x, ydt)
+            backend.set_gemm_tuning(0)
+            assert ((y.double() - y_tiled.double()).norm() / ref.norm()).item() < 2 * bar, (xdt, ydt)
+            if ydt == "f32":
+                assert not torch.equal(y, y_tiled)                         # (another order of summation: it did run)
+            y2 = torch.empty((M, N), dtype=TDT[ydt], device="cuda")
+            backend.matmul_ex(qw, x, y2, "add", r.to(TDT[ydt]))
+            torch.cuda.synchronize()
+            want = ref + r.to(TDT[ydt]).double()
+            assert ((y2.double() - want).norm() / want.norm()).item() < bar, (xdt, ydt)
+        x = _x(64, K, "f16", cfg=62)
+        y64 = _run(backend, qw, x)
+        y37 = _run(backend, qw, x[:37].contiguous())
+        assert torch.equal(y64[:37], y37)
+        x = _x(M, K, "bf16", cfg=62)
+        gamma = (1.0 + 0.1 * torch.from_numpy(synth.activations(64, 1, K))[0]).cuda()
+        y3 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        backend.matmul_norm(qw, x, gamma, 1e-5, y3)
+        torch.cuda.synchronize()
+        xd = x.double()
+        ref = (xd * torch.rsqrt((xd * xd).mean(dim=1, keepdim=True) + 1e-5) * gamma.double()) @ wd.T
+        assert ((y3.double() - ref).norm() / ref.norm()).item() < 2 * FAST
+    finally:
+        backend.set_gemm_tuning(0)
+    qw.free()
+
+
 def test_lm_head_shape(backend, oracle):
     """The LM head of a Llama-3-sized vocabulary (decide/pipeline.md:51): 128256 rows, K = 4096, Q4 -
     8016 strips, several rounds of workgroups per CU.  Weights are made and quantised on the device;
