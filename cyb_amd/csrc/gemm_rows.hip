@@ -17,8 +17,10 @@
 //
 // 4096 -> 14336 at 33 .. 64 bf16 rows: 18.1 - 19.1 us per call (with the staging pass) against 21.5 - 22.1 for
 // the tiled kernel; 4096 -> 28672 31 - 33 against 38 - 39; 8192 -> 14336 30 - 32 against 36.5 - 38.  With eight
-// row blocks per wave (65 .. 128 rows) the operands no longer fit the register file next to 128 accumulator
-// registers and the kernel measured slower than the tiled one (31 against 27 us): those calls stay there.
+// row blocks per wave (65 .. 128 rows) a wave has twice the MFMAs to issue per K tile next to the same
+// dequantisation and the kernel is no quicker than the tiled one (X a whole K tile ahead: the operands no
+// longer fit the register file next to 128 accumulator registers, 31 against 27 us; X half a K tile ahead:
+// 27.5 against 27.4 at 128 rows, 25.3 against 24.2 at 65): those calls stay there.
 #include <algorithm>
 #include <type_traits>
 
