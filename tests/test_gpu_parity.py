@@ -1610,6 +1610,27 @@ def test_first_call_of_a_kernel_may_sit_inside_a_capture(oracle):
         torch.cuda.synchronize()
         assert torch.equal(ye, y)
         qw.free()
+        # FAST mode, 50 rows on a wide output: the kernel whose waves split K (80 KB of LDS for its one exchange)
+        be.set_prefill_mode("fast")
+        N, K, M = 8192 + 64, 4096 + 128, 50
+        q, s = _quant(oracle, 4, N, K, cfg=94)
+        qw = be.upload_quantized(q, s, 4)
+        x = _x(M, K, "bf16", cfg=95)
+        y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            be.matmul(qw, x, y, stream=torch.cuda.current_stream().cuda_stream)
+        for _ in range(2):
+            y.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert oracle.rel_l2(y.cpu().numpy(), oracle.matmul_f64(q, s, x.float().cpu().numpy())) < FAST
+        ye = torch.zeros_like(y)
+        be.matmul(qw, x, ye)
+        torch.cuda.synchronize()
+        assert torch.equal(ye, y)
+        qw.free()
     finally:
         be.close()
 

@@ -39,6 +39,7 @@ def test_static_scratch_matches_allocated_workspace(backend, oracle):
             _case(backend, oracle, 4096, 14336, 512, torch.bfloat16, mode)
             _case(backend, oracle, 1024, 2048, 100, torch.bfloat16, mode)
         _case(backend, oracle, 14336, 4096, 300, torch.float16, "fast")
+        _case(backend, oracle, 14336, 4096, 48, torch.bfloat16, "fast")     # few rows on a wide output: the waves split K
         _case(backend, oracle, 4096, 14336, 16, torch.float16, "fast")      # decode rows on few strips and a long K: tickets and slabs
         _case(backend, oracle, 320, 4096, 1, torch.float16, "fast")         # (other decode rows use no scratch at all)
         _case(backend, oracle, 320, 4096, 24, torch.float32, "fast")
