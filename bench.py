@@ -32,6 +32,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / f16, published
 MALL_BYTES = 256 << 20
 MIN_TIMED_S = 0.050
+SETTLE_LAUNCHES = 4000          # ~27 ms of the timed kernel before the first timed pass (clocks settle in ~10 ms)
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the
 # same counter reads for a plain 256 MiB copy; profiles/decode_gemv_q4_4096x14336_m1.md and
 # profiles/prefill_gemm_q4_4096x14336_m512.md
@@ -59,22 +60,30 @@ class Timer:
         t.cuda.synchronize()
         return a.elapsed_time(b) * 1e-3      # seconds
 
-    def train(self, make_pass, min_s=MIN_TIMED_S, max_passes=400):
-        """Passes enqueued back to back between two synchronisations, each between its own pair of events:
-        make_pass(i) enqueues pass i; returns (mean seconds per pass, per-pass list).  The device does not
-        idle through a host round trip between passes, so a pass of few launches is not timed at the
-        clocks and with the empty queues of a GPU that has just been waited for."""
+    def train(self, make_pass, min_s=MIN_TIMED_S, max_passes=400, group=1):
+        """Passes enqueued back to back between two synchronisations; every `group` consecutive passes sit
+        between their own pair of events (an event pair costs about as much as a short launch: around
+        passes of 20 launches it would be 1 % of what it measures).  make_pass(i) enqueues pass i; returns
+        (mean seconds per pass, per-pass list - a group's time divided by its passes -, seconds of one pass
+        timed alone on an idle device).  The device does not idle through a host round trip between
+        passes, so a pass of few launches is not timed at the clocks and with the empty queues of a GPU that
+        has just been waited for."""
         t = self.torch
         first = self.once(lambda: make_pass(0))
         n = max(2, min(max_passes, int(min_s / max(first, 1e-7)) + 1))
-        evs = [(t.cuda.Event(enable_timing=True), t.cuda.Event(enable_timing=True)) for _ in range(n)]
+        group = max(1, min(group, n // 2))
+        groups = (n + group - 1) // group
+        evs = [(t.cuda.Event(enable_timing=True), t.cuda.Event(enable_timing=True)) for _ in range(groups)]
         t.cuda.synchronize()
-        for i, (a, b) in enumerate(evs):
+        i = 0
+        for a, b in evs:
             a.record()
-            make_pass(1 + i)
+            for _ in range(group):
+                i += 1
+                make_pass(i)
             b.record()
         t.cuda.synchronize()
-        times = [a.elapsed_time(b) * 1e-3 for a, b in evs]
+        times = [a.elapsed_time(b) * 1e-3 / group for a, b in evs]
         return sum(times) / len(times), times, first
 
     def until(self, make_pass, min_s=MIN_TIMED_S, max_passes=400):
@@ -249,21 +258,32 @@ def main():
                 plans[(n, c)] = plan_of(n, c)
             c = (c + n) % copies
 
-    # everything still cached from the set-up (clones, parity) is pushed out first
-    # (and repeated for some 20 ms: a device that has idled through the set-up runs its first
-    # milliseconds of load below its clocks)
+    # (every plan is built first: neither the warm-up nor the timed passes wait for host work, the device
+    # does not idle in between)
+    # A device that has idled through the set-up runs its first ~10 ms of load below its clocks (12 % slower).
+    # Whatever --warmup says, the timed passes are preceded by at least SETTLE_LAUNCHES launches of the timed
+    # kernel: --warmup of them as asked, the rest as an untimed settling walk (named in the record).
+    settle = max(0, SETTLE_LAUNCHES - args.warmup)
+    c = cursor[0]
+    if args.warmup > 0:
+        plans[(args.warmup, c)] = plan_of(args.warmup, c)
+        c = (c + args.warmup) % copies
+    if settle > 0:
+        plans[(settle, c)] = plan_of(settle, c)
+    prepare(args.steps, after=args.warmup + settle)
+    # everything still cached from the set-up (clones, parity) is pushed out
     flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
     for i in range(64):
         flush.fill_(i & 1)
     torch.cuda.synchronize()
     del flush
-    # (every plan is built before the warm-up: the timed passes follow it without the device idling
-    # through host work in between)
-    prepare(args.steps, after=args.warmup)
     if args.warmup > 0:
-        plans[(args.warmup, cursor[0])] = plan_of(args.warmup, cursor[0])
         walk(args.warmup, lambda p: be.matmul_many(p, M, stream))
-    mean_pass, passes, first_pass = timer.train(lambda i: walk(args.steps, lambda p: be.matmul_many(p, M, stream)))
+    if settle > 0:
+        walk(settle, lambda p: be.matmul_many(p, M, stream))
+    # (passes of fewer than 1000 launches share an event pair with their neighbours)
+    pass_group = max(1, (1000 + args.steps - 1) // args.steps)
+    mean_pass, passes, first_pass = timer.train(lambda i: walk(args.steps, lambda p: be.matmul_many(p, M, stream)), group=pass_group)
     us = mean_pass / args.steps * 1e6
     gbs = alg_bytes / (mean_pass / args.steps) / 1e9
     log(f"decode GEMV: {us:.2f} us/launch, {gbs:.0f} GB/s ({len(passes)} passes of {args.steps} steps)")
@@ -314,8 +334,8 @@ def main():
     spread = {"min": round(per[0], 3), "median": round(per[len(per) // 2], 3), "max": round(per[-1], 3),
               "in_order": [round(t / args.steps * 1e6, 3) for t in passes],
               "pass_after_an_idle_device": round(first_pass / args.steps * 1e6, 3),
-              "of": f"{len(per)} timed passes of {args.steps} back-to-back launches, each between its own pair of HIP events, "
-                    "the passes enqueued back to back between two synchronisations; us per launch"}
+              "of": f"{len(per)} timed groups of {pass_group} pass(es) of {args.steps} back-to-back launches, each group between its own "
+                    "pair of HIP events, all enqueued back to back between two synchronisations; us per launch"}
 
     result = {
         "metric": "Q4 GEMV GB/s at 4096x14336 b=1",
@@ -333,7 +353,8 @@ def main():
         "data": "synthetic (seeded Philox: W~N(0,0.02) quantised per 32-group, x~N(0,1))",
         "config": {"workload": "Q4 decode GEMV, K=4096 -> N=14336, M=1, x f16, y f32 (BASELINE configs[1])",
                    "weight_copies_rotated": int(copies), "algorithmic_bytes_per_step": int(alg_bytes),
-                   "timed_passes": len(passes), "timed_device_ms": round(sum(passes) * 1e3, 2)},
+                   "timed_passes": len(passes) * pass_group, "timed_device_ms": round(sum(passes) * pass_group * 1e3, 2),
+                   "untimed_launches_before_the_first_timed_pass": {"warmup": args.warmup, "settling_walk": settle}},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_DECODE_BYTES},
         "parity_rel_l2": rel_l2,
