@@ -303,20 +303,12 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2
         }
     }
 
-    // ---- epilogue: a K split leaves its partial sums in fp32 for splitk_reduce_kernel
+    // ---- epilogue: a K split leaves its partial sums in fp32 for splitk_reduce_kernel (whole runs of a row
+    // through LDS, like the final sums)
     if (splits > 1) {
-        float* dst = part + (int64_t)split * M * w.N;
-#pragma unroll
-        for (int i = 0; i < MF; i++)
-#pragma unroll
-            for (int f = 0; f < NF; f++) {
-                const int n = (nt0 + f) * 16 + row16;
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const int m = m0 + i * 16 + oct * 4 + r;
-                    if (m < M && n < w.N) dst[(int64_t)m * w.N + n] = acc[i][f][r];
-                }
-            }
+        const Epilogue plain = {kEpiNone, nullptr, nullptr, 0, 0.f};
+        write_rows<MF, NF>(acc, reinterpret_cast<float*>(smem) + wv * (16 * NF * 16), m0, nt0, M, w.N, part + (int64_t)split * M * w.N, kF32,
+                           1.0f, plain, lane);
         return;
     }
     if (epi.gamma || ns.unscale) {     // folded RMSNorm: rstd of the row; widened activations: the row's power of two
