@@ -44,11 +44,11 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
                        int num_cus, bool exact, void* workspace, size_t workspace_bytes, const Epilogue& epi,
                        hipStream_t st);
 
-// few rows (33 .. 64) on an output wide enough, FAST mode, activations already staged as f16 operands
+// few rows (33 .. 64 on an output wide enough, 65 .. 128 on a narrow one), FAST mode, activations already staged as f16 operands
 // (gemm_rows.hip); ssq_part / ssq_blocks / unscale: the staging pass's per-row statistics
 bool gemm_rows_serves(const WeightView& w, int M, int num_cus, const Epilogue& epi);
 hipError_t launch_gemm_rows(const WeightView& w, const void* x_staged, int M, void* y, int ydt, const Epilogue& epi,
-                            const float* ssq_part, int ssq_blocks, const float* unscale, hipStream_t st);
+                            const float* ssq_part, int ssq_blocks, const float* unscale, int num_cus, hipStream_t st);
 // test/bench hook: 2 = never take the few-rows kernel, 1 = whatever the width, 0 = automatic
 void set_gemm_tuning(int rows_kernel);
 

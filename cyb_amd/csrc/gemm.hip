@@ -1037,7 +1037,7 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
         if (e != hipSuccess) return e;
         // few rows on a wide output, FAST mode: the kernel of gemm_rows.hip (waves split K, no LDS on the way)
         if (!exact && kdt == kF16 && g_rows_kernel != 2 && gemm_rows_serves(w, mc, g_rows_kernel == 1 ? 1 : num_cus, ec)) {
-            e = launch_gemm_rows(w, workspace, mc, yc, ydt, ec, ns.part, ns.nblk, ns.unscale, st);
+            e = launch_gemm_rows(w, workspace, mc, yc, ydt, ec, ns.part, ns.nblk, ns.unscale, g_rows_kernel == 1 ? 1 : num_cus, st);
             if (e != hipSuccess) return e;
             continue;
         }

@@ -1,26 +1,34 @@
-// gemm_rows.hip - prefill kernel for few rows (33 .. 64) on a wide output, FAST mode (f16 operands).
+// gemm_rows.hip - prefill kernel for calls whose 64-row x 32/64-column pieces fill one round of workgroups
+// (33 .. 64 rows on wide outputs, up to 512 rows on narrow ones), FAST mode (f16 operands).
 //
-// With so few rows a CU's share of the product is small (64 rows x 56 columns at N = 14336) and what
-// the tiled kernels of gemm.hip spend per K tile - a barrier, every weight operand read from LDS by
-// every multiplying wave - no longer hides behind arithmetic: their K loop costs 0.45 - 0.6 us per K
-// tile whatever the tile holds.
+// With so little work per CU (64 rows x 56 columns at N = 14336) what the tiled kernels of gemm.hip spend
+// per K tile - a barrier, every weight operand read from LDS by every multiplying wave - no longer hides
+// behind arithmetic: their K loop costs 0.45 - 0.6 us per K tile whatever the tile holds, and narrow outputs
+// make them split K over workgroups and add the slabs in a second pass.
 //
-// Here the waves of a workgroup share nothing until the end.  The workgroup owns all rows of the call
-// and NF column blocks of 16; wave w takes the K tiles w, w + WAVES, ... and, for those, multiplies ALL
-// rows against ALL column blocks (MF x NF accumulator blocks per wave).  A weight tile is then needed by
-// exactly one wave: global memory -> registers -> dequantised in registers (round_f16(scale * q), the
+// Here the waves of a workgroup share nothing until the end.  The workgroup owns 64 rows (blockIdx.y: which)
+// and NF column blocks of 16; wave w takes the K tiles w, w + WAVES, ... and, for those, multiplies ALL its
+// rows against ALL its column blocks (MF x NF accumulator blocks per wave).  A weight tile is then needed
+// by exactly one wave: global memory -> registers -> dequantised in registers (round_f16(scale * q), the
 // operand of FAST mode) -> MFMA B operand, no LDS, no barrier; and every row of X enters the CU once
 // (staged operand order, 1 KB per load) and meets all NF column blocks from registers.  One wave per SIMD
 // owns the register file (accumulators, a K tile of X and four K tiles of packed weights in flight).  At
 // the end the waves' partial sums meet through LDS and are added in wave order (fixed order: results are
 // reproducible and a row's bits do not depend on the other rows of the batch).
 //
-// 4096 -> 14336 at 33 .. 64 bf16 rows: 18.1 - 19.1 us per call (with the staging pass) against 21.5 - 22.1 for
-// the tiled kernel; 4096 -> 28672 31 - 33 against 38 - 39; 8192 -> 14336 30 - 32 against 36.5 - 38.  With eight
-// row blocks per wave (65 .. 128 rows) a wave has twice the MFMAs to issue per K tile next to the same
-// dequantisation and the kernel is no quicker than the tiled one (X a whole K tile ahead: the operands no
-// longer fit the register file next to 128 accumulator registers, 31 against 27 us; X half a K tile ahead:
-// 27.5 against 27.4 at 128 rows, 25.3 against 24.2 at 65): those calls stay there.
+// A call costs about 1.6 us per K tile of a wave, nearly whatever the number of workgroups, so the kernel
+// takes every call whose workgroups fit one round and fill at least half of it (and up to 64 rows also the
+// widest outputs, in several rounds).  Per call with the staging pass, bf16 rows, against the tiled kernels:
+//   4096 -> 14336 at 33 .. 64 rows   18.1 - 19.1 us against 21.5 - 22.1      4096 -> 28672   31 - 33 against 38 - 39
+//   4096 ->  8192 at 33 .. 64 rows   16.4 - 17.3 against 20.6 - 21.2          8192 -> 14336   30 - 32 against 36.5 - 38
+//   4096 ->  4096 at 65 .. 128 rows  16.4 - 17.2 against 21.6 - 25.5          129 .. 256 rows  17.1 - 20.0 against 21.9 - 22.3
+//   4096 ->  6144 at 65 .. 128 rows  16.6 - 17.5 against 23.4 - 26.8          4096 -> 2048 at 100 .. 300 rows  13.6 - 18.9 against 20.1 - 29.1
+//   4096 ->  1024 at 256 .. 512 rows 15.1 - 20.7 against 21.6 - 27.6
+// With eight row blocks per wave (65 .. 128 rows in one workgroup, for wide outputs whose 64-row pieces would
+// need two rounds) a wave has twice the MFMAs to issue per K tile next to the same dequantisation and the
+// kernel is no quicker than the tiled one (X a whole K tile ahead: the operands no longer fit the register
+// file next to 128 accumulator registers, 31 against 27 us; X half a K tile ahead: 27.5 against 27.4 at 128
+// rows, 25.3 against 24.2 at 65): those calls stay there.
 #include <algorithm>
 #include <type_traits>
 
@@ -56,7 +64,7 @@ __device__ __forceinline__ void dequant_group(const WRegs<BITS>& r, int j, uint3
     for (int p = 0; p < 4; p++) b.u[p] = as_u32(as_h2(bw[p]) * s2);
 }
 
-// MF row blocks of 16 (all rows of the call: M <= 16 * MF; MF = 4), NF column blocks per workgroup, WAVES
+// MF = 4 row blocks of 16 per workgroup (blockIdx.y-th 64 rows of the call), NF column blocks per workgroup, WAVES
 // waves that split K, DEPTH K tiles of packed weights and XD K tiles of X in flight per wave.
 template <int BITS, int MF, int NF, int WAVES, int DEPTH, int XD>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVES / 4, WAVES / 4))) void gemm_rows_kernel(
@@ -89,8 +97,9 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVE
     // stored; the offsets are wave-uniform, the lane's part of an address is one register)
     const u32x4_t* xl = x + lane;
     int xrow[MF];
+    const int rb0 = (int)blockIdx.y * MF;              // my first row block (blockIdx.y: which MF * 16 rows of the call)
 #pragma unroll
-    for (int i = 0; i < MF; i++) xrow[i] = __builtin_amdgcn_readfirstlane(min(i, x_row_blocks - 1) * G * 64);
+    for (int i = 0; i < MF; i++) xrow[i] = __builtin_amdgcn_readfirstlane(min(rb0 + i, x_row_blocks - 1) * G * 64);
     int64_t wtile[NF];
 #pragma unroll
     for (int f = 0; f < NF; f++) wtile[f] = (int64_t)min(nt0 + f, w.NT - 1) * w.KT;
@@ -160,7 +169,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVE
         for (int p = 1; p < WAVES; p++) s += part[(p * FR + blk) * 64 + lane];
         tot[0][f] = s;
     }
-    const int m0 = wv * 16;
+    const int m0 = (rb0 + wv) * 16;
     if (epi.gamma || ns.unscale) {
 #pragma unroll
         for (int r4 = 0; r4 < 4; r4++) {
@@ -178,35 +187,52 @@ hipError_t launch_rows_t(const WeightView& w, const void* x, int M, void* y, int
 {
     constexpr int lds = WAVES * MF * NF * 1024 + MF * 16 * NF * 16 * 4;
     (void)LdsRequest<&gemm_rows_kernel<BITS, MF, NF, WAVES, DEPTH, XD>, lds>::registered;
-    const unsigned groups = (unsigned)((w.NT + NF - 1) / NF);
-    hipLaunchKernelGGL((gemm_rows_kernel<BITS, MF, NF, WAVES, DEPTH, XD>), dim3(groups), dim3(WAVES * 64), lds, st, w.base,
+    const unsigned groups = (unsigned)((w.NT + NF - 1) / NF), row_parts = (unsigned)((M + 16 * MF - 1) / (16 * MF));
+    hipLaunchKernelGGL((gemm_rows_kernel<BITS, MF, NF, WAVES, DEPTH, XD>), dim3(groups, row_parts), dim3(WAVES * 64), lds, st, w.base,
                        reinterpret_cast<const u32x4_t*>(x), w.KT, w.NT, (M + 15) / 16, M, w.N, y, ydt, w.K, epi, ns);
     return hipGetLastError();
 }
 
 }  // namespace
 
+// Column blocks per workgroup (4 or 2) for a call of M rows, or 0 when the kernel does not take it.
+// A call takes about 1.6 us per K tile of a wave whatever the number of workgroups (4096 -> 8192 at 64 rows, 128
+// workgroups: 16.6 us against 20.9 for the tiled kernels; 4096 -> 14336, 224: 18.1 against 21.5), so: one round
+// of workgroups, at least half a round, K of 16 .. 64 tiles (beyond that the tiled kernels split K over
+// workgroups: 14336 -> 4096 33.6 against 43 us here).  65 .. 128 rows are two workgroups per column tile (64
+// rows each): narrow outputs only, where both halves fit one round.
+int rows_column_blocks(const WeightView& w, int M, int num_cus, const Epilogue& epi)
+{
+    if (M <= 32 || M > 512 || epi.kind == kEpiSwiglu || w.KT < 16 || w.KT > 64) return 0;
+    const int64_t parts = (M + 63) / 64;
+    for (int nf : {4, 2}) {
+        const int64_t groups = (w.NT + nf - 1) / nf * parts;
+        if (groups <= num_cus && groups * 2 >= num_cus) return nf;
+        if (nf == 4 && parts == 1 && groups * 2 >= num_cus) return nf;       // (up to 64 rows a wide output may take more than one round)
+    }
+    return 0;
+}
+
 bool gemm_rows_serves(const WeightView& w, int M, int num_cus, const Epilogue& epi)
 {
-    if (M <= 32 || M > 64 || epi.kind == kEpiSwiglu) return false;
-    // A call takes about 1.6 us per K tile of a wave whatever the number of workgroups (4096 -> 8192, 128
-    // workgroups: 16.6 us against 20.9 for the tiled kernels; 4096 -> 14336, 224: 18.1 against 21.5): from
-    // half a round of 64-column workgroups up, and for K up to 8192 (beyond that the tiled kernels split K
-    // over workgroups: 14336 -> 4096 33.6 against 43 us here).
-    const int64_t groups = (w.NT + 3) / 4;
-    return groups * 2 >= (int64_t)num_cus && w.KT >= 16 && w.KT <= 64;
+    return rows_column_blocks(w, M, num_cus, epi) != 0;
 }
 
 hipError_t launch_gemm_rows(const WeightView& w, const void* x_staged, int M, void* y, int ydt, const Epilogue& epi,
-                            const float* ssq_part, int ssq_blocks, const float* unscale, hipStream_t st)
+                            const float* ssq_part, int ssq_blocks, const float* unscale, int num_cus, hipStream_t st)
 {
     const NormStats ns = {ssq_part, ssq_blocks, unscale};
+    const int nf = rows_column_blocks(w, M, num_cus, epi);
     // four waves, one per SIMD with the whole register file: four K tiles of packed weights and one K tile of
     // X in flight per wave.  Measured against it on 4096 -> 14336 at 64 bf16 rows (19.1 us per call with the
     // staging pass; the tiled kernel 22.1): eight waves with two / three weight tiles in flight 22.8 / 20.2;
     // X two / four K tiles ahead 21.7 / 20.4; eight weight tiles ahead 23.9; MFMAs and dequantisation
     // interleaved by scheduling hints 21.2; four staging + four multiplying waves sharing K slots through
     // LDS 26.7.
+    if (nf == 2) {
+        if (w.bits == 8) return launch_rows_t<8, 4, 2, 4, 4, 1>(w, x_staged, M, y, ydt, epi, ns, st);
+        return launch_rows_t<4, 4, 2, 4, 4, 1>(w, x_staged, M, y, ydt, epi, ns, st);
+    }
     if (w.bits == 8) return launch_rows_t<8, 4, 4, 4, 4, 1>(w, x_staged, M, y, ydt, epi, ns, st);
     return launch_rows_t<4, 4, 4, 4, 4, 1>(w, x_staged, M, y, ydt, epi, ns, st);
 }

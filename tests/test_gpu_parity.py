@@ -797,15 +797,20 @@ def test_prefill_role_split_kernel(backend, oracle, bits, shape):
 
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("shape", [(14336, 2048, 64), (8200, 4096 + 128, 33), (8198, 4096 + 256, 47), (14336, 4096, 48),
-                                   (28672, 2048, 40), (8192, 8192, 64)])
+                                   (28672, 2048, 40), (8192, 8192, 64),
+                                   (4096, 4096, 128), (6144 - 16, 4096 + 128, 100), (1024, 4096, 512), (2048, 4096, 300),
+                                   (4102, 8192, 70), (8192, 2048, 65)])
 def test_prefill_few_rows_waves_split_k(backend, oracle, bits, shape):
-    """33 .. 64 rows in FAST mode on an output at least half a round of 64-column workgroups wide, K of 16 ..
-    64 tiles: the kernel whose four waves split K and share nothing until the end (no LDS on the way, one
-    partial-sum exchange).  K tile counts that do not divide by four (waves with unequal shares), N that ends
-    inside a column block with rows of y aligned and not, every activation and output type, residual add,
-    folded RMSNorm; the tiled kernels (the same call with the kernel switched off) agree within the mode's
-    tolerance; a row's bits do not depend on the rows it travels with; reproducible.  (Weights of more than
-    6144 x 4096 elements: smaller ones take two passes of the batched-rows decode kernel at these row counts.)"""
+    """FAST mode, K of 16 .. 64 tiles, one round of workgroups that is at least half full: the kernel whose
+    four waves split K and share nothing until the end (no LDS on the way, one partial-sum exchange).  33 .. 64
+    rows on outputs from 8192 columns (more than a round of workgroups on the widest); from (4096, 4096, 128)
+    on, narrow outputs with up to 512 rows: two to eight workgroups of 64 rows per column tile, two or four
+    column blocks wide, a ragged last row part.  K tile counts that do not divide by four (waves with unequal
+    shares), N that ends inside a column block with rows of y aligned and not, every activation and output
+    type, residual add, folded RMSNorm; the tiled kernels (the same call with the kernel switched off) agree
+    within the mode's tolerance; a row's bits do not depend on the rows it travels with; reproducible.
+    (Up to 64 rows only weights of more than 6144 x 4096 elements get here: smaller ones take two passes of
+    the batched-rows decode kernel.)"""
     N, K, M = shape
     q, s = _quant(oracle, bits, N, K, cfg=61)
     qw = backend.upload_quantized(q, s, bits)
@@ -830,10 +835,12 @@ def test_prefill_few_rows_waves_split_k(backend, oracle, bits, shape):
             torch.cuda.synchronize()
             want = ref + r.to(TDT[ydt]).double()
             assert ((y2.double() - want).norm() / want.norm()).item() < bar, (xdt, ydt)
-        x = _x(64, K, "f16", cfg=62)
-        y64 = _run(backend, qw, x)
-        y37 = _run(backend, qw, x[:37].contiguous())
-        assert torch.equal(y64[:37], y37)
+        parts = (M + 63) // 64                      # fewer rows, the same number of 64-row parts: the same kernel shape
+        fewer = 64 * (parts - 1) + 37
+        x = _x(64 * parts, K, "f16", cfg=62)
+        y_all = _run(backend, qw, x)
+        y_fewer = _run(backend, qw, x[:fewer].contiguous())
+        assert torch.equal(y_all[:fewer], y_fewer)
         x = _x(M, K, "bf16", cfg=62)
         gamma = (1.0 + 0.1 * torch.from_numpy(synth.activations(64, 1, K))[0]).cuda()
         y3 = torch.empty((M, N), dtype=torch.float32, device="cuda")
