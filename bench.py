@@ -544,6 +544,27 @@ def main():
             t.free()
         del wd, qd, sd
         extra["baseline_configs_not_covered_above"] = base
+        # ---- the attention projections of a layer (decide/pipeline.md:51) at a small prefill chunk: narrow outputs,
+        # where a call is a single round of small workgroups
+        proj = {}
+        for Nx in (4096, 6144, 1024):
+            qs_, ss_ = formats.quantize(synth.weights(2, Nx, K), bits)
+            wsm = copies_of(qs_, ss_, bits)
+            for Mr in (128, 256):
+                xr = torch.from_numpy(synth.activations(4, Mr, K)).to(dev).to(torch.bfloat16)
+                yr = torch.empty((Mr, Nx), dtype=torch.float32, device=dev)
+                nr = 100
+                rpl = be.plan_many([wsm[j % len(wsm)] for j in range(nr)], [xr] * nr, [yr] * nr)
+                be.matmul_many(rpl, Mr, stream)
+                tr, _ = timer.until(lambda i: be.matmul_many(rpl, Mr, stream), max_passes=40)
+                tr /= nr
+                proj[f"4096x{Nx}_M{Mr}"] = {"us": round(tr * 1e6, 1), "tflops": round(2.0 * Mr * Nx * K / tr / 1e12, 1)}
+                del xr, yr, rpl
+            for t in wsm:
+                t.free()
+            del wsm, qs_, ss_
+        extra["prefill_attention_projections_bf16_rows"] = proj
+        log("attention projections: " + " ".join(f"{k}:{v['us']}us" for k, v in proj.items()))
         log("other BASELINE configs: " + " ".join(f"{k}:{v['us']}us" for k, v in base.items()))
 
         # ---- LM head: 4096 -> 128256 (/root/reference/decide/pipeline.md:51), weights made on the device

@@ -1,5 +1,6 @@
 // gemm_rows.hip - prefill kernel for calls whose 64-row x 32/64-column pieces fill one round of workgroups
-// (33 .. 64 rows on wide outputs, up to 512 rows on narrow ones), FAST mode (f16 operands).
+// (17 .. 64 rows on wide outputs - up to 32 they are fp32 rows -, up to 512 rows on narrow ones), FAST mode
+// (f16 operands).
 //
 // With so little work per CU (64 rows x 56 columns at N = 14336) what the tiled kernels of gemm.hip spend
 // per K tile - a barrier, every weight operand read from LDS by every multiplying wave - no longer hides
@@ -203,7 +204,7 @@ hipError_t launch_rows_t(const WeightView& w, const void* x, int M, void* y, int
 // rows each): narrow outputs only, where both halves fit one round.
 int rows_column_blocks(const WeightView& w, int M, int num_cus, const Epilogue& epi)
 {
-    if (M <= 32 || M > 512 || epi.kind == kEpiSwiglu || w.KT < 16 || w.KT > 64) return 0;
+    if (M <= 16 || M > 512 || epi.kind == kEpiSwiglu || w.KT < 16 || w.KT > 64) return 0;      // (17 .. 32 rows get here as fp32 rows)
     const int64_t parts = (M + 63) / 64;
     for (int nf : {4, 2}) {
         const int64_t groups = (w.NT + nf - 1) / nf * parts;

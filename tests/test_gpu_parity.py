@@ -854,6 +854,36 @@ def test_prefill_few_rows_waves_split_k(backend, oracle, bits, shape):
     qw.free()
 
 
+@pytest.mark.parametrize("shape", [(14336, 4096, 17), (4096, 4096, 32), (8200, 2048 + 128, 24)])
+def test_prefill_fp32_rows_17_to_32_fast_mode(backend, oracle, shape):
+    """fp32 activations leave the decode kernels at 17 rows; in FAST mode they are rounded to f16 by the staging
+    pass and, where the shape fits, multiplied by the kernel whose waves split K (a 64-row workgroup mostly
+    empty).  Against float64, against the tiled kernels, residual add, reproducible."""
+    N, K, M = shape
+    q, s = _quant(oracle, 4, N, K, cfg=65)
+    qw = backend.upload_quantized(q, s, 4)
+    wd = torch.from_numpy(oracle.dequant(q, s)).cuda().double()
+    x = _x(M, K, "f32", cfg=66)
+    ref = x.double() @ wd.T
+    try:
+        y = _run(backend, qw, x)
+        assert ((y.double() - ref).norm() / ref.norm()).item() < FAST
+        assert torch.equal(_run(backend, qw, x), y)
+        backend.set_gemm_tuning(2)
+        y_tiled = _run(backend, qw, x)
+        backend.set_gemm_tuning(0)
+        assert ((y.double() - y_tiled.double()).norm() / ref.norm()).item() < 2 * FAST
+        assert not torch.equal(y, y_tiled)                                 # (another order of summation: it did run)
+        r = torch.from_numpy(synth.activations(67, M, N)).cuda()
+        y2 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        backend.matmul_ex(qw, x, y2, "add", r)
+        torch.cuda.synchronize()
+        assert ((y2.double() - (ref + r.double())).norm() / (ref + r.double()).norm()).item() < FAST
+    finally:
+        backend.set_gemm_tuning(0)
+    qw.free()
+
+
 def test_lm_head_shape(backend, oracle):
     """The LM head of a Llama-3-sized vocabulary (decide/pipeline.md:51): 128256 rows, K = 4096, Q4 -
     8016 strips, several rounds of workgroups per CU.  Weights are made and quantised on the device;
