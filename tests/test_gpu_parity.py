@@ -1151,6 +1151,29 @@ def test_random_wide_calls_match_float64(backend, oracle, case):
     _check_random_case(backend, oracle, case)
 
 
+def _random_mid_k_cases(seed, count):
+    """Draws over K of 16 .. 34 tiles with few rows on a wide output or up to 512 rows on a narrow one: the calls
+    whose 64-row pieces fill one round of workgroups (the prefill kernel whose waves split K), their neighbours
+    that do not, and the modes and epilogues around them."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        wide = bool(rng.random() < 0.4)
+        N = int(rng.choice([8192, 8200, 12288, 14336])) if wide else int(rng.choice([1024, 1040, 2048, 3072, 4096, 6144]))
+        M = int(rng.choice([17, 24, 33, 48, 64])) if wide else int(rng.choice([17, 40, 65, 100, 128, 129, 200, 256, 300, 384, 512]))
+        cases.append(dict(i=2000 + i, bits=int(rng.choice([4, 4, 8])), layout=int(rng.choice([formats.PLANAR, formats.BLOCK_AOS])),
+                          N=N, K=128 * int(rng.integers(16, 35)), M=M, xdt=str(rng.choice(["f16", "bf16", "f32"])),
+                          ydt=str(rng.choice(["f32", "f32", "f16", "bf16"])), epi=str(rng.choice(["none", "add"])),
+                          norm=bool(rng.random() < 0.3), gdt=str(rng.choice(["f32", "f16", "bf16"])),
+                          mode=str(rng.choice(["fast", "fast", "fast", "exact"]))))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_mid_k_cases(20240609, int(__import__("os").environ.get("CYBQ_FUZZ_MID_COUNT", "24"))), ids=lambda c: "-".join(str(v) for v in c.values()))
+def test_random_mid_k_calls_match_float64(backend, oracle, case):
+    _check_random_case(backend, oracle, case)
+
+
 def _check_random_case(backend, oracle, c):
     bits, N, K, M = c["bits"], c["N"], c["K"], c["M"]
     backend.set_prefill_mode(c["mode"])
