@@ -495,6 +495,15 @@ def main():
         for t in wd:
             t.free()
         del wd
+        # gate and up as one launch (their rows concatenated at load time): the same kernel with twice the
+        # bytes behind one launch
+        qg, sg = formats.quantize(synth.weights(7, 2 * N, K), bits)
+        wg = copies_of(qg, sg, bits)
+        del qg, sg
+        extra["decode_gate_up_as_one_launch_4096x28672"] = sweep_shape(wg, K, 2 * N, (1, 8))
+        for t in wg:
+            t.free()
+        del wg
         # the same kernels on Q8 blocks (twice the bytes per weight)
         q8, s8 = formats.quantize(synth.weights(2, N, K), formats.Q8)
         n8 = max(2, (3 * MALL_BYTES) // formats.weight_bytes(formats.Q8, N, K) + 1)
