@@ -234,6 +234,19 @@ def main():
         for i in range(50):
             be.matmul_norm(ws[i % copies], xb, gam, 1e-5, yb, stream=stream)
         torch.cuda.synchronize()
+        # the prefill kernel whose waves split K: 64 bf16 rows on 4096 -> 14336, 128 rows on 4096 -> 4096
+        x64 = torch.from_numpy(synth.activations(4, 64, K)).to(dev).to(torch.bfloat16)
+        y64 = torch.empty((64, N), dtype=torch.float32, device=dev)
+        for i in range(20):
+            be.matmul(ws[i % copies], x64, y64, stream=stream)
+        qn, sn = formats.quantize(synth.weights(8, K, K), bits)
+        wn = [be.upload_quantized(qn, sn, bits)]
+        wn += [wn[0].clone() for _ in range(copies - 1)]
+        x128 = torch.from_numpy(synth.activations(4, 128, K)).to(dev).to(torch.bfloat16)
+        y128 = torch.empty((128, K), dtype=torch.float32, device=dev)
+        for i in range(20):
+            be.matmul(wn[i % copies], x128, y128, stream=stream)
+        torch.cuda.synchronize()
         log("traffic probe done")
         return
 
@@ -433,6 +446,23 @@ def main():
             del xr, yr, rpl
         extra["prefill_rows_sweep_4096x14336"] = rows_out
         log("prefill rows sweep: " + " ".join(f"{k}:{v['us']}us" for k, v in rows_out.items()))
+
+        # ---- yardstick for the few-row prefill kernel: how fast the CUs take in bytes that sit in the L2 (every CU reads
+        # the same 512 KiB - the staged rows of a 64-row call on K = 4096 - 1 KiB per wave instruction)
+        cbuf = torch.zeros(512 * 1024, dtype=torch.uint8, device=dev)
+        fill = {}
+        for waves, inflight in ((4, 4), (4, 8), (4, 16), (8, 8)):
+            be.debug_cache_read(cbuf, cbuf.numel(), waves, inflight, 8, stream)
+            tf = min(timer.once(lambda: be.debug_cache_read(cbuf, cbuf.numel(), waves, inflight, 64, stream)) for _ in range(3))
+            fill[f"{waves}_waves_x_{inflight}_KiB_in_flight"] = {
+                "TB_per_s_into_all_CUs": round(cus * cbuf.numel() * 64 / tf / 1e12, 2),
+                "GB_per_s_per_CU": round(cbuf.numel() * 64 / tf / 1e9, 1)}
+        extra["l2_to_cu_fill_rate"] = {
+            "what": "one workgroup per CU reads the same 512 KiB 64 times (cybq_debug_cache_read); a 64-row call of the "
+                    "few-row prefill kernel on 4096 -> 14336 brings 660 KB into every CU (512 KB of them staged rows)",
+            **fill}
+        log("L2 -> CU fill: " + " ".join(f"{k}:{v['TB_per_s_into_all_CUs']}TB/s" for k, v in fill.items()))
+        del cbuf
 
         # ---- batch sweep of the decode kernels on the same shape
         def sweep_shape(wl, Kx, Nx, Ms, bitsx=bits, xdtype=torch.float16, roofline=False):

@@ -95,6 +95,7 @@ def load_library() -> ctypes.CDLL:
     lib.cybq_debug_read_weight.argtypes = [vp, i64, vp, ci, vp, vp, vp]
     lib.cybq_debug_read_pattern.argtypes = [vp, i64, vp, ci, vp]
     lib.cybq_debug_mfma_loop.argtypes = [vp, ci, ci, vp, vp]
+    lib.cybq_debug_cache_read.argtypes = [vp, vp, i64, ci, ci, ci, vp]
     _lib = lib
     return lib
 
@@ -436,9 +437,14 @@ class Backend:
         """Diagnostics: `iters` x 16 independent v_mfma_f32_16x16x32_f16 per wave on every SIMD."""
         self._check(self._lib.cybq_debug_mfma_loop(self._ctx, waves_per_simd, iters, _ptr(sink), stream))
 
+    def debug_cache_read(self, buf, nbytes: int, waves: int, in_flight: int, iters: int, stream: int = 0) -> None:
+        """Diagnostics: one workgroup of `waves` waves per CU, each reads the same `nbytes` at `buf` `iters`
+        times, 1 KiB per wave instruction, `in_flight` instructions outstanding per wave."""
+        self._check(self._lib.cybq_debug_cache_read(self._ctx, _ptr(buf), nbytes, waves, in_flight, iters, stream))
+
     def set_gemm_tuning(self, rows_kernel: int = 0) -> None:
-        """Experiments only: 2 keeps 33..64-row prefill calls away from the K-splitting kernel, 1 sends them
-        there whatever the output width, 0 restores the automatic choice."""
+        """Experiments only: 2 keeps prefill calls of up to 512 rows away from the K-splitting kernel, 1 sends
+        calls of up to 64 rows there whatever the output width, 0 restores the automatic choice."""
         self._lib.cybq_debug_set_gemm_tuning(rows_kernel)
 
     def set_gemv_tuning(self, waves: int = 0, rows_kernel: int = 0, unroll: int = 0) -> None:

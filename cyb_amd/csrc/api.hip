@@ -473,11 +473,13 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
     }
     if (M <= 16 || (M <= 32 && cybq::gemv_serves_32((int)xdt, (int)M, epi))) {
         e = cybq::launch_gemv(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->decode_exact, epi, dscr, dscr_bytes, st);
-    } else if (M <= 64 && (int64_t)w->N * w->K <= (int64_t)6144 * 4096 && cybq::gemv_serves_32((int)xdt, 32, epi)) {
-        // 33..64 rows on a small weight (up to 4096 -> 6144): the MFMA kernel would split K over
-        // workgroups and add the slabs in a second pass; two passes of the batched-rows decode kernel
-        // (32 rows, then the rest) are quicker although they stream the weights twice
-        // (4096 -> 4096 at 64 rows 21.8 -> 14.8 us, 4096 -> 1024 17.8 -> 12.6 us) - and exact
+    } else if (M <= 64 && (int64_t)w->N * w->K <= (int64_t)6144 * 4096 && cybq::gemv_serves_32((int)xdt, 32, epi) &&
+               (ctx->prefill_exact || weight_is_wide(w) || !cybq::gemm_rows_takes(v, (int)M, ctx->num_cus, epi))) {
+        // 33..64 rows on a small weight (up to 4096 -> 6144) that the few-rows MFMA kernel does not take (exact
+        // mode, wide scales, K outside 2048 .. 8192, a folded SwiGLU): the tiled MFMA
+        // kernel would split K over workgroups and add the slabs in a second pass; two passes of the
+        // batched-rows decode kernel (32 rows, then the rest) are quicker although they stream the weights twice
+        // (4096 -> 4096 at 64 rows 21.8 -> 14.8 us; the few-rows kernel 13.1) - and exact
         // (a context in CYBQ_PREFILL_EXACT mode asked for exact operands at this row count)
         const bool exact_ops = ctx->decode_exact || ctx->prefill_exact;
         const int64_t n_out = epi.kind == cybq::kEpiSwiglu ? w->N / 2 : w->N;
@@ -731,6 +733,17 @@ int cybq_debug_mfma_loop(cybq_ctx* ctx, int waves_per_simd, int iters, float* si
     if (guard.err != hipSuccess) return fail_hip(ctx, guard.err, "hipSetDevice");
     hipError_t e = cybq::launch_mfma_loop(ctx->num_cus, waves_per_simd, iters, sink, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail_hip(ctx, e, "mfma loop launch");
+    return CYBQ_OK;
+}
+
+int cybq_debug_cache_read(cybq_ctx* ctx, const void* buf, int64_t bytes, int waves, int in_flight, int iters, void* stream)
+{
+    if (!ctx) return CYBQ_ERR_INVALID;
+    DeviceGuard guard(ctx->device);
+    if (guard.err != hipSuccess) return fail_hip(ctx, guard.err, "hipSetDevice");
+    hipError_t e = cybq::launch_cache_read(buf, bytes, waves, in_flight, iters, ctx->num_cus, static_cast<hipStream_t>(stream));
+    if (e == hipErrorInvalidValue) return fail(ctx, CYBQ_ERR_INVALID, "cache read probe: bytes, waves or in_flight out of range");
+    if (e != hipSuccess) return fail_hip(ctx, e, "cache read launch");
     return CYBQ_OK;
 }
 

@@ -50,6 +50,12 @@ int cybq_debug_read_pattern(cybq_ctx* ctx, int64_t count, const cybq_weight* con
  * waves each issue `iters` x 16 instructions.  flops = CUs * 4 * waves_per_simd * iters * 16 * 16384. */
 int cybq_debug_mfma_loop(cybq_ctx* ctx, int waves_per_simd, int iters, float* sink, void* stream);
 
+/* How fast the CUs take in bytes that sit in the L2: one workgroup of `waves` waves per CU, every workgroup
+ * reads the same `bytes` at `buf` (device memory, a multiple of in_flight KiB, at most 1 GiB) `iters` times with
+ * 1 KiB per wave instruction and `in_flight` (4, 8 or 16) instructions outstanding per wave; nothing is stored.
+ * Bytes into the CUs = CUs * bytes * iters. */
+int cybq_debug_cache_read(cybq_ctx* ctx, const void* buf, int64_t bytes, int waves, int in_flight, int iters, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

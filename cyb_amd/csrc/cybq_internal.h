@@ -44,13 +44,15 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
                        int num_cus, bool exact, void* workspace, size_t workspace_bytes, const Epilogue& epi,
                        hipStream_t st);
 
-// few rows (33 .. 64 on an output wide enough, 65 .. 128 on a narrow one), FAST mode, activations already staged as f16 operands
+// few rows (17 .. 64 on an output wide enough, up to 512 on a narrow one), FAST mode, activations already staged as f16 operands
 // (gemm_rows.hip); ssq_part / ssq_blocks / unscale: the staging pass's per-row statistics
 bool gemm_rows_serves(const WeightView& w, int M, int num_cus, const Epilogue& epi);
 hipError_t launch_gemm_rows(const WeightView& w, const void* x_staged, int M, void* y, int ydt, const Epilogue& epi,
                             const float* ssq_part, int ssq_blocks, const float* unscale, int num_cus, hipStream_t st);
 // test/bench hook: 2 = never take the few-rows kernel, 1 = whatever the width, 0 = automatic
 void set_gemm_tuning(int rows_kernel);
+// whether launch_gemm hands a FAST-mode call of M rows with this epilogue to the few-rows kernel (the hook included)
+bool gemm_rows_takes(const WeightView& w, int M, int num_cus, const Epilogue& epi);
 
 hipError_t launch_quantize(int bits, const float* src, int N, int K, void* q_out, void* s_out,
                            hipStream_t st);
@@ -72,6 +74,7 @@ hipError_t launch_read_probe(const WeightView& w, bool io, const void* x, void* 
 // other pure-read patterns over the same bytes (pattern 1 .. 6, see cybq_debug.h)
 hipError_t launch_read_pattern(const WeightView& w, int pattern, int num_cus, hipStream_t st);
 hipError_t launch_mfma_loop(int num_cus, int waves_per_simd, int iters, float* sink, hipStream_t st);
+hipError_t launch_cache_read(const void* buf, int64_t bytes, int waves, int in_flight, int iters, int num_cus, hipStream_t st);
 
 // test/bench hook: overrides the decode kernel's launch heuristics (0 = automatic)
 void set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll);

@@ -170,7 +170,46 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int iters, float* __rest
     if (t == 12345.678f) sink[0] = t;
 }
 
+// every workgroup reads the same `pieces` KiB `iters` times, one KiB per wave instruction, U instructions in
+// flight per wave; wave w takes the pieces w * U .., (w + waves) * U .., every workgroup starts elsewhere
+template <int U>
+__global__ __launch_bounds__(1024) void cache_read_kernel(const u32x4_t* __restrict__ p, int pieces, int iters, float* __restrict__ sink)
+{
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int start = (int)((blockIdx.x * 7u) % (unsigned)pieces);
+    uint32_t acc = 0;
+    for (int it = 0; it < iters; it++) {
+        for (int q0 = wv * U; q0 < pieces; q0 += nw * U) {
+            u32x4_t v[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                int q = q0 + u + start;
+                if (q >= pieces) q -= pieces;
+                v[u] = p[(size_t)q * 64 + lane];
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) acc ^= v[u][0] ^ v[u][1] ^ v[u][2] ^ v[u][3];
+        }
+        asm volatile("" ::: "memory");
+    }
+    if (acc == 0x12345679u && sink) sink[0] = 1.f;
+}
+
 }  // namespace
+
+hipError_t launch_cache_read(const void* buf, int64_t bytes, int waves, int in_flight, int iters, int num_cus, hipStream_t st)
+{
+    if (!buf || bytes < 1024 || bytes % ((int64_t)in_flight * 1024) || bytes > ((int64_t)1 << 30) || waves < 1 || waves > 16 || iters < 1)
+        return hipErrorInvalidValue;
+    const u32x4_t* p = reinterpret_cast<const u32x4_t*>(buf);
+    const int pieces = (int)(bytes / 1024);
+    const dim3 grid((unsigned)num_cus), block((unsigned)waves * 64);
+    if (in_flight == 4) hipLaunchKernelGGL((cache_read_kernel<4>), grid, block, 0, st, p, pieces, iters, (float*)nullptr);
+    else if (in_flight == 8) hipLaunchKernelGGL((cache_read_kernel<8>), grid, block, 0, st, p, pieces, iters, (float*)nullptr);
+    else if (in_flight == 16) hipLaunchKernelGGL((cache_read_kernel<16>), grid, block, 0, st, p, pieces, iters, (float*)nullptr);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
 
 hipError_t launch_read_probe(const WeightView& w, bool io, const void* x, void* y, hipStream_t st)
 {

@@ -968,6 +968,11 @@ __global__ __launch_bounds__(1024) void stage_rows_kernel(const void* __restrict
 int g_rows_kernel = 0;        // (set_gemm_tuning: 2 = experiments switch the few-rows kernel off, 1 = on whatever the width)
 void set_gemm_tuning(int rows_kernel) { g_rows_kernel = rows_kernel; }
 
+bool gemm_rows_takes(const WeightView& w, int M, int num_cus, const Epilogue& epi)
+{
+    return g_rows_kernel != 2 && gemm_rows_serves(w, M, g_rows_kernel == 1 ? 1 : num_cus, epi);
+}
+
 hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
                        int num_cus, bool exact, void* workspace, size_t workspace_bytes, const Epilogue& epi,
                        hipStream_t st)
@@ -1036,7 +1041,7 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         // few rows on a wide output, FAST mode: the kernel of gemm_rows.hip (waves split K, no LDS on the way)
-        if (!exact && kdt == kF16 && g_rows_kernel != 2 && gemm_rows_serves(w, mc, g_rows_kernel == 1 ? 1 : num_cus, ec)) {
+        if (!exact && kdt == kF16 && gemm_rows_takes(w, mc, num_cus, ec)) {
             e = launch_gemm_rows(w, workspace, mc, yc, ydt, ec, ns.part, ns.nblk, ns.unscale, g_rows_kernel == 1 ? 1 : num_cus, st);
             if (e != hipSuccess) return e;
             continue;

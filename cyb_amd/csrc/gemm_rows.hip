@@ -77,7 +77,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVE
 {
     const WeightView w = {wbase, N_, K_, NT_, KT_, BITS};
     constexpr int FR = MF * NF;                        // accumulator blocks per wave
-    static_assert(DEPTH % XD == 0 && MF == 4, "shape");
+    static_assert(DEPTH % XD == 0 && MF >= 1 && MF <= WAVES, "shape");
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     float4_t* part = reinterpret_cast<float4_t*>(smem);                                    // [WAVES][FR][64]
     float* stg = reinterpret_cast<float*>(smem + (size_t)WAVES * FR * 1024);               // [MF][16 * NF * 16]
@@ -199,22 +199,23 @@ hipError_t launch_rows_t(const WeightView& w, const void* x, int M, void* y, int
 
 }  // namespace
 
-// Column blocks per workgroup (4 or 2) for a call of M rows, or 0 when the kernel does not take it.
-// A call takes about 1.6 us per K tile of a wave whatever the number of workgroups (4096 -> 8192 at 64 rows, 128
-// workgroups: 16.6 us against 20.9 for the tiled kernels; 4096 -> 14336, 224: 18.1 against 21.5), so: one round
-// of workgroups, at least half a round, K of 16 .. 64 tiles (beyond that the tiled kernels split K over
-// workgroups: 14336 -> 4096 33.6 against 43 us here).  65 .. 128 rows are two workgroups per column tile (64
-// rows each): narrow outputs only, where both halves fit one round.
+// Column blocks per workgroup (1, 2 or 4) for a call of M rows, or 0 when the kernel does not take it.
+// A call takes about 1.6 us per K tile of a wave whatever the number of workgroups, and less per K tile the fewer
+// column blocks a wave carries, so: the fewest column blocks that still fit one round of workgroups
+// (4096 -> 4096 at 128 rows: 256 workgroups of two column blocks 14.3 us, 128 of four 17.0; 4096 -> 2048 at 24
+// rows: 128 of one 11.6, the tiled kernels 17.5), at least a quarter of a round (4096 -> 1024 at 24 rows, 64
+// workgroups: 11.4 against 17.4), K of 16 .. 64 tiles (beyond that the tiled kernels split K over workgroups:
+// 14336 -> 4096 33.6 against 43 us here).  More than 64 rows are one workgroup per 64 rows and column group:
+// narrow outputs only, where all of them fit one round.
 int rows_column_blocks(const WeightView& w, int M, int num_cus, const Epilogue& epi)
 {
-    if (M <= 16 || M > 512 || epi.kind == kEpiSwiglu || w.KT < 16 || w.KT > 64) return 0;      // (17 .. 32 rows get here as fp32 rows)
+    if (M <= 16 || M > 512 || epi.kind == kEpiSwiglu || w.KT < 16 || w.KT > 64) return 0;
     const int64_t parts = (M + 63) / 64;
-    for (int nf : {4, 2}) {
+    for (int nf : {1, 2, 4}) {
         const int64_t groups = (w.NT + nf - 1) / nf * parts;
-        if (groups <= num_cus && groups * 2 >= num_cus) return nf;
-        if (nf == 4 && parts == 1 && groups * 2 >= num_cus) return nf;       // (up to 64 rows a wide output may take more than one round)
+        if (groups <= num_cus) return groups * 4 >= num_cus ? nf : 0;
     }
-    return 0;
+    return parts == 1 ? 4 : 0;       // (up to 64 rows a wide output may take more than one round)
 }
 
 bool gemm_rows_serves(const WeightView& w, int M, int num_cus, const Epilogue& epi)
@@ -233,12 +234,22 @@ hipError_t launch_gemm_rows(const WeightView& w, const void* x_staged, int M, vo
     // X two / four K tiles ahead 21.7 / 20.4; eight weight tiles ahead 23.9; MFMAs and dequantisation
     // interleaved by scheduling hints 21.2; four staging + four multiplying waves sharing K slots through
     // LDS 26.7.
-    if (nf == 2) {
-        if (w.bits == 8) return launch_rows_t<8, 4, 2, 4, 4, 1>(w, x_staged, M, y, ydt, epi, ns, st);
-        return launch_rows_t<4, 4, 2, 4, 4, 1>(w, x_staged, M, y, ydt, epi, ns, st);
-    }
-    if (w.bits == 8) return launch_rows_t<8, 4, 4, 4, 4, 1>(w, x_staged, M, y, ydt, epi, ns, st);
-    return launch_rows_t<4, 4, 4, 4, 4, 1>(w, x_staged, M, y, ydt, epi, ns, st);
+    // Up to 48 rows the workgroup carries two or three row blocks instead of four: the rows of X are most of what
+    // a CU takes in, and its L1 delivers 64 bytes a cycle.
+    const int mf = M > 48 ? 4 : M > 32 ? 3 : 2;
+    auto go = [&](auto bits, auto nfc) {
+        constexpr int B = decltype(bits)::value, F = decltype(nfc)::value;
+        if (mf == 2) return launch_rows_t<B, 2, F, 4, 4, 1>(w, x_staged, M, y, ydt, epi, ns, st);
+        if (mf == 3) return launch_rows_t<B, 3, F, 4, 4, 1>(w, x_staged, M, y, ydt, epi, ns, st);
+        return launch_rows_t<B, 4, F, 4, 4, 1>(w, x_staged, M, y, ydt, epi, ns, st);
+    };
+    auto with_bits = [&](auto nfc) {
+        if (w.bits == 8) return go(std::integral_constant<int, 8>{}, nfc);
+        return go(std::integral_constant<int, 4>{}, nfc);
+    };
+    if (nf == 1) return with_bits(std::integral_constant<int, 1>{});
+    if (nf == 2) return with_bits(std::integral_constant<int, 2>{});
+    return with_bits(std::integral_constant<int, 4>{});
 }
 
 }  // namespace cybq

@@ -799,18 +799,18 @@ def test_prefill_role_split_kernel(backend, oracle, bits, shape):
 @pytest.mark.parametrize("shape", [(14336, 2048, 64), (8200, 4096 + 128, 33), (8198, 4096 + 256, 47), (14336, 4096, 48),
                                    (28672, 2048, 40), (8192, 8192, 64),
                                    (4096, 4096, 128), (6144 - 16, 4096 + 128, 100), (1024, 4096, 512), (2048, 4096, 300),
-                                   (4102, 8192, 70), (8192, 2048, 65)])
+                                   (4102, 8192, 70), (8192, 2048, 65),
+                                   (1024, 4096 + 128, 60), (4096, 4096, 64), (1030, 2048, 130)])
 def test_prefill_few_rows_waves_split_k(backend, oracle, bits, shape):
-    """FAST mode, K of 16 .. 64 tiles, one round of workgroups that is at least half full: the kernel whose
+    """FAST mode, K of 16 .. 64 tiles, one round of workgroups that is at least a quarter full: the kernel whose
     four waves split K and share nothing until the end (no LDS on the way, one partial-sum exchange).  33 .. 64
     rows on outputs from 8192 columns (more than a round of workgroups on the widest); from (4096, 4096, 128)
-    on, narrow outputs with up to 512 rows: two to eight workgroups of 64 rows per column tile, two or four
-    column blocks wide, a ragged last row part.  K tile counts that do not divide by four (waves with unequal
-    shares), N that ends inside a column block with rows of y aligned and not, every activation and output
-    type, residual add, folded RMSNorm; the tiled kernels (the same call with the kernel switched off) agree
-    within the mode's tolerance; a row's bits do not depend on the rows it travels with; reproducible.
-    (Up to 64 rows only weights of more than 6144 x 4096 elements get here: smaller ones take two passes of
-    the batched-rows decode kernel.)"""
+    on, narrow outputs with up to 512 rows: one to eight workgroups of 64 rows per column group, one, two or
+    four column blocks wide (the last three shapes: one), a ragged last row part.  K tile counts that do not
+    divide by four (waves with unequal shares), N that ends inside a column block with rows of y aligned and
+    not, every activation and output type, residual add, folded RMSNorm; the other kernels (the same call with
+    this kernel switched off: the tiled ones, or two decode passes on a small weight at up to 64 rows) agree
+    within the mode's tolerance; a row's bits do not depend on the rows it travels with; reproducible."""
     N, K, M = shape
     q, s = _quant(oracle, bits, N, K, cfg=61)
     qw = backend.upload_quantized(q, s, bits)
