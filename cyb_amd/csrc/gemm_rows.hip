@@ -1,30 +1,39 @@
-// gemm_rows.hip - prefill kernel for calls whose 64-row x 32/64-column pieces fill one round of workgroups
-// (17 .. 64 rows on wide outputs - up to 32 they are fp32 rows -, up to 512 rows on narrow ones), FAST mode
-// (f16 operands).
+// gemm_rows.hip - prefill kernel for calls whose 64-row x 16/32/64-column pieces fill one round of workgroups
+// (17 .. 64 rows on outputs from 1024 columns up - up to 32 they are fp32 rows -, up to 512 rows on narrow ones),
+// FAST mode (f16 operands).
 //
 // With so little work per CU (64 rows x 56 columns at N = 14336) what the tiled kernels of gemm.hip spend
 // per K tile - a barrier, every weight operand read from LDS by every multiplying wave - no longer hides
 // behind arithmetic: their K loop costs 0.45 - 0.6 us per K tile whatever the tile holds, and narrow outputs
 // make them split K over workgroups and add the slabs in a second pass.
 //
-// Here the waves of a workgroup share nothing until the end.  The workgroup owns 64 rows (blockIdx.y: which)
-// and NF column blocks of 16; wave w takes the K tiles w, w + WAVES, ... and, for those, multiplies ALL its
-// rows against ALL its column blocks (MF x NF accumulator blocks per wave).  A weight tile is then needed
-// by exactly one wave: global memory -> registers -> dequantised in registers (round_f16(scale * q), the
-// operand of FAST mode) -> MFMA B operand, no LDS, no barrier; and every row of X enters the CU once
-// (staged operand order, 1 KB per load) and meets all NF column blocks from registers.  One wave per SIMD
-// owns the register file (accumulators, a K tile of X and four K tiles of packed weights in flight).  At
-// the end the waves' partial sums meet through LDS and are added in wave order (fixed order: results are
-// reproducible and a row's bits do not depend on the other rows of the batch).
+// Here the waves of a workgroup share nothing until the end.  The workgroup owns MF row blocks of 16
+// (blockIdx.y: which) and NF column blocks of 16; wave w takes the K tiles w, w + WAVES, ... and, for those,
+// multiplies ALL its rows against ALL its column blocks (MF x NF accumulator blocks per wave).  A weight tile
+// is then needed by exactly one wave: global memory -> registers -> dequantised in registers
+// (round_f16(scale * q), the operand of FAST mode) -> MFMA B operand, no LDS, no barrier; and every row of X
+// enters the CU once (staged operand order, 1 KB per load) and meets all NF column blocks from registers.  One
+// wave per SIMD owns the register file (accumulators, a K tile of X and four K tiles of packed weights in
+// flight).  At the end the waves' partial sums meet through LDS and are added in wave order (fixed order:
+// results are reproducible and a row's bits do not depend on the other rows of the batch).
 //
-// A call costs about 1.6 us per K tile of a wave, nearly whatever the number of workgroups, so the kernel
-// takes every call whose workgroups fit one round and fill at least half of it (and up to 64 rows also the
-// widest outputs, in several rounds).  Per call with the staging pass, bf16 rows, against the tiled kernels:
-//   4096 -> 14336 at 33 .. 64 rows   18.1 - 19.1 us against 21.5 - 22.1      4096 -> 28672   31 - 33 against 38 - 39
-//   4096 ->  8192 at 33 .. 64 rows   16.4 - 17.3 against 20.6 - 21.2          8192 -> 14336   30 - 32 against 36.5 - 38
-//   4096 ->  4096 at 65 .. 128 rows  16.4 - 17.2 against 21.6 - 25.5          129 .. 256 rows  17.1 - 20.0 against 21.9 - 22.3
-//   4096 ->  6144 at 65 .. 128 rows  16.6 - 17.5 against 23.4 - 26.8          4096 -> 2048 at 100 .. 300 rows  13.6 - 18.9 against 20.1 - 29.1
-//   4096 ->  1024 at 256 .. 512 rows 15.1 - 20.7 against 21.6 - 27.6
+// What bounds it is what a CU takes in: all its rows of X (512 KB for 64 rows at K = 4096) plus its column
+// blocks' weights, through an L1 that delivers 64 bytes a cycle (a workgroup per CU that does nothing but read
+// the same 512 KB with 1-KB wave instructions reaches 21 - 31 TB/s over the chip with four waves, 33 with
+// eight; this kernel takes in 156 MB in 16 us).  Hence: the fewest column blocks that still fit one round of
+// workgroups, and only as many row blocks as the call has (two or three up to 48 rows: a row block costs
+// 1.1 - 1.3 us).  Per call with the staging pass, bf16 rows, against the tiled kernels (up to 64 rows on small
+// weights: against two passes of the batched-rows decode kernel):
+//   4096 -> 14336 at 33 .. 48 / 64 rows  17.8 / 19.1 us against 21.5 / 22.1   4096 -> 28672   31 - 33 against 38 - 39
+//   4096 ->  8192 at 33 / 64 / 128 rows  13.3 / 14.7 / 19.5 against 20.6 / 21.2 / 25.5
+//   4096 ->  4096 at 64 / 128 / 256 rows 12.8 / 14.3 / 19.8 against 14.5 / 25.5 / 22.3
+//   4096 ->  6144 at 64 / 128 rows       14.3 / 17.6 against 19.3 / 26.8     8192 -> 14336 at 33 .. 64 rows 30 - 32 against 36.5 - 38
+//   4096 ->  1024 at 128 / 256 / 512 rows 12.9 / 14.2 / 20.7 against 18.7 / 21.6 / 27.6
+//   fp32 rows, 17 .. 32: 4096 -> 14336 15.9 against 21, 4096 -> 4096 10.7 against 18
+// The same kernel on v_mfma_f32_32x32x16_f16 (one wave per SIMD issues a 16x16x32 MFMA only every ~30 cycles, a
+// 32x32x16 one back to back; both operands load in that shape from the same layouts as four 256-byte runs) measured
+// the same to 0.3 us on every shape: the MFMAs are a quarter of a wave's cycles.  Two workgroups of two column
+// blocks per CU (two waves per SIMD, twice the rows of X into every CU): 23.9 against 19.6 us.
 // With eight row blocks per wave (65 .. 128 rows in one workgroup, for wide outputs whose 64-row pieces would
 // need two rounds) a wave has twice the MFMAs to issue per K tile next to the same dequantisation and the
 // kernel is no quicker than the tiled one (X a whole K tile ahead: the operands no longer fit the register
@@ -68,7 +77,7 @@ __device__ __forceinline__ void dequant_group(const WRegs<BITS>& r, int j, uint3
     for (int p = 0; p < 4; p++) b.u[p] = as_u32(as_h2(bw[p]) * s2);
 }
 
-// MF = 4 row blocks of 16 per workgroup (blockIdx.y-th 64 rows of the call), NF column blocks per workgroup, WAVES
+// MF row blocks of 16 per workgroup (blockIdx.y-th MF * 16 rows of the call), NF column blocks per workgroup, WAVES
 // waves that split K, DEPTH K tiles of packed weights and XD K tiles of X in flight per wave.
 template <int BITS, int MF, int NF, int WAVES, int DEPTH, int XD>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVES / 4, WAVES / 4))) void gemm_rows_kernel(
