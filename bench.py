@@ -417,6 +417,11 @@ def main():
         tm = min(timer.once(lambda: be.debug_mfma_loop(2, 20000, sink, stream)) for _ in range(3))
         cus = torch.cuda.get_device_properties(0).multi_processor_count
         mfma_tfl = cus * 4 * 2 * 20000 * 16 * 16384 / tm / 1e12
+        # the same loop from ONE wave per SIMD, and that wave on 32x32x16 instructions (twice the flops each)
+        tm1 = min(timer.once(lambda: be.debug_mfma_loop(1, 20000, sink, stream)) for _ in range(3))
+        tm32 = min(timer.once(lambda: be.debug_mfma_loop(0, 20000, sink, stream)) for _ in range(3))
+        mfma1_tfl = cus * 4 * 1 * 20000 * 16 * 16384 / tm1 / 1e12
+        mfma32_tfl = cus * 4 * 20000 * 8 * 32768 / tm32 / 1e12
         extra["prefill_gemm_M512"] = {
             "workload": "Q4 prefill GEMM, M=512, K=4096 -> N=14336, X bf16, Y f32 (BASELINE configs[3]), weights rotating "
                         "through HBM; per call = activation staging pass + multiply",
@@ -427,7 +432,9 @@ def main():
                 "torch_matmul_bf16_dense_512x4096x14336_us": round(dense_us, 1),
                 "torch_matmul_bf16_dense_tflops": round(2.0 * Mp * N * K / (dense_us * 1e-6) / 1e12, 1),
                 "pure_mfma_f16_loop_tflops": round(mfma_tfl, 1),
-                "pure_mfma_loop_frac_of_published_peak": round(mfma_tfl / MFMA_BF16_PEAK_TFLOPS, 4)}}
+                "pure_mfma_loop_frac_of_published_peak": round(mfma_tfl / MFMA_BF16_PEAK_TFLOPS, 4),
+                "pure_mfma_f16_loop_one_wave_per_simd_tflops": round(mfma1_tfl, 1),
+                "pure_mfma_32x32x16_loop_one_wave_per_simd_tflops": round(mfma32_tfl, 1)}}
         log(f"prefill GEMM M=512: {elp * 1e6:.1f} us, {tfl:.1f} TFLOP/s, rel_l2 {relp:.2e}; dense bf16 {dense_us:.1f} us; "
             f"MFMA loop {mfma_tfl:.0f} TFLOP/s")
 

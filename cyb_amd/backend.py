@@ -434,7 +434,8 @@ class Backend:
         self._check(self._lib.cybq_debug_read_pattern(self._ctx, plan.count, plan.w, pattern, stream))
 
     def debug_mfma_loop(self, waves_per_simd: int, iters: int, sink, stream: int = 0) -> None:
-        """Diagnostics: `iters` x 16 independent v_mfma_f32_16x16x32_f16 per wave on every SIMD."""
+        """Diagnostics: `iters` x 16 independent v_mfma_f32_16x16x32_f16 per wave on every SIMD
+        (waves_per_simd = 0: one wave per SIMD, `iters` x 8 v_mfma_f32_32x32x16_f16)."""
         self._check(self._lib.cybq_debug_mfma_loop(self._ctx, waves_per_simd, iters, _ptr(sink), stream))
 
     def debug_cache_read(self, buf, nbytes: int, waves: int, in_flight: int, iters: int, stream: int = 0) -> None:

@@ -48,7 +48,9 @@ int cybq_debug_read_weight(cybq_ctx* ctx, int64_t count, const cybq_weight* cons
 int cybq_debug_read_pattern(cybq_ctx* ctx, int64_t count, const cybq_weight* const* w, int pattern, void* stream);
 
 /* A loop of independent v_mfma_f32_16x16x32_f16 on every SIMD of the chip: `waves_per_simd`
- * waves each issue `iters` x 16 instructions.  flops = CUs * 4 * waves_per_simd * iters * 16 * 16384. */
+ * waves each issue `iters` x 16 instructions.  flops = CUs * 4 * waves_per_simd * iters * 16 * 16384.
+ * waves_per_simd = 0: one wave per SIMD issues `iters` x 8 independent v_mfma_f32_32x32x16_f16 instead
+ * (flops = CUs * 4 * iters * 8 * 32768). */
 int cybq_debug_mfma_loop(cybq_ctx* ctx, int waves_per_simd, int iters, float* sink, void* stream);
 
 /* How fast the CUs take in bytes that sit in the L2: one workgroup of `waves` waves per CU, every workgroup

@@ -170,6 +170,29 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int iters, float* __rest
     if (t == 12345.678f) sink[0] = t;
 }
 
+typedef float float16v_t __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void mfma32_loop_kernel(int iters, float* __restrict__ sink)
+{
+    Frag16 a, b;
+    const uint32_t one2 = 0x3C003C00u;
+    a.u = (u32x4_t){one2, one2, one2, one2};
+    b.u = (u32x4_t){threadIdx.x, one2, one2, one2};
+    float16v_t acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[i][e] = 0.f;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.h, b.h, acc[i], 0, 0, 0);
+    }
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) t += acc[i][0];
+    if (t == 12345.678f) sink[0] = t;
+}
+
 // every workgroup reads the same `pieces` KiB `iters` times, one KiB per wave instruction, U instructions in
 // flight per wave; wave w takes the pieces w * U .., (w + waves) * U .., every workgroup starts elsewhere
 template <int U>
@@ -267,6 +290,10 @@ hipError_t launch_read_pattern(const WeightView& w, int pattern, int num_cus, hi
 
 hipError_t launch_mfma_loop(int num_cus, int waves_per_simd, int iters, float* sink, hipStream_t st)
 {
+    if (waves_per_simd == 0 && iters >= 1) {          // one wave per SIMD, 32x32x16: iters x 8 instructions of twice the flops
+        hipLaunchKernelGGL(mfma32_loop_kernel, dim3((unsigned)num_cus), dim3(256), 0, st, iters, sink);
+        return hipGetLastError();
+    }
     if (waves_per_simd < 1 || waves_per_simd > 8 || iters < 1) return hipErrorInvalidValue;
     // 256 threads = one wave per SIMD of a CU; waves_per_simd such workgroups per CU
     hipLaunchKernelGGL(mfma_loop_kernel, dim3((unsigned)(num_cus * waves_per_simd)), dim3(256), 0, st, iters, sink);

@@ -30,7 +30,7 @@
 //   4096 ->  6144 at 64 / 128 rows       14.3 / 17.6 against 19.3 / 26.8     8192 -> 14336 at 33 .. 64 rows 30 - 32 against 36.5 - 38
 //   4096 ->  1024 at 128 / 256 / 512 rows 12.9 / 14.2 / 20.7 against 18.7 / 21.6 / 27.6
 //   fp32 rows, 17 .. 32: 4096 -> 14336 15.9 against 21, 4096 -> 4096 10.7 against 18
-// The same kernel on v_mfma_f32_32x32x16_f16 (one wave per SIMD issues a 16x16x32 MFMA only every ~30 cycles, a
+// The same kernel on v_mfma_f32_32x32x16_f16 (one wave per SIMD issues a 16x16x32 MFMA only every ~27 cycles, a
 // 32x32x16 one back to back; both operands load in that shape from the same layouts as four 256-byte runs) measured
 // the same to 0.3 us on every shape: the MFMAs are a quarter of a wave's cycles.  Two workgroups of two column
 // blocks per CU (two waves per SIMD, twice the rows of X into every CU): 23.9 against 19.6 us.
