@@ -440,7 +440,7 @@ def main():
 
         # ---- the same call at other row counts (bf16 activations, weights rotating through HBM)
         rows_out = {}
-        for Mr in (64, 128, 256, 1024, 2048):
+        for Mr in (40, 64, 128, 256, 1024, 2048):
             xr = torch.from_numpy(synth.activations(4, Mr, K)).to(dev).to(torch.bfloat16)
             yr = torch.empty((Mr, N), dtype=torch.float32, device=dev)
             nr = 50 if Mr <= 256 else 12
@@ -596,7 +596,7 @@ def main():
         for Nx in (4096, 6144, 1024):
             qs_, ss_ = formats.quantize(synth.weights(2, Nx, K), bits)
             wsm = copies_of(qs_, ss_, bits)
-            for Mr in (128, 256):
+            for Mr in (40, 64, 128, 256):
                 xr = torch.from_numpy(synth.activations(4, Mr, K)).to(dev).to(torch.bfloat16)
                 yr = torch.empty((Mr, Nx), dtype=torch.float32, device=dev)
                 nr = 100
