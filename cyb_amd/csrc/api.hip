@@ -490,17 +490,18 @@ int matmul_fused(cybq_ctx* ctx, const cybq_weight* w, const void* x, cybq_dtype 
         if (e == hipSuccess)
             e = cybq::launch_gemv(v, static_cast<const char*>(x) + (size_t)32 * w->K * dtype_size(xdt), xdt, (int)M - 32,
                                   static_cast<char*>(y) + yoff, ydt, ctx->num_cus, exact_ops, ec, dscr, dscr_bytes, st);
-    } else if (!weight_is_wide(w) && (xdt == CYBQ_F32 ? !ctx->prefill_exact : M > 32)) {
+    } else if (!weight_is_wide(w) && (xdt == CYBQ_F32 ? !ctx->prefill_exact : (M > 32 || (!ctx->prefill_exact && cybq::gemm_rows_takes(v, (int)M, ctx->num_cus, epi))))) {
         e = cybq::launch_gemm(v, x, xdt, (int)M, y, ydt, ctx->num_cus, ctx->prefill_exact, workspace, workspace_bytes,
                               epi, st);
     } else {
         // fp32 activations keep full precision through the decode kernel's hi/lo split:
         // exact-mode prefill in fp32 is walked 16 rows at a time (FAST mode rounds them to f16
         // in the staging pass and takes the MFMA kernel from 17 rows on: the LDS decode kernel
-        // needs 52 - 65 us for 24 - 32 fp32 rows, the MFMA kernel 31).  So are 17..32
-        // rows of 16-bit activations with a folded norm: two passes of the batched-rows
-        // kernel stream the weights twice and are still quicker than a 128-row MFMA tile
-        // mostly empty (without the norm they are one pass, two row blocks per weight operand).
+        // needs 52 - 65 us for 24 - 32 fp32 rows, the few-row MFMA kernel 16).  So are 17..32
+        // rows of 16-bit activations with a folded norm where the few-row MFMA kernel does not take
+        // them (FAST mode: 4096 -> 14336 at 32 rows 18.1 us there against 23.0 here): two passes of
+        // the batched-rows kernel stream the weights twice and are still quicker than a 128-row MFMA
+        // tile mostly empty (without the norm they are one pass, two row blocks per weight operand).
         // A tensor with wide scales (scale * q leaves f16) is walked the same way for any M, 32 rows at a
         // time where the batched-rows kernel takes them in one pass: the weights stream once per 32 rows.
         e = hipSuccess;

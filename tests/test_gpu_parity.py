@@ -884,6 +884,52 @@ def test_prefill_fp32_rows_17_to_32_fast_mode(backend, oracle, shape):
     qw.free()
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("shape", [(14336, 4096, 32), (2064, 2048 + 128, 17), (4096, 8192, 25)])
+def test_folded_norm_17_to_32_rows_fast_mode(backend, oracle, bits, shape):
+    """17 .. 32 rows of 16-bit activations with a folded RMSNorm leave the one-pass decode kernel; in FAST mode,
+    where the shape fits, the staging pass folds gamma in and the kernel whose waves split K multiplies (two row
+    blocks per workgroup).  Against float64, against the two decode passes that take the call otherwise, with a
+    residual add, 16-bit outputs; reproducible; a row's bits do not depend on the rows it travels with."""
+    N, K, M = shape
+    q, s = _quant(oracle, bits, N, K, cfg=71)
+    qw = backend.upload_quantized(q, s, bits)
+    wd = torch.from_numpy(oracle.dequant(q, s)).cuda().double()
+    r = torch.from_numpy(synth.activations(73, M, N)).cuda()
+    try:
+        for xdt, gdt, ydt in (("bf16", torch.float16, "f32"), ("f16", torch.float32, "bf16"), ("bf16", torch.bfloat16, "f16")):
+            x = _x(M, K, xdt, cfg=72)
+            gamma = (1.0 + 0.1 * torch.from_numpy(synth.activations(74, 1, K))[0]).cuda().to(gdt)
+            xd = x.double()
+            ref = (xd * torch.rsqrt((xd * xd).mean(dim=1, keepdim=True) + 1e-5) * gamma.double()) @ wd.T
+            bar = 2 * FAST if ydt == "f32" else 4e-3
+            y = torch.empty((M, N), dtype=TDT[ydt], device="cuda")
+            backend.matmul_norm(qw, x, gamma, 1e-5, y)
+            torch.cuda.synchronize()
+            assert ((y.double() - ref).norm() / ref.norm()).item() < bar, (xdt, ydt)
+            y_again = torch.empty_like(y)
+            backend.matmul_norm(qw, x, gamma, 1e-5, y_again)
+            backend.set_gemm_tuning(2)                                     # two passes of the batched-rows decode kernel
+            y_two = torch.empty_like(y)
+            backend.matmul_norm(qw, x, gamma, 1e-5, y_two)
+            backend.set_gemm_tuning(0)
+            fewer = torch.empty((17, N), dtype=TDT[ydt], device="cuda")
+            backend.matmul_norm(qw, x[:17].contiguous(), gamma, 1e-5, fewer)
+            y_add = torch.empty_like(y)
+            backend.matmul_norm(qw, x, gamma, 1e-5, y_add, epilogue="add", residual=r.to(TDT[ydt]))
+            torch.cuda.synchronize()
+            assert torch.equal(y, y_again)
+            assert ((y.double() - y_two.double()).norm() / ref.norm()).item() < 2 * bar, (xdt, ydt)
+            if ydt == "f32":
+                assert not torch.equal(y, y_two)                           # (rounded operands, another order: it did run)
+            assert torch.equal(y[:17], fewer)
+            want = ref + r.to(TDT[ydt]).double()
+            assert ((y_add.double() - want).norm() / want.norm()).item() < bar, (xdt, ydt)
+    finally:
+        backend.set_gemm_tuning(0)
+    qw.free()
+
+
 def test_lm_head_shape(backend, oracle):
     """The LM head of a Llama-3-sized vocabulary (decide/pipeline.md:51): 128256 rows, K = 4096, Q4 -
     8016 strips, several rounds of workgroups per CU.  Weights are made and quantised on the device;
