@@ -885,6 +885,58 @@ def test_prefill_fp32_rows_17_to_32_fast_mode(backend, oracle, shape):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("shape", [(7168, 4096, 48, "bf16"), (2048, 4096 + 128, 100, "f16"), (14336, 2048, 33, "bf16"),
+                                   (1040, 4096, 24, "f32"), (4096, 2048, 64, "bf16")])
+def test_prefill_few_rows_swiglu(backend, oracle, bits, shape):
+    """The SwiGLU epilogue of the kernel whose waves split K (FAST mode): a workgroup holds gate / up column blocks
+    in pairs and the wave that finishes a row block writes silu(gate) * up.  One workgroup per 64 rows, two row
+    parts, more than one round of workgroups, fp32 rows below 33, with a folded RMSNorm; against float64 and
+    against the tiled kernels on the same call."""
+    N, K, M, xdt = shape
+    qg, sg = _quant(oracle, bits, N, K, cfg=81)
+    qu, su = _quant(oracle, bits, N, K, cfg=82)
+    wg, wu = backend.upload_quantized(qg, sg, bits), backend.upload_quantized(qu, su, bits)
+    wf = backend.fuse_pairs(wg, wu)
+    dg = torch.from_numpy(oracle.dequant(qg, sg)).cuda().double()
+    du = torch.from_numpy(oracle.dequant(qu, su)).cuda().double()
+    try:
+        for ydt in ("f32", "bf16"):
+            x = _x(M, K, xdt, cfg=83)
+            g, u = x.double() @ dg.T, x.double() @ du.T
+            ref = g / (1.0 + torch.exp(-g)) * u
+            bar = 2 * FAST if ydt == "f32" else 6e-3
+            y = torch.full((M, N), float("nan"), dtype=TDT[ydt], device="cuda")
+            backend.matmul_ex(wf, x, y, "swiglu")
+            y_again = torch.empty_like(y)
+            backend.matmul_ex(wf, x, y_again, "swiglu")
+            backend.set_gemm_tuning(2)
+            y_tiled = torch.empty_like(y)
+            backend.matmul_ex(wf, x, y_tiled, "swiglu")
+            backend.set_gemm_tuning(0)
+            torch.cuda.synchronize()
+            assert not torch.isnan(y.float()).any()
+            assert ((y.double() - ref).norm() / ref.norm()).item() < bar, ydt
+            assert torch.equal(y, y_again)
+            assert ((y.double() - y_tiled.double()).norm() / ref.norm()).item() < 2 * bar, ydt
+            if ydt == "f32":
+                assert not torch.equal(y, y_tiled)                         # (another kernel: it did run)
+        x = _x(M, K, "bf16", cfg=84)
+        gamma = (1.0 + 0.1 * torch.from_numpy(synth.activations(85, 1, K))[0]).cuda()
+        xd = x.double()
+        xn = xd * torch.rsqrt((xd * xd).mean(dim=1, keepdim=True) + 1e-5) * gamma.double()
+        g, u = xn @ dg.T, xn @ du.T
+        ref = g / (1.0 + torch.exp(-g)) * u
+        y = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        backend.matmul_norm(wf, x, gamma, 1e-5, y, "swiglu")
+        torch.cuda.synchronize()
+        assert ((y.double() - ref).norm() / ref.norm()).item() < 4 * FAST
+    finally:
+        backend.set_gemm_tuning(0)
+    for t in (wf, wg, wu):
+        t.free()
+
+
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("shape", [(14336, 4096, 32), (2064, 2048 + 128, 17), (4096, 8192, 25)])
 def test_folded_norm_17_to_32_rows_fast_mode(backend, oracle, bits, shape):
     """17 .. 32 rows of 16-bit activations with a folded RMSNorm leave the one-pass decode kernel; in FAST mode,
