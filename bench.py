@@ -610,6 +610,28 @@ def main():
                 t.free()
             del wsm, qs_, ss_
         extra["prefill_attention_projections_bf16_rows"] = proj
+        # ---- the fused gate + up projection with the SwiGLU epilogue (4096 -> 2 x 14336) at a few rows
+        qg_, sg_ = formats.quantize(synth.weights(9, N, K), bits)
+        qu_, su_ = formats.quantize(synth.weights(10, N, K), bits)
+        wg_, wu_ = be.upload_quantized(qg_, sg_, bits), be.upload_quantized(qu_, su_, bits)
+        pair = be.fuse_pairs(wg_, wu_)
+        pairs = [pair] + [pair.clone() for _ in range(max(2, (3 * MALL_BYTES) // (2 * formats.weight_bytes(bits, N, K)) + 1) - 1)]
+        gu = {}
+        for Mr in (24, 40, 64):
+            xr = torch.from_numpy(synth.activations(4, Mr, K)).to(dev).to(torch.float32 if Mr < 33 else torch.bfloat16)
+            yr = torch.empty((Mr, N), dtype=torch.float32, device=dev)
+            nr = 60
+            rpl = be.plan_many([pairs[j % len(pairs)] for j in range(nr)], [xr] * nr, [yr] * nr, epilogues=["swiglu"] * nr)
+            be.matmul_many(rpl, Mr, stream)
+            tr, _ = timer.until(lambda i: be.matmul_many(rpl, Mr, stream), max_passes=40)
+            tr /= nr
+            gu[f"M{Mr}_{'f32' if Mr < 33 else 'bf16'}"] = {"us": round(tr * 1e6, 1), "tflops": round(2.0 * Mr * 2 * N * K / tr / 1e12, 1)}
+            del xr, yr, rpl
+        for t in pairs + [wg_, wu_]:
+            t.free()
+        del pairs, pair, wg_, wu_, qg_, sg_, qu_, su_
+        extra["prefill_gate_up_swiglu_4096x28672_rows"] = gu
+        log("gate + up with SwiGLU: " + " ".join(f"{k}:{v['us']}us" for k, v in gu.items()))
         log("attention projections: " + " ".join(f"{k}:{v['us']}us" for k, v in proj.items()))
         log("other BASELINE configs: " + " ".join(f"{k}:{v['us']}us" for k, v in base.items()))
 
