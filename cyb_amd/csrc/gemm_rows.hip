@@ -36,6 +36,9 @@
 // 32x32x16 one back to back; both operands load in that shape from the same layouts as four 256-byte runs) measured
 // the same to 0.3 us on every shape: the MFMAs are a quarter of a wave's cycles.  Two workgroups of two column
 // blocks per CU (two waves per SIMD, twice the rows of X into every CU): 23.9 against 19.6 us.
+// Eight column blocks per workgroup on 32x32x16 (64 rows x 128 columns: 65 .. 128 rows on 4096 -> 14336 in one round,
+// 0.8 MB into a CU instead of the tiled kernel's 1.15): 31.4 against 27.6 us at 128 rows, 30.3 against 24.5 at 65 -
+// one wave's MFMAs, dequantisation and loads then add up instead of overlapping.
 // With eight row blocks per wave (65 .. 128 rows in one workgroup, for wide outputs whose 64-row pieces would
 // need two rounds) a wave has twice the MFMAs to issue per K tile next to the same dequantisation and the
 // kernel is no quicker than the tiled one (X a whole K tile ahead: the operands no longer fit the register
