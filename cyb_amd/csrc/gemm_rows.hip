@@ -36,6 +36,10 @@
 // 32x32x16 one back to back; both operands load in that shape from the same layouts as four 256-byte runs) measured
 // the same to 0.3 us on every shape: the MFMAs are a quarter of a wave's cycles.  Two workgroups of two column
 // blocks per CU (two waves per SIMD, twice the rows of X into every CU): 23.9 against 19.6 us.
+// Two waves per SIMD (eight waves; wave (k share, half) takes two of the four scale groups of each of its K tiles:
+// half the X registers, half of every tile record, nothing loaded or dequantised twice, eight partial sums at the
+// end) is slower on every shape: 4096 -> 4096 at 64 rows 14.2 against 13.1 us, 4096 -> 8192 16.9 against 14.9,
+// 4096 -> 1024 at 128 rows 13.9 against 12.8 (and it spills with four column blocks).
 // Eight column blocks per workgroup on 32x32x16 (64 rows x 128 columns: 65 .. 128 rows on 4096 -> 14336 in one round,
 // 0.8 MB into a CU instead of the tiled kernel's 1.15): 31.4 against 27.6 us at 128 rows, 30.3 against 24.5 at 65 -
 // one wave's MFMAs, dequantisation and loads then add up instead of overlapping.
