@@ -46,6 +46,7 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
 
 // few rows (17 .. 64 on an output wide enough, up to 512 on a narrow one), FAST mode, activations already staged as f16 operands
 // (gemm_rows.hip); ssq_part / ssq_blocks / unscale: the staging pass's per-row statistics
+int gemm_rows_blocks(const WeightView& w, int M, int num_cus, const Epilogue& epi);
 bool gemm_rows_serves(const WeightView& w, int M, int num_cus, const Epilogue& epi);
 hipError_t launch_gemm_rows(const WeightView& w, const void* x_staged, int M, void* y, int ydt, const Epilogue& epi,
                             const float* ssq_part, int ssq_blocks, const float* unscale, int num_cus, hipStream_t st);

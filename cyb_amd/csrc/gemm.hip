@@ -731,6 +731,32 @@ hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt
     return hipErrorInvalidValue;
 }
 
+// The multiply that follows a staging launch starts on weights that come from HBM for the first time (2.4 of the
+// 14.5 us of a 64-row call on 4096 -> 14336 pass before its K loops start).  Extra workgroups of the staging launch,
+// which leaves most of the chip idle, ask for the first K tiles of every column group ahead of it - one dword per
+// 128-byte line, nothing kept: workgroup number b here asks for what workgroup b of the multiply reads first (the
+// hardware deals workgroups to the eight XCDs in turn, so with first_group a multiple of eight the lines land in
+// that workgroup's L2; anywhere else they land in the memory-side cache).
+struct Touch {
+    const uint8_t* base;          // the weight tensor (first_group past the grid: nothing to do)
+    int first_group, NT, KT, NF, tile_bytes, ahead;
+};
+
+__device__ __forceinline__ void touch_weights(const Touch& tc, int b, int tid, int nthreads)
+{
+    const int lines = (tc.tile_bytes + 127) >> 7;
+    const int kt0 = b % tc.KT;                     // (the multiply's workgroups start their K walk there)
+    uint32_t acc = 0;
+    for (int idx = tid; idx < tc.NF * tc.ahead * lines; idx += nthreads) {
+        const int line = idx % lines, ft = idx / lines, t = ft % tc.ahead, f = ft / tc.ahead;
+        const int nt = min(b * tc.NF + f, tc.NT - 1);
+        int kt = kt0 + t;
+        if (kt >= tc.KT) kt -= tc.KT;
+        acc ^= *reinterpret_cast<const uint32_t*>(tc.base + ((int64_t)nt * tc.KT + kt) * tc.tile_bytes + min(line * 128, tc.tile_bytes - 4));
+    }
+    asm volatile("" ::"v"(acc));                   // (the loads have to be issued and waited for; nothing is stored)
+}
+
 // X [M, K] row major (16-bit elements, used as they are) -> A-operand order: for row block rb
 // (16 rows, zero padded) and scale group g, 64 x 16 B where slot (oct, r) = oct*16 + r holds row
 // 16*rb + r, k = 32*g + 8*oct .. +8.  A workgroup moves one row block x 16 groups through LDS:
@@ -851,9 +877,14 @@ __device__ __forceinline__ void row_chunk_values(const RowChunk<XT>& c, float v[
 // most of it the latency of one wave walking its row.
 template <int XT, bool NORM, int CH>
 __global__ __launch_bounds__(1024) void stage_rows_kernel(const void* __restrict__ src, u32x4_t* __restrict__ dst, int M, int K,
-                                                          Epilogue epi, float* __restrict__ ssq, float* __restrict__ unscale)
+                                                          Epilogue epi, float* __restrict__ ssq, float* __restrict__ unscale, Touch touch)
 {
     static_assert(XT == 1 || XT == 2, "bf16 or fp32 activations");
+    if ((int)blockIdx.x >= touch.first_group) {
+        touch_weights(touch, (int)blockIdx.x - touch.first_group, (int)threadIdx.x, 1024);
+        return;
+    }
+    if ((int)(blockIdx.x >> 2) * 16 >= M) return;              // (padding up to first_group)
     constexpr int PW = 4;                                      // waves per row
     __shared__ u32x4_t tile[PW][2][4 * kStagePitch];
     __shared__ float amax_part[4][PW], sq_part[4][PW];
@@ -966,11 +997,33 @@ __global__ __launch_bounds__(1024) void stage_rows_kernel(const void* __restrict
 }  // namespace
 
 int g_rows_kernel = 0;        // (set_gemm_tuning: 2 = experiments switch the few-rows kernel off, 1 = on whatever the width)
-void set_gemm_tuning(int rows_kernel) { g_rows_kernel = rows_kernel; }
+int g_touch = 1;              // (5 = the staging launch asks for no weights ahead of the few-rows kernel)
+void set_gemm_tuning(int rows_kernel) { g_rows_kernel = rows_kernel == 5 ? 0 : rows_kernel; g_touch = rows_kernel != 5; }
 
 bool gemm_rows_takes(const WeightView& w, int M, int num_cus, const Epilogue& epi)
 {
     return g_rows_kernel != 2 && gemm_rows_serves(w, M, g_rows_kernel == 1 ? 1 : num_cus, epi);
+}
+
+// the extra workgroups of a staging launch (grid_x grows by them) when the few-row kernel takes a call of 33 rows
+// or more that goes through the row-scaling pass (bf16 / fp32 rows): up to 16 MB of the tensor, from the K tile every
+// column group starts at.  Per call: 4096 -> 14336 at 64 rows 19.6 -> 18.7 us with 16 of the 32 K tiles (no gain
+// with all of them: the launch then takes as long as the reads), 4096 -> 4096 at 64 / 128 rows 13.6 / 14.6 -> 12.4 /
+// 13.4, 4096 -> 1024 13.1 -> 11.7, 8192 -> 4096 at 128 rows 25.1 -> 22.9.  Not for f16 rows (their pass only
+// reorders and is over before the reads are: 4096 -> 14336 at 64 rows 18.6 -> 19.1), for 17 .. 32 fp32 rows (12.5 ->
+// 13.4 on 4096 -> 8192) or for K up to 2048.
+static Touch plan_touch(const WeightView& w, int mc, int num_cus, const Epilogue& ec, bool exact, unsigned& grid_x)
+{
+    Touch tc = {nullptr, 0x7fffffff, w.NT, w.KT, 1, tile_bytes(w.bits), 0};
+    if (g_touch == 0 || exact || mc < 33 || w.KT < 32 || !gemm_rows_takes(w, mc, num_cus, ec)) return tc;
+    const int nf = gemm_rows_blocks(w, mc, g_rows_kernel == 1 ? 1 : num_cus, ec);
+    const int64_t per_k_tile = (int64_t)w.NT * tile_bytes(w.bits);
+    tc.base = w.base;
+    tc.NF = nf;
+    tc.ahead = (int)std::min<int64_t>(w.KT, std::max<int64_t>(4, ((int64_t)16 << 20) / per_k_tile));
+    tc.first_group = (int)((grid_x + 7) / 8 * 8);
+    grid_x = (unsigned)(tc.first_group + (w.NT + nf - 1) / nf);
+    return tc;
 }
 
 hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void* y, int ydt,
@@ -1014,12 +1067,13 @@ hipError_t launch_gemm(const WeightView& w, const void* x, int xdt, int M, void*
         if (widen) {
             // per-row scaled f16 operands; one sum of squares per row
             ns = NormStats{ssq_part, 1, unscale};
-            const dim3 rgrid((unsigned)((mc + 15) / 16) * 4);
+            dim3 rgrid((unsigned)((mc + 15) / 16) * 4);
+            const Touch touch = plan_touch(w, mc, num_cus, ec, exact, rgrid.x);
             // pieces of 512 k a lane keeps in registers (a row is split over four waves): the whole row when it has
             // at most 16384 (bf16) or 8192 (fp32) elements
             const int batches = ((K8 + 63) / 64 + 3) / 4;
 #define CYBQ_STAGE_ROWS(XT, NORM, CH) \
-    hipLaunchKernelGGL((stage_rows_kernel<XT, NORM, CH>), rgrid, dim3(1024), 0, st, xs, xst, mc, w.K, epi, ssq_part, unscale)
+    hipLaunchKernelGGL((stage_rows_kernel<XT, NORM, CH>), rgrid, dim3(1024), 0, st, xs, xst, mc, w.K, epi, ssq_part, unscale, touch)
 #define CYBQ_STAGE_ROWS_CH(XT, NORM, C1, C2, C3)              \
     do {                                                      \
         if (batches <= C1) CYBQ_STAGE_ROWS(XT, NORM, C1);     \

@@ -249,6 +249,8 @@ int rows_column_blocks(const WeightView& w, int M, int num_cus, const Epilogue& 
     return parts == 1 ? 4 : 0;       // (up to 64 rows a wide output may take more than one round)
 }
 
+int gemm_rows_blocks(const WeightView& w, int M, int num_cus, const Epilogue& epi) { return rows_column_blocks(w, M, num_cus, epi); }
+
 bool gemm_rows_serves(const WeightView& w, int M, int num_cus, const Epilogue& epi)
 {
     return rows_column_blocks(w, M, num_cus, epi) != 0;
