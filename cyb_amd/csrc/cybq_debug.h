@@ -23,7 +23,8 @@ int cybq_debug_set_gemv_tuning(int waves_per_group, int rows_kernel, int unroll)
 /* Which prefill kernel takes calls of up to 512 rows in FAST mode: 0 automatic (the kernel whose waves
  * split K where its workgroups of up to 64 rows fit one round of CUs and fill a quarter of it), 1 that kernel for
  * up to 64 rows whatever the width, 2 never that kernel (the tiled kernels - on small weights at up to 64 rows two
- * passes of the batched-rows decode kernel - take the call as they do for other shapes). */
+ * passes of the batched-rows decode kernel - take the call as they do for other shapes); 5: automatic, but the
+ * staging launch asks for no weights ahead of the multiply; 6: automatic, it asks only ahead of that kernel. */
 int cybq_debug_set_gemm_tuning(int rows_kernel);
 
 /* Ceiling probes for the one-row decode kernel: a kernel that issues exactly that kernel's

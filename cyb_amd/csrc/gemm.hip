@@ -740,11 +740,16 @@ hipError_t launch_nf(const WeightView& w, const void* x, int M, void* y, int ydt
 struct Touch {
     const uint8_t* base;          // the weight tensor (first_group past the grid: nothing to do)
     int first_group, NT, KT, NF, tile_bytes, ahead;
+    int per_xcd, tiles;           // the tiled kernels' order: workgroup b works on column tile (b % 8) * per_xcd + b / 8 of `tiles` (0: on b)
 };
 
 __device__ __forceinline__ void touch_weights(const Touch& tc, int b, int tid, int nthreads)
 {
     const int lines = (tc.tile_bytes + 127) >> 7;
+    if (tc.per_xcd) {
+        b = (b & 7) * tc.per_xcd + (b >> 3);
+        if (b >= tc.tiles) return;
+    }
     const int kt0 = b % tc.KT;                     // (the multiply's workgroups start their K walk there)
     uint32_t acc = 0;
     for (int idx = tid; idx < tc.NF * tc.ahead * lines; idx += nthreads) {
@@ -997,32 +1002,54 @@ __global__ __launch_bounds__(1024) void stage_rows_kernel(const void* __restrict
 }  // namespace
 
 int g_rows_kernel = 0;        // (set_gemm_tuning: 2 = experiments switch the few-rows kernel off, 1 = on whatever the width)
-int g_touch = 1;              // (5 = the staging launch asks for no weights ahead of the few-rows kernel)
-void set_gemm_tuning(int rows_kernel) { g_rows_kernel = rows_kernel == 5 ? 0 : rows_kernel; g_touch = rows_kernel != 5; }
+int g_touch = 2;              // (5 = the staging launch asks for no weights ahead of the multiply, 6 = only ahead of the few-rows kernel)
+void set_gemm_tuning(int rows_kernel) { g_rows_kernel = rows_kernel >= 5 ? 0 : rows_kernel; g_touch = rows_kernel == 5 ? 0 : rows_kernel == 6 ? 1 : 2; }
 
 bool gemm_rows_takes(const WeightView& w, int M, int num_cus, const Epilogue& epi)
 {
     return g_rows_kernel != 2 && gemm_rows_serves(w, M, g_rows_kernel == 1 ? 1 : num_cus, epi);
 }
 
-// the extra workgroups of a staging launch (grid_x grows by them) when the few-row kernel takes a call of 33 rows
-// or more that goes through the row-scaling pass (bf16 / fp32 rows): up to 16 MB of the tensor, from the K tile every
-// column group starts at.  Per call: 4096 -> 14336 at 64 rows 19.6 -> 18.7 us with 16 of the 32 K tiles (no gain
-// with all of them: the launch then takes as long as the reads), 4096 -> 4096 at 64 / 128 rows 13.6 / 14.6 -> 12.4 /
-// 13.4, 4096 -> 1024 13.1 -> 11.7, 8192 -> 4096 at 128 rows 25.1 -> 22.9.  Not for f16 rows (their pass only
-// reorders and is over before the reads are: 4096 -> 14336 at 64 rows 18.6 -> 19.1), for 17 .. 32 fp32 rows (12.5 ->
-// 13.4 on 4096 -> 8192) or for K up to 2048.
+// the extra workgroups of a staging launch (grid_x grows by them) for a call of 33 rows or more that goes through the
+// row-scaling pass (bf16 / fp32 rows) and on to the few-row kernel or to the tiled kernels' 64-column tiles: up to
+// 16 MB of the tensor, from the K tile every column group starts at.  Per call: 4096 -> 14336 at 64 rows 19.6 -> 18.7
+// us with 16 of the 32 K tiles (no gain with all of them: the launch then takes as long as the reads), 4096 -> 4096
+// at 64 / 128 rows 13.6 / 14.6 -> 12.4 / 13.4, 4096 -> 1024 13.1 -> 11.7, 8192 -> 4096 at 128 rows 25.1 -> 22.9.  Not
+// for f16 rows (their pass only reorders and is over before the reads are: 4096 -> 14336 at 64 rows 18.6 -> 19.1),
+// for 17 .. 32 fp32 rows (12.5 -> 13.4 on 4096 -> 8192) or for K up to 2048.
+// whether launch_nf gives a FAST-mode call of M rows the 64-column tiles (one row tile of up to 128 rows)
+static bool few_rows_tiles64(const WeightView& w, int M, int num_cus, const Epilogue& epi)
+{
+    if (M > 128 || epi.kind == kEpiSwiglu) return false;
+    const int64_t tiles64 = (w.NT + 3) / 4;
+    return tiles64 * 4 >= 3 * num_cus || (tiles64 * 2 >= num_cus && w.KT <= 48);
+}
+
 static Touch plan_touch(const WeightView& w, int mc, int num_cus, const Epilogue& ec, bool exact, unsigned& grid_x)
 {
-    Touch tc = {nullptr, 0x7fffffff, w.NT, w.KT, 1, tile_bytes(w.bits), 0};
-    if (g_touch == 0 || exact || mc < 33 || w.KT < 32 || !gemm_rows_takes(w, mc, num_cus, ec)) return tc;
-    const int nf = gemm_rows_blocks(w, mc, g_rows_kernel == 1 ? 1 : num_cus, ec);
+    Touch tc = {nullptr, 0x7fffffff, w.NT, w.KT, 1, tile_bytes(w.bits), 0, 0, 0};
+    if (g_touch == 0 || exact || mc < 33 || w.KT < 32) return tc;
     const int64_t per_k_tile = (int64_t)w.NT * tile_bytes(w.bits);
+    int nf = 0, groups = 0;
+    if (gemm_rows_takes(w, mc, num_cus, ec)) {
+        nf = gemm_rows_blocks(w, mc, g_rows_kernel == 1 ? 1 : num_cus, ec);
+        groups = (w.NT + nf - 1) / nf;
+    } else if (g_touch >= 2 && per_k_tile * w.KT <= ((int64_t)40 << 20) && few_rows_tiles64(w, mc, num_cus, ec)) {
+        // the 128 x 64 / 64 x 64 tiles of the tiled kernels (65 .. 128 rows on wide outputs; 4096 -> 14336 at 128 rows:
+        // 27.5 us, 24.3 with the same tensor every call): 4096 -> 14336 at 65 / 100 / 128 rows 25.3 / 27.1 / 28.1 ->
+        // 23.9 / 26.0 / 27.3 us, 4096 -> 11008 23.9 / 25.5 / 26.5 -> 23.3 / 24.6 / 25.2; nothing on tensors of 66 MB
+        nf = 4;
+        tc.tiles = (w.NT + 3) / 4;
+        groups = (tc.tiles + 7) / 8 * 8;
+        tc.per_xcd = groups / 8;
+    } else {
+        return tc;
+    }
     tc.base = w.base;
     tc.NF = nf;
     tc.ahead = (int)std::min<int64_t>(w.KT, std::max<int64_t>(4, ((int64_t)16 << 20) / per_k_tile));
     tc.first_group = (int)((grid_x + 7) / 8 * 8);
-    grid_x = (unsigned)(tc.first_group + (w.NT + nf - 1) / nf);
+    grid_x = (unsigned)(tc.first_group + groups);
     return tc;
 }
 
