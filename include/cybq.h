@@ -74,10 +74,12 @@ typedef enum cybq_layout { CYBQ_LAYOUT_PLANAR = 0, CYBQ_LAYOUT_BLOCK_AOS = 1 } c
 
 typedef enum cybq_dtype { CYBQ_F32 = 0, CYBQ_F16 = 1, CYBQ_BF16 = 2 } cybq_dtype;
 
-/* How the prefill kernel (M > 32) feeds the matrix cores.  Both stay inside the
- * operator's 1e-3 relative-L2 tolerance.  (Calls of up to 32 rows, and 33 .. 64 rows on weights of up
- * to 6144 x 4096, take the decode kernels, whose operand form cybq_decode_mode describes; with
- * CYBQ_PREFILL_EXACT those 33 .. 64-row calls use the decode kernels' EXACT operands.)
+/* How the prefill kernels (M > 32; in FAST mode also 17 .. 32 rows of fp32 activations, or of 16-bit
+ * activations with a folded RMSNorm, on weights with K of 2048 .. 8192) feed the matrix cores.  Both stay
+ * inside the operator's 1e-3 relative-L2 tolerance.  (Calls of up to 16 rows, other calls of up to 32 rows,
+ * and 33 .. 64 rows on weights of up to 6144 x 4096 that the FAST kernels do not take - always so with
+ * CYBQ_PREFILL_EXACT, which gives them the decode kernels' EXACT operands - take the decode kernels, whose
+ * operand form cybq_decode_mode describes.)
  *   FAST   (default) one f16 MFMA per 32-group; the weight operand is
  *          round_f16(scale * q), relative error <= 2^-11 per weight (about 2e-4
  *          relative L2 on y).  bf16 and fp32 activations become f16 operands behind a
